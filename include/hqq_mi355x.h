@@ -1,0 +1,150 @@
+/*
+ * hqq_mi355x -- C ABI of the MI355X (gfx950) HQQ quantized-linear library.
+ *
+ * Every entry point takes plain device pointers, sizes and a hipStream_t passed
+ * as void*; nothing here depends on PyTorch.  All pointers are borrowed, the
+ * caller allocates every output and workspace, no entry point synchronises the
+ * stream or the device, and none of them calls hipMalloc / hipFree.
+ *
+ * Return value: 0 = success, negative = argument error (HQQ_E_*), positive =
+ * the hipError_t of the failed runtime call.  hqq_error_string() explains both.
+ *
+ * "Reference" citations are into dvmazur/mixtral-offloading (src/...): each
+ * entry point names the Python function of the reference that it replaces.
+ */
+#ifndef HQQ_MI355X_H
+#define HQQ_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HQQ_ABI_VERSION 1
+
+enum {
+    HQQ_OK = 0,
+    HQQ_E_NULL = -1,      /* a required pointer is NULL                       */
+    HQQ_E_NBITS = -2,     /* nbits not in {2,3,4}                             */
+    HQQ_E_SHAPE = -3,     /* sizes disagree (the reference's asserts)         */
+    HQQ_E_ALIGN = -4,     /* pointer or row pitch not aligned as documented   */
+    HQQ_E_WORKSPACE = -5, /* workspace too small (see hqq_workspace_bytes)    */
+    HQQ_E_UNSUPPORTED = -6,
+    HQQ_E_CACHE = -7      /* expert-cache policy error (see hqq_lru_*)        */
+};
+
+/* How a (G, K) scale or zero table is stored.
+ *   HQQ_TABLE_F16 : fp16 values, G*K of them                                  (meta['scale'] / meta['zero'])
+ *   HQQ_TABLE_U8  : uint8 values, G*K of them, with fp16 meta scale / zero of `meta_cols` entries; entry i of the table
+ *                   de-quantises as fp16(fp16(q[i] - mz[i % meta_cols]) * ms[i % meta_cols]).  meta_cols == 1 is the
+ *                   whole-tensor (scalar) case.                               (meta['scale_q'] + meta['meta_scale'])
+ * Reference: src/custom_layers.py:62-66 expands HQQ_TABLE_U8 to fp16 on every forward.                               */
+enum { HQQ_TABLE_F16 = 0, HQQ_TABLE_U8 = 1 };
+
+typedef struct hqq_table {
+    const void *data;      /* fp16[G*K] or uint8[G*K]                          */
+    const void *meta_scale; /* fp16[meta_cols] (HQQ_TABLE_U8 only)             */
+    const void *meta_zero;  /* fp16[meta_cols] (HQQ_TABLE_U8 only)             */
+    int64_t meta_cols;
+    int32_t kind;
+    int32_t reserved;
+} hqq_table;
+
+/* One HQQ-quantised linear layer in the kernel layout of the reference
+ * (src/custom_layers.py:41-47 `repack`, consumed at :68-86):
+ *   nbits 4: codes uint8 (N/2, K), byte = q[2p] << 4 | q[2p+1]                        (src/packing.py:10-17)
+ *   nbits 2: codes uint8 (N/4, K), byte = q[4p]<<6 | q[4p+1]<<4 | q[4p+2]<<2 | q[4p+3] (src/packing.py:36-41)
+ *   nbits 3: codes int32 (ceil(N/10), K), code i of a word at bit 3*(9-i)              (src/packing.py:62-81)
+ * Weight (n, k) uses table row n % G, G = N / group_size (src/triton_kernels.py:86-88).
+ * codes must be 16-byte aligned and K a multiple of 16 for the fast kernels; other shapes take a slower general kernel. */
+typedef struct hqq_linear {
+    int32_t nbits;
+    int32_t group_size;
+    int64_t N; /* out features */
+    int64_t K; /* in features  */
+    const void *codes;
+    hqq_table scale;
+    hqq_table zero;
+    const void *bias; /* fp16[N] or NULL */
+} hqq_linear;
+
+int hqq_abi_version(void);
+const char *hqq_error_string(int code);
+
+/* ---- bit packers: replace Quantizer.pack / Quantizer.unpack entries '4bit_u8', '2bit_u8', '3bit_32'
+ *      installed by src/packing.py:105-111 (functions at :10-27, :36-53, :62-97).
+ * `rows` is the height of the UNPACKED array for pack_* and of the PACKED array for unpack_*; `cols` is the product of
+ * the trailing dimensions.  Unpacked codes are uint8.  unpack_3bit always writes 10*rows rows (spare rows are zero).  */
+int hqq_pack_4bit_u8(const uint8_t *q, int64_t rows, int64_t cols, uint8_t *out, void *stream);
+int hqq_pack_2bit_u8(const uint8_t *q, int64_t rows, int64_t cols, uint8_t *out, void *stream);
+int hqq_pack_3bit_i32(const uint8_t *q, int64_t rows, int64_t cols, int32_t *out, void *stream);
+int hqq_unpack_4bit_u8(const uint8_t *in, int64_t rows, int64_t cols, uint8_t *q, void *stream);
+int hqq_unpack_2bit_u8(const uint8_t *in, int64_t rows, int64_t cols, uint8_t *q, void *stream);
+int hqq_unpack_3bit_i32(const int32_t *in, int64_t rows, int64_t cols, uint8_t *q, void *stream);
+
+/* ---- 8-bit table -> fp16 table: replaces Quantizer.dequantize(meta['scale_q'], meta['meta_scale']) and the same for
+ *      zero at src/custom_layers.py:63-66.  out is fp16[count].                                                      */
+int hqq_table_to_f16(const hqq_table *t, int64_t count, void *out_f16, void *stream);
+
+/* ---- full de-quantisation to fp16 (N, K): replaces HQQLinearTritonSavable.dequantize, src/custom_layers.py:95-116.
+ *      Bit-exact: W = fp16(fp16(q - z) * s).                                                                         */
+int hqq_dequantize(const hqq_linear *l, void *w_out_f16, void *stream);
+
+/* ---- y = x @ dequant(W).T (+ bias): replaces triton_matmul4_transpose / triton_matmul2_transpose /
+ *      triton_matmul3_transpose (src/triton_kernels.py:133-191, 321-380, 511-564) together with the meta expansion of
+ *      forward_triton (src/custom_layers.py:55-92).  x is fp16 (M, K) contiguous, y is fp16 (M, N).  fp32 accumulation.
+ *      `workspace` must hold hqq_matmul_workspace_bytes(l, M) bytes, 256-byte aligned; it holds split-K partial sums
+ *      and needs no initialisation.                                                                                   */
+size_t hqq_matmul_workspace_bytes(const hqq_linear *l, int64_t M);
+/* same, with the kernel family forced (-1 = automatic choice, else 0..3 as hqq_matmul_kernel_family reports):
+ * HQQ_E_UNSUPPORTED when that family does not take the configuration.  For tests and profiling.                    */
+int hqq_matmul_transpose_ex(const hqq_linear *l, const void *x_f16, int64_t M, void *y_f16, void *workspace,
+                            size_t workspace_bytes, int family, void *stream);
+int hqq_matmul_transpose(const hqq_linear *l, const void *x_f16, int64_t M, void *y_f16, void *workspace,
+                         size_t workspace_bytes, void *stream);
+
+/* ---- y = w2( silu(w1 x) * (w3 x) ): replaces MixtralBLockSparseTop2MLP_HQQ.forward, src/custom_layers.py:253-256.
+ *      x fp16 (M, hidden), y fp16 (M, hidden).  When `row_scale_f16` is not NULL, row m of the result is multiplied by
+ *      row_scale_f16[m] (the routing weight, src/custom_layers.py:308) and when `accumulate` is non-zero the result is
+ *      added to y in fp16 instead of stored (the index_add_ at :312 for a single row block).                          */
+size_t hqq_expert_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, int64_t M);
+int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *x_f16, int64_t M,
+                   void *y_f16, const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
+                   void *stream);
+
+/* ---- which kernel family a call would use (for tests and profiles): 0 general, 1 MFMA small-batch, 2 MFMA tile,
+ *      3 three-bit vector kernel.                                                                                     */
+int hqq_matmul_kernel_family(const hqq_linear *l, int64_t M);
+
+/* ---- expert offload: replaces the two copies of ExpertCache._swap (src/expert_cache.py:186-189).
+ *      Enqueues one asynchronous host-to-device copy of a whole expert slab from pinned host memory on `copy_stream`,
+ *      records `done_event` (a hipEvent_t) after it when not NULL.  The reference's device-to-host copy of the evicted
+ *      expert is not needed: weights are immutable and every expert keeps its pinned host copy.                       */
+int hqq_slab_h2d_async(void *dst_device, const void *src_pinned, size_t bytes, void *copy_stream, void *done_event);
+/* make `stream` wait for `event` without blocking the host */
+int hqq_stream_wait_event(void *stream, void *event);
+
+/* ---- LRU policy of one eviction group (host only, no GPU calls): replaces EvictionGroupInfo and the bookkeeping of
+ *      ExpertCache.load_experts / _swap (src/expert_cache.py:20-52, 120-201).  Experts are integers 0..n_experts-1;
+ *      `slots` device slots exist.                                                                                    */
+typedef struct hqq_lru hqq_lru;
+hqq_lru *hqq_lru_create(int32_t n_experts, int32_t slots);
+void hqq_lru_destroy(hqq_lru *c);
+/* place expert `e` into a free device slot at load time (src/expert_cache.py:102-110); returns the slot or HQQ_E_CACHE */
+int hqq_lru_add_resident(hqq_lru *c, int32_t e);
+/* Plan one load_experts(..., unordered=True) call for `n` distinct experts: marks every one used, then decides the
+ * evictions.  Outputs, each of length n, in the order the experts must be run (resident first, then misses in request
+ * order): order[i] = expert, slot[i] = device slot it will occupy, victim[i] = expert evicted to make room or -1 for a
+ * hit.  Returns 0 or HQQ_E_CACHE (unknown expert, duplicates, more misses than slots).                               */
+int hqq_lru_plan(hqq_lru *c, const int32_t *experts, int32_t n, int32_t *order, int32_t *slot, int32_t *victim);
+int64_t hqq_lru_hits(const hqq_lru *c);
+int64_t hqq_lru_misses(const hqq_lru *c);
+/* device slot of expert e, or -1 when it is not resident */
+int hqq_lru_slot_of(const hqq_lru *c, int32_t e);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HQQ_MI355X_H */

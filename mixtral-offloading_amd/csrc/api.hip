@@ -1,0 +1,229 @@
+// C ABI: argument checks (the reference's asserts become error codes),
+// kernel-family dispatch and workspace carving.
+#include "hqq_common.hpp"
+
+namespace hqq {
+
+static int validate_table(const hqq_table &t)
+{
+    if (!t.data)
+        return HQQ_E_NULL;
+    if (t.kind == HQQ_TABLE_F16)
+        return HQQ_OK;
+    if (t.kind != HQQ_TABLE_U8)
+        return HQQ_E_SHAPE;
+    if (!t.meta_scale || !t.meta_zero)
+        return HQQ_E_NULL;
+    if (t.meta_cols < 1)
+        return HQQ_E_SHAPE;
+    return HQQ_OK;
+}
+
+int validate_linear(const hqq_linear *l)
+{
+    if (!l || !l->codes)
+        return HQQ_E_NULL;
+    if (l->nbits != 2 && l->nbits != 3 && l->nbits != 4) // reference src/custom_layers.py:24
+        return HQQ_E_NBITS;
+    if (l->N <= 0 || l->K <= 0 || l->group_size <= 0)
+        return HQQ_E_SHAPE;
+    if (l->N % l->group_size != 0) // table row n % G needs G = N / group_size to be whole
+        return HQQ_E_SHAPE;
+    if ((l->nbits == 4 && l->N % 2) || (l->nbits == 2 && l->N % 4))
+        return HQQ_E_SHAPE;
+    int rc = validate_table(l->scale);
+    if (rc != HQQ_OK)
+        return rc;
+    return validate_table(l->zero);
+}
+
+static inline size_t align256(size_t v) { return (v + 255u) & ~(size_t)255u; }
+
+enum { FAM_GENERAL = 0, FAM_SMALLBATCH = 1, FAM_TILE = 2, FAM_VEC3 = 3 };
+
+static int pick_family(const hqq_linear *l, int64_t M)
+{
+    if (smallbatch_supported(l, M))
+        return FAM_SMALLBATCH;
+    if (vec3_supported(l, M))
+        return FAM_VEC3;
+    if (tile_supported(l, M))
+        return FAM_TILE;
+    return FAM_GENERAL;
+}
+
+static size_t family_workspace(const hqq_linear *l, int64_t M, int fam)
+{
+    if (fam == FAM_SMALLBATCH)
+        return smallbatch_workspace_bytes(l, M);
+    if (fam == FAM_VEC3)
+        return vec3_workspace_bytes(l, M);
+    return 0;
+}
+
+static int run_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, int fam,
+                      hipStream_t s)
+{
+    if (M == 0)
+        return HQQ_OK;
+    switch (fam) {
+    case FAM_SMALLBATCH:
+        return launch_smallbatch_matmul(l, x, M, y, ws, ws_bytes, SmallBatchEpilogue{}, s);
+    case FAM_VEC3:
+        return launch_vec3_matmul(l, x, M, y, ws, ws_bytes, s);
+    case FAM_TILE:
+        return launch_tile_matmul(l, x, M, y, s);
+    default:
+        return launch_general_matmul(l, x, M, y, s);
+    }
+}
+
+} // namespace hqq
+
+using namespace hqq;
+
+extern "C" {
+
+int hqq_abi_version(void) { return HQQ_ABI_VERSION; }
+
+const char *hqq_error_string(int code)
+{
+    switch (code) {
+    case HQQ_OK: return "ok";
+    case HQQ_E_NULL: return "a required pointer is NULL";
+    case HQQ_E_NBITS: return "nbits must be 2, 3 or 4";
+    case HQQ_E_SHAPE: return "sizes disagree";
+    case HQQ_E_ALIGN: return "pointer or pitch is not aligned as documented";
+    case HQQ_E_WORKSPACE: return "workspace is too small or misaligned";
+    case HQQ_E_UNSUPPORTED: return "configuration not supported by the requested kernel family";
+    case HQQ_E_CACHE: return "expert cache policy error";
+    default: break;
+    }
+    if (code > 0)
+        return hipGetErrorString(static_cast<hipError_t>(code));
+    return "unknown error";
+}
+
+int hqq_matmul_kernel_family(const hqq_linear *l, int64_t M)
+{
+    int rc = validate_linear(l);
+    if (rc != HQQ_OK)
+        return rc;
+    return pick_family(l, M);
+}
+
+size_t hqq_matmul_workspace_bytes(const hqq_linear *l, int64_t M)
+{
+    if (validate_linear(l) != HQQ_OK || M <= 0)
+        return 0;
+    // large enough for whichever family is chosen or forced
+    size_t a = smallbatch_supported(l, M) ? smallbatch_workspace_bytes(l, M) : 0;
+    size_t b = vec3_supported(l, M) ? vec3_workspace_bytes(l, M) : 0;
+    return align256(a > b ? a : b);
+}
+
+int hqq_matmul_transpose_ex(const hqq_linear *l, const void *x_f16, int64_t M, void *y_f16, void *workspace,
+                            size_t workspace_bytes, int family, void *stream)
+{
+    int rc = validate_linear(l);
+    if (rc != HQQ_OK)
+        return rc;
+    if (M < 0)
+        return HQQ_E_SHAPE;
+    if (M == 0)
+        return HQQ_OK;
+    if (!x_f16 || !y_f16)
+        return HQQ_E_NULL;
+    int fam = family < 0 ? pick_family(l, M) : family;
+    if (fam == FAM_SMALLBATCH && !smallbatch_supported(l, M))
+        return HQQ_E_UNSUPPORTED;
+    if (fam == FAM_VEC3 && !vec3_supported(l, M))
+        return HQQ_E_UNSUPPORTED;
+    if (fam == FAM_TILE && !tile_supported(l, M))
+        return HQQ_E_UNSUPPORTED;
+    if (fam < 0 || fam > FAM_VEC3)
+        return HQQ_E_UNSUPPORTED;
+    const size_t need = family_workspace(l, M, fam);
+    if (need > 0 && (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)))
+        return HQQ_E_WORKSPACE;
+    return run_matmul(l, (const f16 *)x_f16, M, (f16 *)y_f16, workspace, workspace_bytes, fam, (hipStream_t)stream);
+}
+
+int hqq_matmul_transpose(const hqq_linear *l, const void *x_f16, int64_t M, void *y_f16, void *workspace,
+                         size_t workspace_bytes, void *stream)
+{
+    return hqq_matmul_transpose_ex(l, x_f16, M, y_f16, workspace, workspace_bytes, -1, stream);
+}
+
+// workspace of the FFN: [h: M x ffn fp16][t: M x hidden fp16][a, b: M x ffn fp16 each (unfused path)][matmul scratch]
+size_t hqq_expert_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, int64_t M)
+{
+    if (validate_linear(w1) != HQQ_OK || validate_linear(w2) != HQQ_OK || validate_linear(w3) != HQQ_OK || M <= 0)
+        return 0;
+    size_t mm = hqq_matmul_workspace_bytes(w1, M);
+    size_t m2 = hqq_matmul_workspace_bytes(w2, M);
+    size_t m3 = 2 * hqq_matmul_workspace_bytes(w3, M); // fused gate/up pass keeps two sets of partial sums
+    if (m2 > mm)
+        mm = m2;
+    if (m3 > mm)
+        mm = m3;
+    return 3 * align256((size_t)M * w1->N * 2) + align256((size_t)M * w2->N * 2) + mm;
+}
+
+int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *x_f16, int64_t M,
+                   void *y_f16, const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
+                   void *stream)
+{
+    int rc;
+    if ((rc = validate_linear(w1)) != HQQ_OK || (rc = validate_linear(w2)) != HQQ_OK ||
+        (rc = validate_linear(w3)) != HQQ_OK)
+        return rc;
+    if (M < 0 || w1->N != w3->N || w1->K != w3->K || w2->K != w1->N || w2->N != w1->K)
+        return HQQ_E_SHAPE;
+    if (M == 0)
+        return HQQ_OK;
+    if (!x_f16 || !y_f16)
+        return HQQ_E_NULL;
+    const size_t need = hqq_expert_ffn_workspace_bytes(w1, w2, w3, M);
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return HQQ_E_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    char *p = static_cast<char *>(workspace);
+    const size_t mid = align256((size_t)M * w1->N * 2), outb = align256((size_t)M * w2->N * 2);
+    f16 *h = (f16 *)p;
+    f16 *t = (f16 *)(p + mid);
+    f16 *a = (f16 *)(p + mid + outb);
+    f16 *b = (f16 *)(p + 2 * mid + outb);
+    void *mm = p + 3 * mid + outb;
+    const size_t mm_bytes = workspace_bytes - (3 * mid + outb);
+    const f16 *x = (const f16 *)x_f16;
+    f16 *y = (f16 *)y_f16;
+
+    const bool fast13 = smallbatch_supported(w1, M) && smallbatch_supported(w3, M) && !w1->bias && !w3->bias &&
+                        w1->nbits == w3->nbits && w1->group_size == w3->group_size;
+    if (fast13) {
+        rc = launch_smallbatch_gate_up(w1, w3, x, M, h, mm, mm_bytes, s);
+        if (rc != HQQ_OK)
+            return rc;
+    } else {
+        if ((rc = run_matmul(w1, x, M, a, mm, mm_bytes, pick_family(w1, M), s)) != HQQ_OK)
+            return rc;
+        if ((rc = run_matmul(w3, x, M, b, mm, mm_bytes, pick_family(w3, M), s)) != HQQ_OK)
+            return rc;
+        if ((rc = launch_silu_mul(a, b, h, M * w1->N, s)) != HQQ_OK)
+            return rc;
+    }
+    if (smallbatch_supported(w2, M)) {
+        SmallBatchEpilogue ep;
+        ep.row_scale = (const f16 *)row_scale_f16;
+        ep.accumulate = accumulate;
+        return launch_smallbatch_matmul(w2, h, M, y, mm, mm_bytes, ep, s);
+    }
+    if (!row_scale_f16 && !accumulate)
+        return run_matmul(w2, h, M, y, mm, mm_bytes, pick_family(w2, M), s);
+    if ((rc = run_matmul(w2, h, M, t, mm, mm_bytes, pick_family(w2, M), s)) != HQQ_OK)
+        return rc;
+    return launch_scale_store(t, y, (const f16 *)row_scale_f16, accumulate, M, w2->N, s);
+}
+
+} // extern "C"

@@ -1,0 +1,110 @@
+// Shared declarations of the gfx950 HQQ library: the C ABI, vector types and
+// the table accessors every kernel uses.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "hqq_mi355x.h"
+
+namespace hqq {
+
+typedef _Float16 f16;
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+
+// Device-side copy of hqq_table with typed pointers.
+struct Table {
+    const void *data;
+    const f16 *ms;
+    const f16 *mz;
+    int64_t meta_cols;
+    int kind;
+};
+
+inline Table make_table(const hqq_table &t)
+{
+    Table r;
+    r.data = t.data;
+    r.ms = static_cast<const f16 *>(t.meta_scale);
+    r.mz = static_cast<const f16 *>(t.meta_zero);
+    r.meta_cols = t.meta_cols;
+    r.kind = t.kind;
+    return r;
+}
+
+// fp16 value of table entry c: either stored, or fp16(fp16(q - mz) * ms) with
+// two roundings exactly as the reference's meta de-quantisation
+// (reference src/custom_layers.py:63-66, formula restated at :111).
+__device__ __forceinline__ f16 table_at(const Table &t, int64_t c)
+{
+    if (t.kind == HQQ_TABLE_F16)
+        return static_cast<const f16 *>(t.data)[c];
+    const int64_t mc = (t.meta_cols == 1) ? 0 : (c % t.meta_cols);
+    const f16 q = (f16)(float)static_cast<const uint8_t *>(t.data)[c];
+    const f16 d = q - t.mz[mc];
+    return d * t.ms[mc];
+}
+
+// Code of weight (n, k) in the kernel layout
+// (reference src/triton_kernels.py:84,91 / :272,279 / :462,469).
+template <int NBITS>
+__device__ __forceinline__ uint32_t code_at(const void *codes, int64_t n, int64_t k, int64_t K)
+{
+    if constexpr (NBITS == 4)
+        return (static_cast<const uint8_t *>(codes)[(n >> 1) * K + k] >> (((n + 1) & 1) * 4)) & 0xFu;
+    else if constexpr (NBITS == 2)
+        return (static_cast<const uint8_t *>(codes)[(n >> 2) * K + k] >> ((3 - (n & 3)) * 2)) & 0x3u;
+    else
+        return (static_cast<const uint32_t *>(codes)[(n / 10) * K + k] >> ((9 - n % 10) * 3)) & 0x7u;
+}
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1)
+        v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// launch-status helper: kernels are launched with <<<>>> and checked once
+inline int launch_status()
+{
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? HQQ_OK : static_cast<int>(e);
+}
+
+// implemented in the individual translation units
+int validate_linear(const hqq_linear *l);
+int launch_general_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, hipStream_t s);
+bool smallbatch_supported(const hqq_linear *l, int64_t M);
+size_t smallbatch_workspace_bytes(const hqq_linear *l, int64_t M);
+// epilogue selector of the small-batch kernel
+struct SmallBatchEpilogue {
+    const f16 *row_scale = nullptr; // optional per-row multiplier (routing weight)
+    int accumulate = 0;             // add into y instead of storing
+};
+int launch_smallbatch_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
+                             const SmallBatchEpilogue &ep, hipStream_t s);
+// fused w1/w3 pass: h = silu(x w1^T) * (x w3^T), fp16 (M, N)
+int launch_smallbatch_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
+                              size_t ws_bytes, hipStream_t s);
+bool tile_supported(const hqq_linear *l, int64_t M);
+int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, hipStream_t s);
+bool vec3_supported(const hqq_linear *l, int64_t M);
+size_t vec3_workspace_bytes(const hqq_linear *l, int64_t M);
+int launch_vec3_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s);
+int launch_silu_mul(const f16 *a, const f16 *b, f16 *h, int64_t count, hipStream_t s);
+int launch_scale_store(const f16 *src, f16 *dst, const f16 *row_scale, int accumulate, int64_t M, int64_t N,
+                       hipStream_t s);
+
+} // namespace hqq

@@ -1,0 +1,362 @@
+// Bit packers, 8-bit table expansion and the bit-exact de-quantiser.
+//
+// These are streaming byte kernels, bounded by HBM: every thread moves whole
+// 32-bit or 128-bit words and does its bit work on four codes per lane-op.
+// Layouts follow the reference packers (src/packing.py:10-97).
+#include "hqq_common.hpp"
+
+namespace hqq {
+namespace {
+
+constexpr int kThreads = 256;
+
+// the same byte mask in every byte of a word, for scalar bytes and 128-bit words
+template <typename WordT> __device__ __forceinline__ WordT byte_mask(uint32_t b)
+{
+    if constexpr (sizeof(WordT) == 1) {
+        return (WordT)b;
+    } else {
+        const uint32_t m = b * 0x01010101u;
+        WordT r = {m, m, m, m};
+        return r;
+    }
+}
+
+// ---------------------------------------------------------------- 4 / 2 bit
+// One thread handles VEC consecutive columns of one packed row.
+template <int NBITS, typename WordT>
+__global__ __launch_bounds__(kThreads) void unpack_u8_kernel(const uint8_t *__restrict__ in, int64_t prows,
+                                                             int64_t cols, uint8_t *__restrict__ out)
+{
+    constexpr int F = 8 / NBITS;
+    constexpr int VEC = sizeof(WordT);
+    const int64_t chunks = cols / VEC;
+    const int64_t total = prows * chunks;
+    for (int64_t idx = blockIdx.x * (int64_t)kThreads + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * kThreads) {
+        const int64_t p = idx / chunks, c = (idx - p * chunks) * VEC;
+        const WordT w = *reinterpret_cast<const WordT *>(in + p * cols + c);
+#pragma unroll
+        for (int i = 0; i < F; ++i) {
+            WordT v;
+            if constexpr (NBITS == 4)
+                v = (WordT)(w >> (4 * (1 - i))) & byte_mask<WordT>(0x0Fu);
+            else
+                v = (WordT)(w >> (2 * (3 - i))) & byte_mask<WordT>(0x03u);
+            *reinterpret_cast<WordT *>(out + (F * p + i) * cols + c) = v;
+        }
+    }
+}
+
+template <int NBITS, typename WordT>
+__global__ __launch_bounds__(kThreads) void pack_u8_kernel(const uint8_t *__restrict__ q, int64_t prows, int64_t cols,
+                                                           uint8_t *__restrict__ out)
+{
+    constexpr int F = 8 / NBITS;
+    constexpr int VEC = sizeof(WordT);
+    const int64_t chunks = cols / VEC;
+    const int64_t total = prows * chunks;
+    for (int64_t idx = blockIdx.x * (int64_t)kThreads + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * kThreads) {
+        const int64_t p = idx / chunks, c = (idx - p * chunks) * VEC;
+        WordT acc = byte_mask<WordT>(0);
+#pragma unroll
+        for (int i = 0; i < F; ++i) {
+            const WordT v = *reinterpret_cast<const WordT *>(q + (F * p + i) * cols + c);
+            // uint8 shift as in the reference: bits pushed past bit 7 are lost, the last row is OR-ed unmasked
+            const int sh = NBITS * (F - 1 - i);
+            acc |= (WordT)(v << sh) & byte_mask<WordT>((0xFFu << sh) & 0xFFu);
+        }
+        *reinterpret_cast<WordT *>(out + p * cols + c) = acc;
+    }
+}
+
+// ------------------------------------------------------------------- 3 bit
+// One thread handles VEC consecutive columns of one word row: VEC words in,
+// VEC bytes to each of ten unpacked rows (or the reverse).
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void unpack3_kernel(const uint32_t *__restrict__ in, int64_t words,
+                                                           int64_t cols, uint8_t *__restrict__ out)
+{
+    const int64_t chunks = cols / VEC;
+    const int64_t total = words * chunks;
+    for (int64_t idx = blockIdx.x * (int64_t)kThreads + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * kThreads) {
+        const int64_t p = idx / chunks, c = (idx - p * chunks) * VEC;
+        uint32_t w[VEC];
+        if constexpr (VEC == 4) {
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(in + p * cols + c);
+            w[0] = v.x, w[1] = v.y, w[2] = v.z, w[3] = v.w;
+        } else {
+            w[0] = in[p * cols + c];
+        }
+#pragma unroll
+        for (int i = 0; i < 10; ++i) {
+            const int sh = 3 * (9 - i);
+            uint8_t *dst = out + (10 * p + i) * cols + c;
+            if constexpr (VEC == 4) {
+                const uint32_t b = ((w[0] >> sh) & 7u) | (((w[1] >> sh) & 7u) << 8) | (((w[2] >> sh) & 7u) << 16) |
+                                   (((w[3] >> sh) & 7u) << 24);
+                *reinterpret_cast<uint32_t *>(dst) = b;
+            } else {
+                *dst = (uint8_t)((w[0] >> sh) & 7u);
+            }
+        }
+    }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void pack3_kernel(const uint8_t *__restrict__ q, int64_t rows, int64_t cols,
+                                                         uint32_t *__restrict__ out)
+{
+    const int64_t words = (rows + 9) / 10;
+    const int64_t chunks = cols / VEC;
+    const int64_t total = words * chunks;
+    for (int64_t idx = blockIdx.x * (int64_t)kThreads + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * kThreads) {
+        const int64_t p = idx / chunks, c = (idx - p * chunks) * VEC;
+        uint32_t w[VEC] = {};
+#pragma unroll
+        for (int i = 0; i < 10; ++i) {
+            const int64_t r = 10 * p + i;
+            if (r < rows) { // lanes past the last row stay zero
+                const int sh = 3 * (9 - i);
+                if constexpr (VEC == 4) {
+                    const uint32_t b = *reinterpret_cast<const uint32_t *>(q + r * cols + c);
+                    // codes are widened to 32 bits and shifted unmasked, as the reference does
+                    w[0] |= (b & 0xFFu) << sh;
+                    w[1] |= ((b >> 8) & 0xFFu) << sh;
+                    w[2] |= ((b >> 16) & 0xFFu) << sh;
+                    w[3] |= (b >> 24) << sh;
+                } else {
+                    w[0] |= (uint32_t)q[r * cols + c] << sh;
+                }
+            }
+        }
+        if constexpr (VEC == 4) {
+            u32x4 v;
+            v.x = w[0], v.y = w[1], v.z = w[2], v.w = w[3];
+            *reinterpret_cast<u32x4 *>(out + p * cols + c) = v;
+        } else {
+            out[p * cols + c] = w[0];
+        }
+    }
+}
+
+// ------------------------------------------------------- table -> fp16
+__global__ __launch_bounds__(kThreads) void table_to_f16_kernel(Table t, int64_t count, f16 *__restrict__ out)
+{
+    for (int64_t i = blockIdx.x * (int64_t)kThreads + threadIdx.x; i < count; i += (int64_t)gridDim.x * kThreads)
+        out[i] = table_at(t, i);
+}
+
+// ------------------------------------------------------- de-quantise
+// W[n,k] = fp16(fp16(q - Z[n%G,k]) * S[n%G,k]); one thread per (word, 4 columns).
+template <int NBITS>
+__global__ __launch_bounds__(kThreads) void dequantize_kernel(const void *__restrict__ codes, Table sc, Table zr,
+                                                              int64_t N, int64_t K, int64_t G, f16 *__restrict__ w)
+{
+    constexpr int F = NBITS == 3 ? 10 : 8 / NBITS;
+    const int64_t prows = (N + F - 1) / F;
+    const int64_t kchunks = (K + 3) / 4;
+    const int64_t total = prows * kchunks;
+    for (int64_t idx = blockIdx.x * (int64_t)kThreads + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * kThreads) {
+        const int64_t p = idx / kchunks, k0 = (idx - p * kchunks) * 4;
+#pragma unroll
+        for (int i = 0; i < F; ++i) {
+            const int64_t n = F * p + i;
+            if (n >= N)
+                break;
+            const int64_t j = n % G;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int64_t k = k0 + e;
+                if (k < K) {
+                    const f16 q = (f16)(float)code_at<NBITS>(codes, n, k, K);
+                    const f16 d = q - table_at(zr, j * K + k); // first rounding
+                    w[n * K + k] = d * table_at(sc, j * K + k); // second rounding
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------- small elementwise
+__global__ __launch_bounds__(kThreads) void silu_mul_kernel(const f16 *__restrict__ a, const f16 *__restrict__ b,
+                                                            f16 *__restrict__ h, int64_t count)
+{
+    for (int64_t i = blockIdx.x * (int64_t)kThreads + threadIdx.x; i < count; i += (int64_t)gridDim.x * kThreads) {
+        const float x = (float)a[i];
+        const f16 act = (f16)(x / (1.0f + __expf(-x))); // silu in fp32, one rounding
+        h[i] = act * b[i];
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void scale_store_kernel(const f16 *__restrict__ src, f16 *__restrict__ dst,
+                                                               const f16 *__restrict__ row_scale, int accumulate,
+                                                               int64_t M, int64_t N)
+{
+    for (int64_t i = blockIdx.x * (int64_t)kThreads + threadIdx.x; i < M * N; i += (int64_t)gridDim.x * kThreads) {
+        f16 v = src[i];
+        if (row_scale)
+            v = v * row_scale[i / N];
+        dst[i] = accumulate ? (f16)(dst[i] + v) : v;
+    }
+}
+
+inline int grid_for(int64_t total)
+{
+    int64_t b = (total + kThreads - 1) / kThreads;
+    if (b < 1)
+        b = 1;
+    if (b > 256 * 32)
+        b = 256 * 32;
+    return (int)b;
+}
+
+template <int NBITS>
+int unpack_u8(const uint8_t *in, int64_t prows, int64_t cols, uint8_t *out, hipStream_t s)
+{
+    if (!in || !out)
+        return HQQ_E_NULL;
+    if (prows < 0 || cols < 0)
+        return HQQ_E_SHAPE;
+    if (prows == 0 || cols == 0)
+        return HQQ_OK;
+    if (cols % 16 == 0 && aligned16(in) && aligned16(out))
+        unpack_u8_kernel<NBITS, u32x4><<<grid_for(prows * cols / 16), kThreads, 0, s>>>(in, prows, cols, out);
+    else
+        unpack_u8_kernel<NBITS, uint8_t><<<grid_for(prows * cols), kThreads, 0, s>>>(in, prows, cols, out);
+    return launch_status();
+}
+
+template <int NBITS>
+int pack_u8(const uint8_t *q, int64_t rows, int64_t cols, uint8_t *out, hipStream_t s)
+{
+    constexpr int F = 8 / NBITS;
+    if (!q || !out)
+        return HQQ_E_NULL;
+    if (rows < 0 || cols < 0 || rows % F != 0) // reference asserts an even height for 4 bit (src/packing.py:12)
+        return HQQ_E_SHAPE;
+    if (rows == 0 || cols == 0)
+        return HQQ_OK;
+    const int64_t prows = rows / F;
+    if (cols % 16 == 0 && aligned16(q) && aligned16(out))
+        pack_u8_kernel<NBITS, u32x4><<<grid_for(prows * cols / 16), kThreads, 0, s>>>(q, prows, cols, out);
+    else
+        pack_u8_kernel<NBITS, uint8_t><<<grid_for(prows * cols), kThreads, 0, s>>>(q, prows, cols, out);
+    return launch_status();
+}
+
+} // namespace
+
+int launch_silu_mul(const f16 *a, const f16 *b, f16 *h, int64_t count, hipStream_t s)
+{
+    if (count <= 0)
+        return HQQ_OK;
+    silu_mul_kernel<<<grid_for(count), kThreads, 0, s>>>(a, b, h, count);
+    return launch_status();
+}
+
+int launch_scale_store(const f16 *src, f16 *dst, const f16 *row_scale, int accumulate, int64_t M, int64_t N,
+                       hipStream_t s)
+{
+    if (M * N <= 0)
+        return HQQ_OK;
+    scale_store_kernel<<<grid_for(M * N), kThreads, 0, s>>>(src, dst, row_scale, accumulate, M, N);
+    return launch_status();
+}
+
+} // namespace hqq
+
+using namespace hqq;
+
+extern "C" {
+
+int hqq_pack_4bit_u8(const uint8_t *q, int64_t rows, int64_t cols, uint8_t *out, void *stream)
+{
+    return pack_u8<4>(q, rows, cols, out, (hipStream_t)stream);
+}
+int hqq_pack_2bit_u8(const uint8_t *q, int64_t rows, int64_t cols, uint8_t *out, void *stream)
+{
+    return pack_u8<2>(q, rows, cols, out, (hipStream_t)stream);
+}
+int hqq_unpack_4bit_u8(const uint8_t *in, int64_t rows, int64_t cols, uint8_t *q, void *stream)
+{
+    return unpack_u8<4>(in, rows, cols, q, (hipStream_t)stream);
+}
+int hqq_unpack_2bit_u8(const uint8_t *in, int64_t rows, int64_t cols, uint8_t *q, void *stream)
+{
+    return unpack_u8<2>(in, rows, cols, q, (hipStream_t)stream);
+}
+
+int hqq_pack_3bit_i32(const uint8_t *q, int64_t rows, int64_t cols, int32_t *out, void *stream)
+{
+    if (!q || !out)
+        return HQQ_E_NULL;
+    if (rows < 0 || cols < 0)
+        return HQQ_E_SHAPE;
+    if (rows == 0 || cols == 0)
+        return HQQ_OK;
+    const int64_t words = (rows + 9) / 10;
+    hipStream_t s = (hipStream_t)stream;
+    if (cols % 4 == 0 && aligned16(out) && (reinterpret_cast<uintptr_t>(q) & 3u) == 0)
+        pack3_kernel<4><<<grid_for(words * cols / 4), kThreads, 0, s>>>(q, rows, cols, (uint32_t *)out);
+    else
+        pack3_kernel<1><<<grid_for(words * cols), kThreads, 0, s>>>(q, rows, cols, (uint32_t *)out);
+    return launch_status();
+}
+
+int hqq_unpack_3bit_i32(const int32_t *in, int64_t rows, int64_t cols, uint8_t *q, void *stream)
+{
+    if (!in || !q)
+        return HQQ_E_NULL;
+    if (rows < 0 || cols < 0)
+        return HQQ_E_SHAPE;
+    if (rows == 0 || cols == 0)
+        return HQQ_OK;
+    hipStream_t s = (hipStream_t)stream;
+    if (cols % 4 == 0 && aligned16(in) && (reinterpret_cast<uintptr_t>(q) & 3u) == 0)
+        unpack3_kernel<4><<<grid_for(rows * cols / 4), kThreads, 0, s>>>((const uint32_t *)in, rows, cols, q);
+    else
+        unpack3_kernel<1><<<grid_for(rows * cols), kThreads, 0, s>>>((const uint32_t *)in, rows, cols, q);
+    return launch_status();
+}
+
+int hqq_table_to_f16(const hqq_table *t, int64_t count, void *out_f16, void *stream)
+{
+    if (!t || !t->data || !out_f16)
+        return HQQ_E_NULL;
+    if (t->kind == HQQ_TABLE_U8 && (!t->meta_scale || !t->meta_zero))
+        return HQQ_E_NULL;
+    if (count < 0 || (t->kind == HQQ_TABLE_U8 && t->meta_cols < 1) || (t->kind != HQQ_TABLE_U8 && t->kind != HQQ_TABLE_F16))
+        return HQQ_E_SHAPE;
+    if (count == 0)
+        return HQQ_OK;
+    table_to_f16_kernel<<<grid_for(count), kThreads, 0, (hipStream_t)stream>>>(make_table(*t), count, (f16 *)out_f16);
+    return launch_status();
+}
+
+int hqq_dequantize(const hqq_linear *l, void *w_out_f16, void *stream)
+{
+    int rc = validate_linear(l);
+    if (rc != HQQ_OK)
+        return rc;
+    if (!w_out_f16)
+        return HQQ_E_NULL;
+    const int64_t G = l->N / l->group_size;
+    const int F = l->nbits == 3 ? 10 : 8 / l->nbits;
+    const int64_t total = ((l->N + F - 1) / F) * ((l->K + 3) / 4);
+    hipStream_t s = (hipStream_t)stream;
+    const Table sc = make_table(l->scale), zr = make_table(l->zero);
+    if (l->nbits == 4)
+        dequantize_kernel<4><<<grid_for(total), kThreads, 0, s>>>(l->codes, sc, zr, l->N, l->K, G, (f16 *)w_out_f16);
+    else if (l->nbits == 2)
+        dequantize_kernel<2><<<grid_for(total), kThreads, 0, s>>>(l->codes, sc, zr, l->N, l->K, G, (f16 *)w_out_f16);
+    else
+        dequantize_kernel<3><<<grid_for(total), kThreads, 0, s>>>(l->codes, sc, zr, l->N, l->K, G, (f16 *)w_out_f16);
+    return launch_status();
+}
+
+} // extern "C"

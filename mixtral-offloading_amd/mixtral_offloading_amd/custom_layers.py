@@ -1,0 +1,216 @@
+"""Quantised linear, expert FFN and sparse-MoE block with the reference's
+module surface (reference ``src/custom_layers.py``), computing on the HIP
+library.
+
+``HQQLinearTritonSavable`` keeps its reference name although nothing here is
+Triton: the name is the drop-in contract.  Differences that do not change
+results: the 8-bit scale / zero tables are de-quantised inside the matmul
+kernel rather than expanded to fp16 per call (reference :62-66), the code
+layout is tracked by an explicit flag next to the ``PackedTensor`` tag
+(reference src/packing.py:29-33 relies on the tag alone), and the non-tensor
+meta is computed in closed form (reference :118-134 quantises a dummy layer)."""
+from __future__ import annotations
+
+import copy
+from typing import Any, Dict
+
+import torch
+from torch import nn
+from torch.nn import functional as F
+
+from . import hip_kernels
+from .hqq_core import HQQLinear, Quantizer, closed_form_meta
+from .packing import PackedTensor
+
+_META_TENSOR_KEYS = {"scale_q", "meta_scale.scale", "meta_scale.zero", "zero_q", "meta_zero.scale",
+                     "meta_zero.zero", "scale", "zero"}
+
+
+def _codes_shape(meta) -> tuple:
+    n, k = int(meta["shape"][0]), int(meta["shape"][1])
+    nbits = meta["nbits"]
+    if nbits == 3:
+        return ((n + 9) // 10, k)
+    return (n * nbits // 8, k)
+
+
+class HQQLinearTritonSavable(HQQLinear):
+    def __init__(self, layer, quant_config, meta=None, **kwargs):
+        """``meta`` for an empty layer comes from ``get_hqq_meta((in, out), quant_config)``."""
+        assert quant_config["weight_quant_params"]["nbits"] in [2, 3, 4]
+        super().__init__(layer, quant_config, **kwargs)
+        self._desc_cache = None
+        if not hasattr(self, "meta"):
+            assert meta is not None
+            self.meta = copy.deepcopy(meta)
+        self._register_state_dict_hook(self._add_to_state_dict_hook)
+        self._register_load_state_dict_pre_hook(self._load_from_state_dict_hook)
+
+    # ---------------------------------------------------------------- layout
+    def quantize(self, *args, **kwargs):
+        super().quantize(*args, **kwargs)
+        self.repack()
+
+    def in_kernel_layout(self) -> bool:
+        return self.W_q is not None and tuple(self.W_q.shape) == _codes_shape(self.meta)
+
+    def repack(self):
+        """Quantise-time layout (gs/f, N*K/gs) -> kernel layout (N/f, K)
+        (reference src/custom_layers.py:41-47)."""
+        if not self.in_kernel_layout():
+            sh = tuple(int(v) for v in self.meta["shape"])
+            codes = Quantizer.unpack[self.meta["packing"]](self.W_q)
+            codes = codes.reshape((-1,) + sh[1:])[: sh[0], ...]
+            self.W_q = Quantizer.pack[self.meta["packing"]](codes.contiguous())
+        elif not isinstance(self.W_q, PackedTensor):
+            self.W_q = PackedTensor(self.W_q)
+        self._desc_cache = None
+
+    # --------------------------------------------------------------- compute
+    def _desc(self) -> hip_kernels.LinearDesc:
+        meta = self.meta
+        ptrs = (self.W_q.data_ptr(),
+                meta["scale_q"].data_ptr() if meta.get("quant_scale") else meta["scale"].data_ptr(),
+                meta["zero_q"].data_ptr() if meta.get("quant_zero") else meta["zero"].data_ptr(),
+                self.bias.data_ptr() if getattr(self, "bias", None) is not None else 0)
+        if self._desc_cache is None or self._desc_cache[0] != ptrs:
+            assert self.in_kernel_layout(), "codes are not in the kernel layout; call repack()"
+            self._desc_cache = (ptrs, hip_kernels.LinearDesc(self.W_q, meta, getattr(self, "bias", None)))
+        return self._desc_cache[1]
+
+    def forward(self, x):
+        return self.forward_triton(x)
+
+    def set_backend(self, backend):
+        pass
+
+    @torch.inference_mode()
+    def forward_triton(self, x):
+        """y = x @ dequant(W).T (+ bias) (reference src/custom_layers.py:55-92)."""
+        assert self.ready, "model was not quantized"
+        assert self.meta["axis"] == 0
+        if self.meta["nbits"] not in (2, 3, 4):
+            raise RuntimeError(f"nbits == {self.meta['nbits']} isn't yet supported")
+        if x.dtype != torch.float16:
+            x = x.to(torch.float16)
+        return hip_kernels.matmul(self._desc(), x.contiguous())
+
+    forward_hip = forward_triton
+
+    @torch.inference_mode()
+    def dequantize(self):
+        """fp16 (N, K) weights, bit-exact ``(q - z) * s`` (reference src/custom_layers.py:95-116)."""
+        assert self.ready, "model was not quantized"
+        return hip_kernels.dequantize(self._desc()).reshape(tuple(self.meta["shape"]))
+
+    @classmethod
+    def get_hqq_meta(cls, linear_shape, quant_config):
+        return closed_form_meta(linear_shape, quant_config)
+
+    # ------------------------------------------------------------ state dict
+    @staticmethod
+    def _add_to_state_dict_hook(self, state_dict, prefix, local_metadata):
+        """Flat key schema of the reference (src/custom_layers.py:136-166)."""
+        assert set(self._get_tensor_paths(self.meta)).issubset(_META_TENSOR_KEYS)
+        out = {"W_q": torch.Tensor.as_subclass(self.W_q, torch.Tensor)}
+        if self.bias is not None:
+            out["bias"] = self.bias
+        meta = self.meta
+        if "meta_scale" in meta and "scale_q" in meta:
+            out["meta.scale_q"] = meta["scale_q"]
+            out["meta.meta_scale.scale"] = meta["meta_scale"]["scale"]
+            out["meta.meta_scale.zero"] = meta["meta_scale"]["zero"]
+        else:
+            out["meta.scale"] = meta["scale"]
+        if "meta_zero" in meta and "zero_q" in meta:
+            out["meta.zero_q"] = meta["zero_q"]
+            out["meta.meta_zero.scale"] = meta["meta_zero"]["scale"]
+            out["meta.meta_zero.zero"] = meta["meta_zero"]["zero"]
+        else:
+            out["meta.zero"] = meta["zero"]
+        for name, value in out.items():
+            state_dict[prefix + name] = value
+        return state_dict
+
+    def _load_from_state_dict_hook(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                                   error_msgs):
+        """Inverse of the hook above (reference src/custom_layers.py:168-222); ends in ``repack``."""
+        mine = [k[len(prefix):] for k in state_dict if k.startswith(prefix)]
+        assert {k[len("meta."):] for k in mine if k.startswith("meta.")}.issubset(_META_TENSOR_KEYS)
+
+        def take(name):
+            return state_dict.pop(prefix + name)
+
+        self.W_q = take("W_q")
+        self.bias = take("bias") if (prefix + "bias") in state_dict else None
+        if not hasattr(self, "meta"):
+            self.meta = {}
+        meta = self.meta
+        if (prefix + "meta.meta_scale.scale") in state_dict:
+            meta["scale_q"] = take("meta.scale_q")
+            meta["quant_scale"] = True
+            meta.setdefault("meta_scale", {})
+            meta["meta_scale"].update(scale=take("meta.meta_scale.scale"), zero=take("meta.meta_scale.zero"))
+            if meta["scale_q"].dtype != torch.uint8:  # codes saved as fp16 numbers 0..255
+                meta["scale_q"] = meta["scale_q"].to(torch.uint8)
+        else:
+            meta["scale"] = take("meta.scale")
+            meta["quant_scale"] = False
+        if (prefix + "meta.meta_zero.scale") in state_dict:
+            meta["zero_q"] = take("meta.zero_q")
+            meta["quant_zero"] = True
+            meta.setdefault("meta_zero", {})
+            meta["meta_zero"].update(scale=take("meta.meta_zero.scale"), zero=take("meta.meta_zero.zero"))
+            if meta["zero_q"].dtype != torch.uint8:
+                meta["zero_q"] = meta["zero_q"].to(torch.uint8)
+        else:
+            meta["zero"] = take("meta.zero")
+            meta["quant_zero"] = False
+        self.ready = True
+        self.repack()
+
+    @classmethod
+    def _get_tensor_paths(cls, state: Dict[str, Any], prefix=""):
+        paths = []
+        for k, v in state.items():
+            if isinstance(v, dict):
+                paths += cls._get_tensor_paths(v, prefix=k + ".")
+            elif isinstance(v, torch.Tensor):
+                paths.append(prefix + k)
+        return paths
+
+    def state_dict(self, *args, **kwargs):
+        return nn.Module.state_dict(self, *args, **kwargs)
+
+    def load_state_dict(self, *args, **kwargs):
+        nn.Module.load_state_dict(self, *args, **kwargs)
+
+
+class MixtralBLockSparseTop2MLP_HQQ(nn.Module):
+    """Expert FFN ``w2(act(w1 x) * w3 x)`` (reference src/custom_layers.py:243-256).
+
+    ``config`` only needs ``hidden_act``; SiLU runs fused in the HIP library,
+    any other activation takes three separate matmuls."""
+
+    def __init__(self, config, quant_config: Dict[str, Any], meta1, meta2):
+        super().__init__()
+        self.w1 = HQQLinearTritonSavable(None, quant_config, meta1)
+        self.w2 = HQQLinearTritonSavable(None, quant_config, meta2)
+        self.w3 = HQQLinearTritonSavable(None, quant_config, meta1)
+        self.hidden_act = getattr(config, "hidden_act", "silu")
+
+    @torch.inference_mode()
+    def forward(self, hidden_states, out=None, row_scale=None, accumulate=False):
+        if self.hidden_act != "silu":
+            from transformers.activations import ACT2FN
+
+            y = self.w2(ACT2FN[self.hidden_act](self.w1(hidden_states)) * self.w3(hidden_states))
+            if row_scale is not None:
+                y = y * row_scale[:, None]
+            if out is None:
+                return y
+            return out.add_(y) if accumulate else out.copy_(y)
+        x = hidden_states.to(torch.float16).contiguous()
+        y = hip_kernels.expert_ffn(self.w1._desc(), self.w2._desc(), self.w3._desc(), x, out=out,
+                                   row_scale=row_scale, accumulate=accumulate)
+        return y.view(hidden_states.shape[:-1] + (y.shape[-1],)) if out is None else out

@@ -1,0 +1,196 @@
+"""Host side of the unpack-dequantise-matmul kernels.
+
+Keeps the call signatures of the reference's ``src/triton_kernels.py``
+wrappers (``triton_matmul4_transpose`` at :133, ``triton_matmul2_transpose``
+at :321, ``triton_matmul3_transpose`` at :511) and adds the fused entry the
+module layer uses, where the 8-bit scale / zero tables are de-quantised inside
+the kernel instead of being expanded to fp16 first
+(src/custom_layers.py:62-66)."""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import HqqLinear, HqqTable
+
+_workspaces = {}
+
+
+def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    """Per (device, stream) scratch for split-K partial sums; grows on demand.
+    Calls on one stream are ordered, so sharing it between them is safe."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def _table(values: torch.Tensor, meta: Optional[dict]) -> tuple:
+    """(HqqTable, keep-alive) for a scale or zero table: fp16 values, or uint8
+    codes plus the fp16 meta pair of ``Quantizer.quantize``."""
+    t = HqqTable()
+    if meta is None:
+        assert values.dtype == torch.float16, "scale/zero tables must be fp16"
+        v = values.contiguous()
+        t.data, t.kind, t.meta_cols = v.data_ptr(), _lib.HQQ_TABLE_F16, 0
+        return t, (v,)
+    assert values.dtype == torch.uint8, "8-bit scale/zero codes must be uint8"
+    v = values.contiguous()
+    ms = meta["scale"].to(torch.float16).contiguous()
+    mz = meta["zero"].to(torch.float16).contiguous()
+    assert ms.numel() == mz.numel()
+    t.data, t.kind = v.data_ptr(), _lib.HQQ_TABLE_U8
+    t.meta_scale, t.meta_zero, t.meta_cols = ms.data_ptr(), mz.data_ptr(), ms.numel()
+    return t, (v, ms, mz)
+
+
+class LinearDesc:
+    """``hqq_linear`` descriptor of one layer plus the tensors it points into."""
+
+    def __init__(self, W_q: torch.Tensor, meta: dict, bias: Optional[torch.Tensor] = None,
+                 scale: Optional[torch.Tensor] = None, zero: Optional[torch.Tensor] = None):
+        N, K = int(meta["shape"][0]), int(meta["shape"][1])
+        nbits = int(meta["nbits"])
+        codes = W_q.contiguous()
+        if nbits == 3:
+            assert codes.dtype == torch.int32
+            assert 0 <= codes.numel() // K * 10 - N < 10  # reference src/triton_kernels.py:536
+        else:
+            assert codes.dtype == torch.uint8
+            assert codes.numel() == N * K * nbits // 8, "codes are not in the kernel layout (call repack)"
+        if scale is None:
+            scale_t, keep_s = (_table(meta["scale_q"], meta["meta_scale"]) if meta.get("quant_scale")
+                               else _table(meta["scale"], None))
+        else:
+            scale_t, keep_s = _table(scale, None)
+        if zero is None:
+            zero_t, keep_z = (_table(meta["zero_q"], meta["meta_zero"]) if meta.get("quant_zero")
+                              else _table(meta["zero"], None))
+        else:
+            zero_t, keep_z = _table(zero, None)
+        s_cnt = N * K // int(meta["group_size"])
+        for kp in (keep_s, keep_z):
+            assert kp[0].numel() == s_cnt, "scale/zero table does not have N*K/group_size entries"
+        d = HqqLinear()
+        d.nbits, d.group_size, d.N, d.K = nbits, int(meta["group_size"]), N, K
+        d.codes, d.scale, d.zero = codes.data_ptr(), scale_t, zero_t
+        b = None
+        if bias is not None:
+            b = bias.to(torch.float16).contiguous().view(-1)
+            assert b.numel() == N
+            d.bias = b.data_ptr()
+        self.c = d
+        self.N, self.K, self.nbits = N, K, nbits
+        self.device = codes.device
+        self._keep = (codes, keep_s, keep_z, b)
+
+    @property
+    def ref(self):
+        return ctypes.byref(self.c)
+
+
+def matmul(desc: LinearDesc, a: torch.Tensor, family: int = -1) -> torch.Tensor:
+    """C = a @ dequant(W).T (+ bias) on the GPU; fp16 in, fp16 out."""
+    assert a.shape[-1] == desc.K  # reference src/triton_kernels.py:150
+    assert a.is_contiguous(), "A must be contiguous"  # :151
+    assert a.dtype == torch.float16 and a.is_cuda and a.device == desc.device
+    x = a.view(-1, desc.K)
+    M = x.shape[0]
+    c = torch.empty((M, desc.N), device=a.device, dtype=torch.float16)
+    if M > 0:
+        with torch.cuda.device(a.device):
+            need = _lib.lib.hqq_matmul_workspace_bytes(desc.ref, M)
+            ws = workspace(a.device, need)
+            _lib.check(_lib.lib.hqq_matmul_transpose_ex(desc.ref, x.data_ptr(), M, c.data_ptr(), ws.data_ptr(),
+                                                        ws.numel(), family, _lib.current_stream_ptr(a.device)),
+                       "hqq_matmul_transpose")
+    return c.view(a.shape[:-1] + (desc.N,))
+
+
+def kernel_family(desc: LinearDesc, M: int) -> int:
+    return _lib.lib.hqq_matmul_kernel_family(desc.ref, M)
+
+
+def _matmul_fp16_tables(nbits, groupsize, a, qweight, scales, zeros, N, bias):
+    assert scales.shape[1] == zeros.shape[1]  # reference src/triton_kernels.py:152
+    assert scales.shape[1] == qweight.shape[1]  # :153
+    K = qweight.shape[1]
+    meta = {"nbits": nbits, "group_size": groupsize, "shape": (N, K)}
+    desc = LinearDesc(qweight, meta, None, scale=scales, zero=zeros)
+    c = matmul(desc, a)
+    if bias is not None:
+        c = c + bias  # reference :188-189
+    return c
+
+
+def hip_matmul4_transpose(groupsize: int, a, qweight, scales, zeros, bias=None):
+    """Drop-in for ``triton_matmul4_transpose`` (reference src/triton_kernels.py:133-191):
+    ``a`` (..., K) fp16, ``qweight`` (N//2, K) uint8, ``scales`` / ``zeros`` (G, K) fp16."""
+    return _matmul_fp16_tables(4, groupsize, a, qweight, scales, zeros, qweight.shape[0] * 2, bias)
+
+
+def hip_matmul2_transpose(groupsize: int, a, qweight, scales, zeros, bias=None):
+    """Drop-in for ``triton_matmul2_transpose`` (reference src/triton_kernels.py:321-380)."""
+    return _matmul_fp16_tables(2, groupsize, a, qweight, scales, zeros, qweight.shape[0] * 4, bias)
+
+
+def hip_matmul3_transpose(groupsize: int, a, qweight, scales, zeros, N: int, bias=None):
+    """Drop-in for ``triton_matmul3_transpose`` (reference src/triton_kernels.py:511-564)."""
+    assert 0 <= (qweight.shape[0] * 10 - N) < 10  # :536
+    return _matmul_fp16_tables(3, groupsize, a, qweight, scales, zeros, N, bias)
+
+
+# the reference's names, so call sites need no edit
+triton_matmul4_transpose = hip_matmul4_transpose
+triton_matmul2_transpose = hip_matmul2_transpose
+triton_matmul3_transpose = hip_matmul3_transpose
+
+
+def dequantize(desc: LinearDesc) -> torch.Tensor:
+    w = torch.empty((desc.N, desc.K), dtype=torch.float16, device=desc.device)
+    with torch.cuda.device(desc.device):
+        _lib.check(_lib.lib.hqq_dequantize(desc.ref, w.data_ptr(), _lib.current_stream_ptr(desc.device)),
+                   "hqq_dequantize")
+    return w
+
+
+def table_to_f16(values: torch.Tensor, meta: dict) -> torch.Tensor:
+    """``Quantizer.dequantize`` of an 8-bit scale / zero table (reference src/custom_layers.py:63-66)."""
+    t, keep = _table(values, meta)
+    out = torch.empty(meta["shape"] if "shape" in meta else values.shape, dtype=torch.float16, device=values.device)
+    with torch.cuda.device(values.device):
+        _lib.check(_lib.lib.hqq_table_to_f16(ctypes.byref(t), values.numel(), out.data_ptr(),
+                                             _lib.current_stream_ptr(values.device)), "hqq_table_to_f16")
+    del keep
+    return out
+
+
+def expert_ffn(w1: LinearDesc, w2: LinearDesc, w3: LinearDesc, x: torch.Tensor, out: Optional[torch.Tensor] = None,
+               row_scale: Optional[torch.Tensor] = None, accumulate: bool = False) -> torch.Tensor:
+    """w2(silu(w1 x) * w3 x), optionally scaled per row and accumulated into ``out``
+    (reference src/custom_layers.py:253-256, :308-312)."""
+    assert x.dtype == torch.float16 and x.is_contiguous() and x.shape[-1] == w1.K
+    xv = x.view(-1, w1.K)
+    M = xv.shape[0]
+    if out is None:
+        assert not accumulate
+        out = torch.empty((M, w2.N), dtype=torch.float16, device=x.device)
+    assert out.is_contiguous() and out.numel() == M * w2.N
+    if M == 0:
+        return out
+    if row_scale is not None:
+        row_scale = row_scale.to(torch.float16).contiguous()
+        assert row_scale.numel() == M
+    with torch.cuda.device(x.device):
+        need = _lib.lib.hqq_expert_ffn_workspace_bytes(w1.ref, w2.ref, w3.ref, M)
+        ws = workspace(x.device, need)
+        _lib.check(_lib.lib.hqq_expert_ffn(w1.ref, w2.ref, w3.ref, xv.data_ptr(), M, out.data_ptr(),
+                                           row_scale.data_ptr() if row_scale is not None else None,
+                                           int(accumulate), ws.data_ptr(), ws.numel(),
+                                           _lib.current_stream_ptr(x.device)), "hqq_expert_ffn")
+    return out

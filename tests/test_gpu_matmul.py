@@ -1,0 +1,146 @@
+"""GPU parity of hqq_matmul_transpose (every kernel family) against the oracle.
+
+Tolerance (stated by the path's specification): |y - ref| <= 1e-2*|ref| + 1e-3*||x_m||*||w_n||."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import hqq_oracle as o
+from helpers import assert_matmul_close, desc_of, layer_to_device, to_dev
+
+pytestmark = pytest.mark.gpu
+
+# (nbits, N, K, gs, meta_gs, quant_scale, quant_zero)
+SHAPES = [
+    (4, 128, 128, 64, 128, True, True),
+    (4, 256, 512, 64, 128, True, True),
+    (4, 64, 64, 16, 8, False, False),
+    (4, 1024, 256, 64, 256, True, True),
+    (2, 64, 128, 16, 128, True, True),
+    (2, 896, 256, 16, 128, True, True),
+    (2, 256, 448, 16, 128, True, True),
+    (2, 128, 64, 32, 8, False, True),
+    (3, 640, 128, 64, 128, True, True),
+    (3, 448, 256, 64, 128, True, True),
+    (3, 40, 24, 8, 4, False, False),
+    (3, 1280, 192, 64, 128, True, True),
+]
+BATCHES = [1, 2, 4, 8, 16, 17, 33, 128]
+
+
+def _check(layer, x, family=-1, bias=None):
+    from mixtral_offloading_amd import hip_kernels
+    desc = desc_of(layer, bias=bias)
+    y = hip_kernels.matmul(desc, to_dev(x), family=family).cpu().numpy()
+    ref = o.matmul_transpose(x, layer, bias=bias)
+    assert y.shape == ref.shape and y.dtype == np.float16
+    atol = o.matmul_tolerance(x, layer).reshape(ref.shape)
+    return assert_matmul_close(y, ref, atol)
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "w%d_%dx%d_g%d" % s[:4])
+@pytest.mark.parametrize("m", BATCHES)
+def test_matmul_auto_family(shape, m):
+    nbits, n, k, gs, mgs, qs, qz = shape
+    rng = np.random.default_rng(n * 7 + k + m)
+    layer, _ = o.random_layer(rng, n, k, nbits, gs, qs, qz, meta_group_size=mgs)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    _check(layer, x)
+
+
+@pytest.mark.parametrize("family", [0, 1, 2, 3])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "w%d_%dx%d_g%d" % s[:4])
+def test_matmul_forced_family(shape, family):
+    """Every family that accepts a configuration must meet the same tolerance."""
+    from mixtral_offloading_amd import _lib
+    nbits, n, k, gs, mgs, qs, qz = shape
+    rng = np.random.default_rng(n + 3 * k + family)
+    layer, _ = o.random_layer(rng, n, k, nbits, gs, qs, qz, meta_group_size=mgs)
+    ran = 0
+    for m in (1, 5, 16, 40):
+        x = rng.standard_normal((m, k)).astype(np.float16)
+        try:
+            _check(layer, x, family=family)
+            ran += 1
+        except _lib.HqqError as e:
+            assert e.code == -6  # HQQ_E_UNSUPPORTED is the only acceptable refusal
+    if family == 0:
+        assert ran == 4
+
+
+def test_bias_leading_dims_and_empty():
+    from mixtral_offloading_amd import hip_kernels
+    rng = np.random.default_rng(5)
+    layer, _ = o.random_layer(rng, 128, 128, 4, 64)
+    bias = rng.standard_normal(128).astype(np.float16)
+    x = rng.standard_normal((2, 3, 128)).astype(np.float16)
+    _check(layer, x, bias=bias)
+    desc = desc_of(layer)
+    y = hip_kernels.matmul(desc, torch.zeros((0, 128), dtype=torch.float16, device="cuda"))
+    assert tuple(y.shape) == (0, 128)
+
+
+def test_reference_named_wrappers_with_fp16_tables():
+    """triton_matmul{4,2,3}_transpose(groupsize, a, qweight, scales, zeros[, N], bias) signatures."""
+    from mixtral_offloading_amd import hip_kernels
+    rng = np.random.default_rng(9)
+    for nbits, n, k, gs in [(4, 128, 64, 64), (2, 128, 64, 16), (3, 130, 64, 13)]:
+        layer, _ = o.random_layer(rng, n, k, nbits, gs, False, False)
+        x = rng.standard_normal((3, k)).astype(np.float16)
+        bias = rng.standard_normal(n).astype(np.float16)
+        wq, meta = layer_to_device(layer)
+        G = n // gs
+        args = (gs, to_dev(x), wq, meta["scale"].view(G, k), meta["zero"].view(G, k))
+        if nbits == 4:
+            y = hip_kernels.triton_matmul4_transpose(*args, bias=to_dev(bias))
+        elif nbits == 2:
+            y = hip_kernels.triton_matmul2_transpose(*args, bias=to_dev(bias))
+        else:
+            y = hip_kernels.triton_matmul3_transpose(*args, N=n, bias=to_dev(bias))
+        ref = o.matmul_transpose(x, layer, bias=bias)
+        assert_matmul_close(y.cpu().numpy(), ref, o.matmul_tolerance(x, layer))
+    with pytest.raises(AssertionError):  # reference src/triton_kernels.py:150
+        hip_kernels.triton_matmul4_transpose(gs, to_dev(x[:, :-2].copy()), wq, meta["scale"].view(G, k),
+                                             meta["zero"].view(G, k))
+
+
+def _full_size_layer(nbits, n, k, gs, seed):
+    """Random codes / tables at full size, built on the GPU (the values need not come from a quantiser)."""
+    from mixtral_offloading_amd import hip_kernels, packing
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    s_cnt = n * k // gs
+    q = torch.randint(0, 2 ** nbits, (n, k), dtype=torch.uint8, device="cuda", generator=g)
+    pack = {4: packing.pack_4bit_u8_common, 2: packing.pack_2bit_u8_common, 3: packing.pack_3bit_i32_common}[nbits]
+    step = 0.07 / (2 ** nbits - 1)
+    meta = {"nbits": nbits, "group_size": gs, "shape": (n, k), "quant_scale": True, "quant_zero": True,
+            "scale_q": torch.randint(0, 256, (128, s_cnt // 128), dtype=torch.uint8, device="cuda", generator=g),
+            "meta_scale": {"scale": torch.full((1, s_cnt // 128), step / 255, device="cuda").half(),
+                           "zero": torch.full((1, s_cnt // 128), -128.0, device="cuda").half()},
+            "zero_q": torch.randint(0, 256, (1, s_cnt), dtype=torch.uint8, device="cuda", generator=g),
+            "meta_zero": {"scale": torch.tensor([(2 ** nbits - 1) / 255.0], device="cuda").half(),
+                          "zero": torch.tensor([0.0], device="cuda").half()}}
+    return hip_kernels.LinearDesc(pack(q), meta)
+
+
+@pytest.mark.parametrize("nbits,n,k,gs", [(4, 4096, 4096, 64), (4, 1024, 4096, 64), (2, 14336, 4096, 16),
+                                          (2, 4096, 14336, 16), (3, 14336, 4096, 64), (3, 4096, 14336, 64)])
+@pytest.mark.parametrize("m", [1, 4, 8, 16, 128])
+def test_full_size_against_dequantize_then_matmul(nbits, n, k, gs, m):
+    """Mixtral shapes: the library's own bit-exact de-quantiser (checked against the oracle elsewhere) followed by an
+    fp32 torch matmul is the reference's PyTorch path; the fused kernels must agree with it within tolerance."""
+    from mixtral_offloading_amd import hip_kernels
+    desc = _full_size_layer(nbits, n, k, gs, seed=n + k + nbits)
+    g = torch.Generator(device="cuda").manual_seed(m)
+    x = torch.randn((m, k), device="cuda", generator=g).half()
+    w = hip_kernels.dequantize(desc).float()
+    ref = (x.float() @ w.t())
+    y = hip_kernels.matmul(desc, x)
+    atol = 1e-3 * x.float().norm(dim=1)[:, None] * w.norm(dim=1)[None, :]
+    err = (y.float() - ref).abs()
+    bound = 1e-2 * ref.abs() + atol + ref.abs() * 2.0 ** -11  # + fp16 rounding of the reference itself
+    assert bool((err <= bound).all()), float((err / bound).max())
+    # linearity: doubling x doubles y exactly in fp16 (power of two), whatever the summation order
+    # (outputs that round to fp16 subnormals lose that exactness and are left out)
+    y2 = hip_kernels.matmul(desc, (x * 2).contiguous())
+    normal = y.abs() >= 2.0 ** -14
+    assert torch.equal(y2[normal], (y * 2)[normal])
