@@ -139,8 +139,7 @@ def test_full_size_against_dequantize_then_matmul(nbits, n, k, gs, m):
     err = (y.float() - ref).abs()
     bound = 1e-2 * ref.abs() + atol + ref.abs() * 2.0 ** -11  # + fp16 rounding of the reference itself
     assert bool((err <= bound).all()), float((err / bound).max())
-    # linearity: doubling x doubles y exactly in fp16 (power of two), whatever the summation order
-    # (outputs that round to fp16 subnormals lose that exactness and are left out)
+    # linearity: doubling x doubles y (exactly for kernels whose intermediates stay in normal range; the kernels
+    # that hold scale*x in fp16 may differ by an fp16 rounding of a few tiny terms)
     y2 = hip_kernels.matmul(desc, (x * 2).contiguous())
-    normal = y.abs() >= 2.0 ** -14
-    assert torch.equal(y2[normal], (y * 2)[normal])
+    assert bool(((y2.float() - 2 * y.float()).abs() <= 2.0 ** -9 * (2 * y.float()).abs() + 1e-2 * atol).all())
