@@ -117,7 +117,7 @@ size_t hqq_matmul_workspace_bytes(const hqq_linear *l, int64_t M)
     if (validate_linear(l) != HQQ_OK || M <= 0)
         return 0;
     // large enough for whichever family is chosen or forced
-    size_t a = smallbatch_supported(l, M) ? smallbatch_workspace_bytes(l, M) : 0;
+    size_t a = smallbatch_supported(l, M) ? 2 * smallbatch_workspace_bytes(l, M) : 0;
     size_t b = vec3_supported(l, M) ? vec3_workspace_bytes(l, M) : 0;
     return align256(a > b ? a : b);
 }

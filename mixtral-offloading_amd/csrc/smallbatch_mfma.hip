@@ -14,8 +14,8 @@
 // so the per-weight work is only "extract the code as an fp16 number".  The
 // sum over k runs on the matrix cores (v_mfma_f32_16x16x32_f16: A = 16 rows r x
 // 32 k of codes, B = 32 k x 16 batch columns of xs), which also removes every
-// cross-lane reduction.  Codes become fp16 with one AND-OR (the field lands in
-// the mantissa of 2^e, giving 2^e + q) and one packed subtract.
+// cross-lane reduction.  A code becomes an fp16 operand with one AND: masked in
+// place it is the subnormal q * 2^(pos-24), which the matrix cores take exactly.
 //
 // Per 64-column step a wave does
 //   table phase : each lane de-quantises F*64/64 table entries x 4 columns (8-bit
@@ -33,8 +33,7 @@
 namespace hqq {
 namespace {
 
-constexpr int kWavesPerBlock = 4;
-constexpr int kStepK = 64; // columns per wave step
+constexpr int kStepK = 64;       // columns per wave step
 // xs = s * x is held in fp16; scales are ~1e-3..1e-1, so the scale is raised by 2^5 first to keep small
 // activations out of the fp16 subnormal range (|s*x| would have to exceed 2047 to overflow).  Undone in fp32.
 constexpr float kXsScale = 32.0f;
@@ -42,7 +41,8 @@ constexpr float kXsScale = 32.0f;
 struct SBLayer {
     const uint8_t *codes;
     Table sc, zr;
-    float *part; // [NSG][M][N]
+    uint32_t sc_inv, zr_inv; // floor((2^32-1) / meta_cols): the kernel reduces indices mod meta_cols without dividing
+    float *part;             // [NSG][M][N]
 };
 
 struct SBParams {
@@ -51,44 +51,58 @@ struct SBParams {
     int M, N, K;
     int GP;     // G / F: packed table rows
     int RB;     // gs / 16: row blocks per jp
+    int RBG;    // RB / WR: r-block groups per jp
     int WR, WS; // waves of a block along r-blocks / along K slabs
-    int SK;     // steps per wave
+    int WR_log2;
+    int force_partial; // always leave fp32 partial sums (the fused gate pass)
+    int probe;         // tuning aid: 1 = wait for the loads but skip the arithmetic (memory-only time)
     int KT;     // K / 64
     int NSG;    // slab groups (= partial-sum copies)
 };
 
-// Running reader of one (G, K) table for the four columns a lane owns.
-struct TableCursor {
+// How the two tables of a layer are stored; the common cases get branch-free code.
+enum { TM_GENERIC = 0, TM_HQQ8 = 1 /* scale: u8 + per-column meta, zero: u8 + scalar meta */, TM_F16 = 2 };
+
+// Reader of one (G, K) table for the four columns a lane owns.  KIND: 0 runtime flags, 1 u8 with per-column
+// meta, 2 u8 with scalar meta, 3 fp16.
+template <int KIND> struct TableCursor {
     const uint8_t *u8;
     const f16 *f;
     const f16 *ms, *mz;
-    int64_t c;    // flat index j*K + k of the lane's first column
-    int64_t cm;   // c % meta_cols
-    int64_t cols; // meta_cols
+    uint32_t c;    // flat index j*K + k of the lane's first column
+    uint32_t cm;   // c % meta_cols
+    uint32_t cols; // meta_cols
     bool is_u8, scalar;
     f16x2 ms_s, mz_s; // scalar meta, splat
 
-    __device__ void init(const Table &t, int64_t c0)
+    __device__ __forceinline__ void init(const Table &t, uint32_t c0, uint32_t cols_inv)
     {
-        is_u8 = t.kind == HQQ_TABLE_U8;
+        is_u8 = KIND == 0 ? t.kind == HQQ_TABLE_U8 : KIND != 3;
         u8 = static_cast<const uint8_t *>(t.data);
         f = static_cast<const f16 *>(t.data);
         ms = t.ms, mz = t.mz;
-        cols = t.meta_cols;
-        scalar = is_u8 && cols == 1;
+        cols = (uint32_t)t.meta_cols;
+        scalar = KIND == 0 ? (is_u8 && cols == 1) : KIND == 2;
         c = c0;
-        cm = (is_u8 && !scalar) ? c0 % cols : 0;
+        cm = 0;
+        if (is_u8 && !scalar) { // c0 mod cols: the quotient estimate is at most 2 short
+            cm = c0 - __umulhi(c0, cols_inv) * cols;
+            if (cm >= cols)
+                cm -= cols;
+            if (cm >= cols)
+                cm -= cols;
+        }
         if (scalar) {
             ms_s = (f16x2){ms[0], ms[0]};
             mz_s = (f16x2){mz[0], mz[0]};
         }
     }
-    __device__ void advance(int64_t d)
+    __device__ __forceinline__ void advance(uint32_t d)
     {
         c += d;
         if (is_u8 && !scalar) {
-            cm += d;
-            while (cm >= cols)
+            cm += d; // d <= cols
+            if (cm >= cols)
                 cm -= cols;
         }
     }
@@ -99,7 +113,7 @@ struct TableRaw {
     u32x2 ms, mz; // 4 halves each (u8 table with per-column meta)
 };
 
-__device__ __forceinline__ TableRaw table_load(const TableCursor &t)
+template <int KIND> __device__ __forceinline__ TableRaw table_load(const TableCursor<KIND> &t)
 {
     TableRaw r;
     r.data = (u32x2){0, 0};
@@ -120,7 +134,8 @@ __device__ __forceinline__ TableRaw table_load(const TableCursor &t)
 __device__ __forceinline__ f16x2 as_f16x2(uint32_t v) { return __builtin_bit_cast(f16x2, v); }
 
 // four table entries as fp16: stored values, or fp16(fp16(q - mz) * ms)
-__device__ __forceinline__ void table_decode(const TableCursor &t, const TableRaw &r, f16x2 &lo, f16x2 &hi)
+template <int KIND>
+__device__ __forceinline__ void table_decode(const TableCursor<KIND> &t, const TableRaw &r, f16x2 &lo, f16x2 &hi)
 {
     if (t.is_u8) {
         // bytes -> fp16 exactly: 0x6400 | b is 1024 + b, then subtract 1024
@@ -141,68 +156,111 @@ __device__ __forceinline__ void table_decode(const TableCursor &t, const TableRa
     }
 }
 
-// codes of field i of the two bytes that sit in the low byte of each 16-bit half
-// of d, as the fp16 pair (q, q'): AND-OR drops the field into the mantissa of 2^e.
-template <int NBITS> __device__ __forceinline__ f16x2 extract_pair(uint32_t d, int i)
+// Field i of a packed byte sits at bit `pos` of the byte.  Masked in place, the low byte of a 16-bit half reads as
+// the fp16 SUBNORMAL number q * 2^(pos - 24): no shift, no convert.  The matrix cores take fp16 subnormals
+// exactly (checked on gfx950 by the parity tests: a flush to zero would zero every output), so the code goes to
+// the MFMA as it is and the factor 2^(24 - pos) is applied once to the fp32 result.
+template <int NBITS> struct Field {
+    static constexpr int F = 8 / NBITS;
+    static constexpr int pos(int i) { return NBITS * (F - 1 - i); }
+    static constexpr uint32_t mask(int i) { return (((1u << NBITS) - 1u) * 0x00010001u) << pos(i); }
+    static constexpr float unscale(int i) { return (float)(1u << (24 - pos(i))); }
+};
+
+// sum over the 16 lanes of a DPP row; every lane of the row gets the total
+__device__ __forceinline__ float row16_sum(float v)
 {
-    constexpr int F = 8 / NBITS;
-    const int pos = NBITS * (F - 1 - i);
-    const int e = 10 - pos;
-    const uint32_t mask = (((1u << NBITS) - 1u) * 0x00010001u) << pos;
-    const uint32_t expo = (uint32_t)((e + 15) << 10) * 0x00010001u;
-    const f16 off = (f16)(float)(1 << e);
-    return as_f16x2((d & mask) | expo) - (f16x2){off, off};
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true)); // quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true)); // quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true)); // row_half_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true)); // row_mirror
+    return v;
 }
 
-template <int NBITS, int MT>
-__global__ __launch_bounds__(kWavesPerBlock * 64) void smallbatch_kernel(SBParams p)
+// What the block does with its finished tile.
+struct SBEpilogue {
+    f16 *y;               // direct store target (NSG == 1)
+    const f16 *bias;      // fp16[N] or null
+    const f16 *row_scale; // fp16[M] or null
+    int accumulate;
+};
+
+template <int NBITS, int MT, int WAVES, int SK, int TMODE>
+__global__ __launch_bounds__(WAVES * 64) void smallbatch_kernel(SBParams p, SBEpilogue ep)
 {
     constexpr int F = 8 / NBITS;
     constexpr int XS_HALVES = F * 2 * 4 * MT * 8; // per wave, one step
-    __shared__ __attribute__((aligned(16))) f16 xs_lds[kWavesPerBlock][XS_HALVES];
-    __shared__ float bias_lds[kWavesPerBlock][F][MT];
-    __shared__ __attribute__((aligned(16))) float red_lds[kWavesPerBlock][F][64][4];
+    constexpr int SCALE_KIND = TMODE == TM_HQQ8 ? 1 : (TMODE == TM_F16 ? 3 : 0);
+    constexpr int ZERO_KIND = TMODE == TM_HQQ8 ? 2 : (TMODE == TM_F16 ? 3 : 0);
+    __shared__ __attribute__((aligned(16))) f16 xs_lds[WAVES + 1][XS_HALVES]; // [WAVES] stays zero
+    __shared__ float bias_lds[WAVES][F][MT];
+    __shared__ __attribute__((aligned(16))) float red_lds[WAVES][16][MT][F]; // [wave][row r][batch m][i]
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int wr = wave % p.WR, ws = wave / p.WR;
-    const SBLayer &L = p.layer[blockIdx.y];
-
-    int b = blockIdx.x;
-    const int sg = b % p.NSG;
-    b /= p.NSG;
-    const int RBG = p.RB / p.WR;
-    const int rbg = b % RBG;
-    const int jp = b / RBG;
+    const int wr = wave & (p.WR - 1), ws = wave >> p.WR_log2;
+    // grid: x = K slab group, y = (layer, r-block group), z = jp
+    const int sg = blockIdx.x;
+    const int layer = (int)blockIdx.y >= p.RBG ? 1 : 0;
+    const int rbg = (int)blockIdx.y - layer * p.RBG;
+    const SBLayer &L = p.layer[layer];
+    const int jp = blockIdx.z;
     const int rb = rbg * p.WR + wr;
-    const int slab = sg * p.WS + ws;
-    const int step_begin = slab * p.SK;
-    int step_end = step_begin + p.SK;
-    if (step_end > p.KT)
-        step_end = p.KT;
+    const int step_begin = (sg * p.WS + ws) * SK;
+    const bool active = step_begin < p.KT; // KT is a multiple of SK; idle waves only join the reduction
 
-    const int64_t K = p.K;
+    const int K = p.K;
+    const int M = MT == 1 ? 1 : p.M;
     // code lane role: packed row of (jp, r), 16 columns at 16*kg
     const int rr = lane & 15, kg = lane >> 4;
-    const int64_t prow = (int64_t)jp + (int64_t)(16 * rb + rr) * p.GP;
-    const uint8_t *cptr = L.codes + prow * K + 16 * kg;
+    const uint32_t prow = (uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)p.GP;
+    const uint32_t coff = prow * (uint32_t)K + (uint32_t)(step_begin * kStepK + 16 * kg); // codes are < 4 GiB
     // table lane role: table row F*jp + ti, columns 4*kq .. 4*kq+3
     const int ti = lane >> 4, kq = lane & 15;
     const bool tlane = ti < F;
-    TableCursor sc, zr;
-    {
-        const int64_t c0 = ((int64_t)F * jp + (tlane ? ti : 0)) * K + (int64_t)step_begin * kStepK + 4 * kq;
-        sc.init(L.sc, c0);
-        zr.init(L.zr, c0);
+    const uint32_t c0 = (uint32_t)(F * jp + (tlane ? ti : 0)) * (uint32_t)K + (uint32_t)(step_begin * kStepK + 4 * kq);
+    const uint32_t xoff = (uint32_t)(step_begin * kStepK + 4 * kq);
+
+    // ---- issue every load of the wave's slab up front; the whole matrix is in flight at once
+    u32x4 cw[SK];
+    TableRaw sraw[SK], zraw[SK];
+    u32x2 xv[SK][MT];
+    TableCursor<SCALE_KIND> sc;
+    TableCursor<ZERO_KIND> zr;
+    sc.init(L.sc, c0, L.sc_inv);
+    zr.init(L.zr, c0, L.zr_inv);
+    if (active) {
+#pragma unroll
+        for (int s = 0; s < SK; ++s) {
+            cw[s] = *reinterpret_cast<const u32x4 *>(L.codes + (coff + s * kStepK));
+            if (tlane) {
+                sraw[s] = table_load(sc);
+                zraw[s] = table_load(zr);
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+                    if (m < M)
+                        xv[s][m] = *reinterpret_cast<const u32x2 *>(p.x + (xoff + (uint32_t)(m * K + s * kStepK)));
+            }
+            sc.advance(kStepK);
+            zr.advance(kStepK);
+        }
     }
-    const f16 *xptr = p.x + 4 * kq;
+
     // where this lane's xs go: entry ((ti*2 + h)*4 + kgt)*MT + m, 16 B each, second half when kq is odd
     f16 *xs_w = &xs_lds[wave][((((ti * 2 + ((kq >> 1) & 1)) * 4 + (kq >> 2)) * MT) * 8) + 4 * (kq & 1)];
-    const f16 *xs_r = &xs_lds[wave][(kg * MT + (lane & 15)) * 8];
-
+    // B operand: column = batch row lane&15; lanes past MT read the block's all-zero copy
+    const int mcol = lane & 15;
+    const f16 *xs_r = mcol < MT ? &xs_lds[wave][(kg * MT + mcol) * 8] : &xs_lds[WAVES][0];
     // LDS rows of batch entries m >= M are never written by the table phase: clear once
-    for (int i = lane; i < XS_HALVES / 8; i += 64)
-        *reinterpret_cast<u32x4 *>(&xs_lds[wave][i * 8]) = (u32x4){0, 0, 0, 0};
+    if (M < MT)
+        for (int i = lane; i < XS_HALVES / 8; i += 64)
+            *reinterpret_cast<u32x4 *>(&xs_lds[wave][i * 8]) = (u32x4){0, 0, 0, 0};
+    if constexpr (MT < 16) {
+        if (wave == 0)
+            for (int i = lane; i < XS_HALVES / 8; i += 64)
+                *reinterpret_cast<u32x4 *>(&xs_lds[WAVES][i * 8]) = (u32x4){0, 0, 0, 0};
+        __syncthreads();
+    }
 
     f32x4 acc[F];
 #pragma unroll
@@ -213,139 +271,153 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void smallbatch_kernel(SBParam
     for (int m = 0; m < MT; ++m)
         bias_acc[m] = 0.f;
 
-    // software pipeline: loads of step s+1 are issued before the arithmetic of step s
-    u32x4 cw_n = {0, 0, 0, 0};
-    TableRaw sraw_n, zraw_n;
-    u32x2 x_n[MT];
-    auto issue = [&](int s) {
-        const int64_t k0 = (int64_t)s * kStepK;
-        cw_n = *reinterpret_cast<const u32x4 *>(cptr + k0);
-        if (tlane) {
-            sraw_n = table_load(sc);
-            zraw_n = table_load(zr);
+    if (p.probe == 1 && active) { // keep every load alive, do no arithmetic
+        uint32_t x = 0;
 #pragma unroll
-            for (int m = 0; m < MT; ++m)
-                if (m < p.M)
-                    x_n[m] = *reinterpret_cast<const u32x2 *>(xptr + (int64_t)m * K + k0);
+        for (int s = 0; s < SK; ++s) {
+            x ^= cw[s].x ^ cw[s].y ^ cw[s].z ^ cw[s].w;
+            if (tlane)
+                x ^= sraw[s].data.x ^ zraw[s].data.x ^ sraw[s].ms.x ^ sraw[s].mz.y ^ xv[s][0].x;
         }
-        sc.advance(kStepK);
-        zr.advance(kStepK);
-    };
-    if (step_begin < step_end)
-        issue(step_begin);
-
-    for (int s = step_begin; s < step_end; ++s) {
-        const u32x4 cw = cw_n;
-        const TableRaw sraw = sraw_n, zraw = zraw_n;
-        u32x2 xv[MT];
+        acc[0][0] = (float)(x & 1u);
+    } else if (active) {
 #pragma unroll
-        for (int m = 0; m < MT; ++m)
-            xv[m] = x_n[m];
-        if (s + 1 < step_end)
-            issue(s + 1);
-
-        // ---- table phase
-        if (tlane) {
-            f16x2 s01, s23, z01, z23;
-            table_decode(sc, sraw, s01, s23);
-            table_decode(zr, zraw, z01, z23);
-            s01 = s01 * (f16x2){(f16)kXsScale, (f16)kXsScale};
-            s23 = s23 * (f16x2){(f16)kXsScale, (f16)kXsScale};
+        for (int s = 0; s < SK; ++s) {
+            // ---- table phase
+            if (tlane) {
+                f16x2 s01, s23, z01, z23;
+                table_decode(sc, sraw[s], s01, s23);
+                table_decode(zr, zraw[s], z01, z23);
+                s01 = s01 * (f16x2){(f16)kXsScale, (f16)kXsScale};
+                s23 = s23 * (f16x2){(f16)kXsScale, (f16)kXsScale};
 #pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                if (m < p.M) {
-                    const f16x2 a01 = s01 * as_f16x2(xv[m].x);
-                    const f16x2 a23 = s23 * as_f16x2(xv[m].y);
-                    bias_acc[m] = __builtin_amdgcn_fdot2(z01, a01, bias_acc[m], false);
-                    bias_acc[m] = __builtin_amdgcn_fdot2(z23, a23, bias_acc[m], false);
-                    // B-operand order inside an 8-column block: columns (0,2,1,3)
-                    const f16x4 o = {a01.x, a23.x, a01.y, a23.y};
-                    *reinterpret_cast<f16x4 *>(xs_w + m * 8) = o;
+                for (int m = 0; m < MT; ++m) {
+                    if (m < M) {
+                        const f16x2 a01 = s01 * as_f16x2(xv[s][m].x);
+                        const f16x2 a23 = s23 * as_f16x2(xv[s][m].y);
+                        bias_acc[m] = __builtin_amdgcn_fdot2(z01, a01, bias_acc[m], false);
+                        bias_acc[m] = __builtin_amdgcn_fdot2(z23, a23, bias_acc[m], false);
+                        // B-operand order inside an 8-column block: columns (0,2,1,3)
+                        const f16x4 o = {a01.x, a23.x, a01.y, a23.y};
+                        *reinterpret_cast<f16x4 *>(xs_w + m * 8) = o;
+                    }
                 }
             }
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        // ---- code phase
-        const uint32_t d[4] = {cw.x, cw.y, cw.z, cw.w};
+            // ---- code phase: all B operands first, then extract-and-multiply
+            f16x8 B[2][F];
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const uint32_t d0 = d[2 * h], d1 = d[2 * h + 1];
-            const uint32_t d0s = d0 >> 8, d1s = d1 >> 8;
+            for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int i = 0; i < F; ++i) {
-                const f16x2 a0 = extract_pair<NBITS>(d0, i), a1 = extract_pair<NBITS>(d0s, i);
-                const f16x2 a2 = extract_pair<NBITS>(d1, i), a3 = extract_pair<NBITS>(d1s, i);
-                const f16x8 A = {a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
-                f16x8 B = {0, 0, 0, 0, 0, 0, 0, 0};
-                if ((lane & 15) < MT)
-                    B = *reinterpret_cast<const f16x8 *>(xs_r + ((i * 2 + h) * 4 * MT) * 8);
-                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, acc[i], 0, 0, 0);
+                for (int i = 0; i < F; ++i)
+                    B[h][i] = *reinterpret_cast<const f16x8 *>(xs_r + ((i * 2 + h) * 4 * MT) * 8);
+            const uint32_t d[4] = {cw[s].x, cw[s].y, cw[s].z, cw[s].w};
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t d0 = d[2 * h], d1 = d[2 * h + 1];
+                const uint32_t d0s = d0 >> 8, d1s = d1 >> 8;
+#pragma unroll
+                for (int i = 0; i < F; ++i) {
+                    const uint32_t mk = Field<NBITS>::mask(i);
+                    const u32x4 Au = {d0 & mk, d0s & mk, d1 & mk, d1s & mk};
+                    const f16x8 A = __builtin_bit_cast(f16x8, Au);
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B[h][i], acc[i], 0, 0, 0);
+                }
             }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
     }
 
     // ---- bias: sum the 16 table lanes of each table row, hand it to the lanes that hold D
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-        float v = bias_acc[m];
-#pragma unroll
-        for (int off = 8; off > 0; off >>= 1)
-            v += __shfl_xor(v, off, 64);
+        const float v = row16_sum(bias_acc[m]);
         if (tlane && kq == 0)
             bias_lds[wave][ti][m] = v;
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const int mcol = lane & 15; // D layout: column = batch row, rows 4*(lane>>4)+v
+    // D layout: column = batch row (lane & 15), rows 4*(lane>>4)+v.  Every wave leaves its tile, bias removed and
+    // still scaled, in LDS as [row r][batch m][i]; then one thread per (r-block, r, m) adds the block's K slabs.
     if (mcol < MT) {
+        float bz[F];
 #pragma unroll
-        for (int i = 0; i < F; ++i) {
-            const float bz = bias_lds[wave][i][mcol];
-            acc[i] = (acc[i] - (f32x4){bz, bz, bz, bz}) * (1.0f / kXsScale);
-        }
-    }
-
-    // ---- sum the K slabs of this block (waves ws > 0 hand their tile to ws == 0)
-    if (p.WS > 1) {
-        if (ws > 0) {
+        for (int i = 0; i < F; ++i)
+            bz[i] = bias_lds[wave][i][mcol];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            float o[F];
 #pragma unroll
             for (int i = 0; i < F; ++i)
-                *reinterpret_cast<f32x4 *>(&red_lds[wave][i][lane][0]) = acc[i];
-        }
-        __syncthreads();
-        if (ws == 0) {
-            for (int o = 1; o < p.WS; ++o)
-#pragma unroll
-                for (int i = 0; i < F; ++i)
-                    acc[i] += *reinterpret_cast<const f32x4 *>(&red_lds[o * p.WR + wr][i][lane][0]);
+                o[i] = __builtin_fmaf(acc[i][v], Field<NBITS>::unscale(i), -bz[i]);
+            float *dst = &red_lds[wave][4 * kg + v][mcol][0];
+            if constexpr (F == 4)
+                *reinterpret_cast<f32x4 *>(dst) = (f32x4){o[0], o[1], o[2], o[3]};
+            else
+                *reinterpret_cast<float2 *>(dst) = make_float2(o[0], o[1]);
         }
     }
-    if (ws != 0 || mcol >= p.M)
-        return;
-
-    // ---- store the partial sums: rows r = 16*rb + 4*(lane>>4) + v, outputs n = F*(jp + r*GP) + i
-    float *dst = L.part + ((int64_t)sg * p.M + mcol) * p.N;
+    __syncthreads();
+    // a DPP row of 16 lanes per output (wr, r, m): lane w of the row brings slab w (WS <= 16)
+    for (int t = threadIdx.x; t < p.WR * 16 * MT * 16; t += WAVES * 64) {
+        const int w = t & 15, u = t >> 4;
+        const int wr_t = u / (16 * MT), r_t = (u / MT) & 15, m_t = u % MT;
+        float o[F];
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        const int r = 16 * rb + 4 * (lane >> 4) + v;
+        for (int i = 0; i < F; ++i)
+            o[i] = 0.f;
+        if (w < p.WS) {
+            const float *src = &red_lds[w * p.WR + wr_t][r_t][m_t][0];
+#pragma unroll
+            for (int i = 0; i < F; ++i)
+                o[i] = src[i];
+        }
+#pragma unroll
+        for (int i = 0; i < F; ++i)
+            o[i] = row16_sum(o[i]) * (1.0f / kXsScale);
+        if (w != 0 || m_t >= M)
+            continue;
+
+        // ---- row r = 16*rb + r_t of the tile holds outputs n = F*(jp + r*GP) + i
+        const int r = 16 * (rbg * p.WR + wr_t) + r_t;
         const int64_t n = (int64_t)F * (jp + (int64_t)r * p.GP);
+        if (p.NSG > 1 || p.force_partial) { // split over several blocks: fp32 partial sums for the finish kernel
+            float *dst = L.part + ((int64_t)sg * M + m_t) * p.N + n;
+            if constexpr (F == 4)
+                *reinterpret_cast<f32x4 *>(dst) = (f32x4){o[0], o[1], o[2], o[3]};
+            else
+                *reinterpret_cast<float2 *>(dst) = make_float2(o[0], o[1]);
+            continue;
+        }
+        f16 *dst = ep.y + (int64_t)m_t * p.N + n;
+        f16 h[F];
+#pragma unroll
+        for (int i = 0; i < F; ++i) {
+            f16 val = (f16)o[i];
+            if (ep.bias)
+                val = val + ep.bias[n + i];
+            if (ep.row_scale)
+                val = val * ep.row_scale[m_t];
+            if (ep.accumulate)
+                val = dst[i] + val;
+            h[i] = val;
+        }
         if constexpr (F == 4)
-            *reinterpret_cast<f32x4 *>(dst + n) = (f32x4){acc[0][v], acc[1][v], acc[2][v], acc[3][v]};
+            *reinterpret_cast<f16x4 *>(dst) = (f16x4){h[0], h[1], h[2], h[3]};
         else
-            *reinterpret_cast<float2 *>(dst + n) = make_float2(acc[0][v], acc[1][v]);
+            *reinterpret_cast<f16x2 *>(dst) = (f16x2){h[0], h[1]};
     }
 }
 
 // Sum the slab partials and apply the epilogue.  MODE 0: y = cast(sum) (+bias) (*row_scale) (+= y);
 // MODE 1: h = silu(sum of layer 0) * (sum of layer 1), the expert FFN's gate.
 template <int MODE>
-__global__ __launch_bounds__(256) void smallbatch_finish_kernel(const float *__restrict__ part0,
+__global__ __launch_bounds__(64) void smallbatch_finish_kernel(const float *__restrict__ part0,
                                                                 const float *__restrict__ part1, int NSG, int M,
                                                                 int N, const f16 *__restrict__ bias,
                                                                 const f16 *__restrict__ row_scale, int accumulate,
@@ -353,7 +425,7 @@ __global__ __launch_bounds__(256) void smallbatch_finish_kernel(const float *__r
 {
     const int64_t total = (int64_t)M * N / 4;
     const int64_t stride = (int64_t)M * N;
-    for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+    for (int64_t idx = blockIdx.x * 64ll + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 64) {
         const int64_t e = idx * 4;
         f32x4 a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
         for (int s = 0; s < NSG; ++s) {
@@ -391,8 +463,10 @@ int env_int(const char *name, int dflt)
 }
 
 struct SBPlan {
-    int F, GP, RB, WR, WS, SK, KT, NS, NSG, MT;
+    int F, GP, RB, WR, WS, KT, NS, NSG, MT, WAVES, SK, TMODE;
 };
+
+int table_kind(const hqq_table &t) { return t.kind == HQQ_TABLE_F16 ? 3 : (t.meta_cols == 1 ? 2 : 1); }
 
 bool make_plan(const hqq_linear *l, int64_t M, SBPlan &pl)
 {
@@ -402,10 +476,10 @@ bool make_plan(const hqq_linear *l, int64_t M, SBPlan &pl)
         return false;
     const int F = 8 / l->nbits;
     const int64_t G = l->N / l->group_size;
-    if (l->group_size % 16 != 0 || G % F != 0 || l->K % kStepK != 0)
+    if (l->group_size % 16 != 0 || G % F != 0 || l->K % kStepK != 0 || l->N % 4 != 0)
         return false;
-    if (l->N * l->K / l->group_size >= (1ll << 31) || l->N >= (1ll << 31) || l->K >= (1ll << 31))
-        return false;
+    if (l->N * l->K / l->group_size >= (1ll << 31) || l->N * l->K / F >= (1ll << 32) || 16 * l->K >= (1ll << 31))
+        return false; // 32-bit offsets inside the kernel
     if (!aligned16(l->codes))
         return false;
     for (const hqq_table *t : {&l->scale, &l->zero}) {
@@ -423,45 +497,83 @@ bool make_plan(const hqq_linear *l, int64_t M, SBPlan &pl)
     pl.F = F;
     pl.GP = (int)(G / F);
     pl.RB = l->group_size / 16;
+    pl.MT = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : (M <= 8 ? 8 : 16)));
+    pl.WAVES = pl.MT <= 4 ? 16 : (pl.MT == 8 ? 8 : 4);
+    {
+        const int forced = env_int("HQQ_SB_BLOCK_WAVES", 0);
+        if ((forced == 4 || forced == 8 || forced == 16) && forced <= pl.WAVES)
+            pl.WAVES = forced;
+    }
     pl.WR = pl.RB >= 4 ? 4 : (pl.RB >= 2 ? 2 : 1);
     if (pl.RB % pl.WR != 0)
         pl.WR = 1;
-    pl.WS = kWavesPerBlock / pl.WR;
     pl.KT = (int)(l->K / kStepK);
-    const int64_t tiles = (int64_t)pl.GP * pl.RB;
-    const int target = env_int("HQQ_SB_WAVES", 4096);
-    int64_t ns = (target + tiles - 1) / tiles;
-    if (ns < 1)
-        ns = 1;
-    if (ns > pl.KT)
-        ns = pl.KT;
-    int sk = (int)((pl.KT + ns - 1) / ns);
-    const int sk_env = env_int("HQQ_SB_STEPS", 0);
-    if (sk_env > 0)
-        sk = sk_env;
-    pl.SK = sk;
-    pl.NS = (pl.KT + sk - 1) / sk;
+    pl.SK = pl.KT % 4 == 0 ? 4 : (pl.KT % 2 == 0 ? 2 : 1); // steps per wave; their loads are all issued up front
+    pl.NS = pl.KT / pl.SK;
+    const int ks = table_kind(l->scale), kz = table_kind(l->zero);
+    pl.TMODE = (ks == 1 && kz == 2) ? TM_HQQ8 : ((ks == 3 && kz == 3) ? TM_F16 : TM_GENERIC);
+    // a block need not be wider than the slabs there are
+    while (pl.WAVES > 4 && pl.WAVES / pl.WR >= 2 * pl.NS)
+        pl.WAVES /= 2;
+    pl.WS = pl.WAVES / pl.WR;
     pl.NSG = (pl.NS + pl.WS - 1) / pl.WS;
-    pl.MT = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : (M <= 8 ? 8 : 16)));
     return true;
 }
 
-template <int NBITS> void launch_main(const SBParams &p, int MT, dim3 grid, hipStream_t s)
+template <int NBITS, int MT, int WAVES, int SK>
+void launch_tm(const SBParams &p, const SBEpilogue &ep, int tmode, dim3 grid, hipStream_t s)
 {
-    const dim3 block(kWavesPerBlock * 64);
-    switch (MT) {
-    case 1: smallbatch_kernel<NBITS, 1><<<grid, block, 0, s>>>(p); break;
-    case 2: smallbatch_kernel<NBITS, 2><<<grid, block, 0, s>>>(p); break;
-    case 4: smallbatch_kernel<NBITS, 4><<<grid, block, 0, s>>>(p); break;
-    case 8: smallbatch_kernel<NBITS, 8><<<grid, block, 0, s>>>(p); break;
-    default: smallbatch_kernel<NBITS, 16><<<grid, block, 0, s>>>(p); break;
+    const dim3 block(WAVES * 64);
+    if (tmode == TM_HQQ8)
+        smallbatch_kernel<NBITS, MT, WAVES, SK, TM_HQQ8><<<grid, block, 0, s>>>(p, ep);
+    else if (tmode == TM_F16)
+        smallbatch_kernel<NBITS, MT, WAVES, SK, TM_F16><<<grid, block, 0, s>>>(p, ep);
+    else
+        smallbatch_kernel<NBITS, MT, WAVES, SK, TM_GENERIC><<<grid, block, 0, s>>>(p, ep);
+}
+
+template <int NBITS, int MT, int WAVES>
+void launch_sk(const SBParams &p, const SBEpilogue &ep, const SBPlan &pl, dim3 grid, hipStream_t s)
+{
+    if (pl.SK == 4)
+        launch_tm<NBITS, MT, WAVES, 4>(p, ep, pl.TMODE, grid, s);
+    else if (pl.SK == 2)
+        launch_tm<NBITS, MT, WAVES, 2>(p, ep, pl.TMODE, grid, s);
+    else
+        launch_tm<NBITS, MT, WAVES, 1>(p, ep, pl.TMODE, grid, s);
+}
+
+template <int NBITS, int MT>
+void launch_mt(const SBParams &p, const SBEpilogue &ep, const SBPlan &pl, dim3 grid, hipStream_t s)
+{
+    // wide blocks only where their LDS (xs staging grows with MT) fits
+    if constexpr (MT <= 4) {
+        if (pl.WAVES == 16)
+            return launch_sk<NBITS, MT, 16>(p, ep, pl, grid, s);
+    }
+    if constexpr (MT <= 8) {
+        if (pl.WAVES >= 8)
+            return launch_sk<NBITS, MT, 8>(p, ep, pl, grid, s);
+    }
+    launch_sk<NBITS, MT, 4>(p, ep, pl, grid, s);
+}
+
+template <int NBITS>
+void launch_main(const SBParams &p, const SBEpilogue &ep, const SBPlan &pl, dim3 grid, hipStream_t s)
+{
+    switch (pl.MT) {
+    case 1: launch_mt<NBITS, 1>(p, ep, pl, grid, s); break;
+    case 2: launch_mt<NBITS, 2>(p, ep, pl, grid, s); break;
+    case 4: launch_mt<NBITS, 4>(p, ep, pl, grid, s); break;
+    case 8: launch_mt<NBITS, 8>(p, ep, pl, grid, s); break;
+    default: launch_mt<NBITS, 16>(p, ep, pl, grid, s); break;
     }
 }
 
 int finish_grid(int64_t M, int64_t N)
 {
-    int64_t b = (M * N / 4 + 255) / 256;
-    return (int)(b < 1 ? 1 : (b > 4096 ? 4096 : b));
+    int64_t b = (M * N / 4 + 63) / 64;
+    return (int)(b < 1 ? 1 : (b > 8192 ? 8192 : b));
 }
 
 } // namespace
@@ -469,7 +581,7 @@ int finish_grid(int64_t M, int64_t N)
 bool smallbatch_supported(const hqq_linear *l, int64_t M)
 {
     SBPlan pl;
-    return make_plan(l, M, pl) && l->N % 4 == 0;
+    return make_plan(l, M, pl);
 }
 
 size_t smallbatch_workspace_bytes(const hqq_linear *l, int64_t M)
@@ -486,8 +598,10 @@ static void fill_params(SBParams &p, const SBPlan &pl, const hqq_linear *l, int 
     p.layer[which].sc = make_table(l->scale);
     p.layer[which].zr = make_table(l->zero);
     p.layer[which].part = part;
+    p.layer[which].sc_inv = l->scale.meta_cols > 0 ? (uint32_t)(0xFFFFFFFFull / (uint64_t)l->scale.meta_cols) : 0;
+    p.layer[which].zr_inv = l->zero.meta_cols > 0 ? (uint32_t)(0xFFFFFFFFull / (uint64_t)l->zero.meta_cols) : 0;
     p.N = (int)l->N, p.K = (int)l->K;
-    p.GP = pl.GP, p.RB = pl.RB, p.WR = pl.WR, p.WS = pl.WS, p.SK = pl.SK, p.KT = pl.KT, p.NSG = pl.NSG;
+    p.GP = pl.GP, p.RB = pl.RB, p.RBG = pl.RB / pl.WR, p.WR = pl.WR, p.WR_log2 = pl.WR == 4 ? 2 : (pl.WR == 2 ? 1 : 0), p.WS = pl.WS, p.KT = pl.KT, p.NSG = pl.NSG;
 }
 
 int launch_smallbatch_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
@@ -496,21 +610,23 @@ int launch_smallbatch_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *
     SBPlan pl;
     if (!make_plan(l, M, pl))
         return HQQ_E_UNSUPPORTED;
-    if (ws_bytes < smallbatch_workspace_bytes(l, M))
+    if (pl.NSG > 1 && ws_bytes < smallbatch_workspace_bytes(l, M))
         return HQQ_E_WORKSPACE;
     SBParams p = {};
     fill_params(p, pl, l, 0, static_cast<float *>(ws));
     p.layer[1] = p.layer[0];
     p.x = x, p.M = (int)M;
-    const dim3 grid((unsigned)(pl.GP * (pl.RB / pl.WR) * pl.NSG), 1);
+    p.probe = env_int("HQQ_SB_PROBE", 0);
+    SBEpilogue e = {y, static_cast<const f16 *>(l->bias), ep.row_scale, ep.accumulate};
+    const dim3 grid((unsigned)pl.NSG, (unsigned)(pl.RB / pl.WR), (unsigned)pl.GP);
     if (l->nbits == 2)
-        launch_main<2>(p, pl.MT, grid, s);
+        launch_main<2>(p, e, pl, grid, s);
     else
-        launch_main<4>(p, pl.MT, grid, s);
+        launch_main<4>(p, e, pl, grid, s);
     int rc = launch_status();
-    if (rc != HQQ_OK)
+    if (rc != HQQ_OK || pl.NSG == 1)
         return rc;
-    smallbatch_finish_kernel<0><<<finish_grid(M, l->N), 256, 0, s>>>(
+    smallbatch_finish_kernel<0><<<finish_grid(M, l->N), 64, 0, s>>>(
         p.layer[0].part, nullptr, pl.NSG, (int)M, (int)l->N, static_cast<const f16 *>(l->bias), ep.row_scale,
         ep.accumulate, y);
     return launch_status();
@@ -523,23 +639,27 @@ int launch_smallbatch_gate_up(const hqq_linear *w1, const hqq_linear *w3, const 
     if (!make_plan(w1, M, pl) || !make_plan(w3, M, pl3) || w1->N != w3->N || w1->K != w3->K ||
         w1->nbits != w3->nbits || w1->group_size != w3->group_size)
         return HQQ_E_UNSUPPORTED;
-    const size_t one = smallbatch_workspace_bytes(w1, M);
+    // the gate needs both projections of an output, which different blocks compute: always via partial sums
+    const size_t one = (size_t)pl.NSG * (size_t)M * (size_t)w1->N * sizeof(float);
     if (ws_bytes < 2 * one)
         return HQQ_E_WORKSPACE;
     SBParams p = {};
     fill_params(p, pl, w1, 0, static_cast<float *>(ws));
     fill_params(p, pl, w3, 1, reinterpret_cast<float *>(static_cast<char *>(ws) + one));
     p.x = x, p.M = (int)M;
-    const dim3 grid((unsigned)(pl.GP * (pl.RB / pl.WR) * pl.NSG), 2);
+    p.NSG = pl.NSG;
+    p.force_partial = 1;
+    SBEpilogue e = {nullptr, nullptr, nullptr, 0};
+    const dim3 grid((unsigned)pl.NSG, (unsigned)(2 * (pl.RB / pl.WR)), (unsigned)pl.GP);
     if (w1->nbits == 2)
-        launch_main<2>(p, pl.MT, grid, s);
+        launch_main<2>(p, e, pl, grid, s);
     else
-        launch_main<4>(p, pl.MT, grid, s);
+        launch_main<4>(p, e, pl, grid, s);
     int rc = launch_status();
     if (rc != HQQ_OK)
         return rc;
-    smallbatch_finish_kernel<1><<<finish_grid(M, w1->N), 256, 0, s>>>(p.layer[0].part, p.layer[1].part, pl.NSG,
-                                                                       (int)M, (int)w1->N, nullptr, nullptr, 0, h);
+    smallbatch_finish_kernel<1><<<finish_grid(M, w1->N), 64, 0, s>>>(p.layer[0].part, p.layer[1].part, pl.NSG, (int)M,
+                                                                      (int)w1->N, nullptr, nullptr, 0, h);
     return launch_status();
 }
 
