@@ -1,0 +1,179 @@
+#!/usr/bin/env python3
+"""Headline benchmark: HQQ dequant-GEMV throughput on one MI355X.
+
+A "step" is one pass of the hot path over one batch of synthetic input: the
+2-bit expert FFN of Mixtral-8x7B at batch 1 (w1, w3: 14336x4096, w2: 4096x14336,
+group 16, 8-bit meta-quantised scale/zero), y = w2(silu(w1 x) * w3 x).  Steps
+rotate over several distinct experts (more than the 256 MB Infinity Cache holds)
+so that every weight byte really comes from HBM.  Inputs are resident in HBM
+before the timed region.
+
+Prints ONE JSON line.  ``value`` is algorithmic bytes per step / time per step.
+``roofline`` is the dominant kernel alone (the fused w1/w3 pass), timed with HIP
+events on the stream it is launched on.  ``cpu_baseline`` times the reference's
+PyTorch dequantise-then-matmul path (restated in oracle/torch_path.py) on the
+host cores for a bounded sample of the same steps."""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "mixtral-offloading_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HIDDEN, FFN = 4096, 14336
+NBITS, GROUP, META_GROUP = 2, 16, 128
+HBM_PEAK_GBS = 8000.0
+
+
+def layer_bytes(n, k):
+    s_cnt = n * k // GROUP
+    return n * k * NBITS // 8 + 2 * s_cnt + 2 * 2 * (s_cnt // META_GROUP) + 4
+
+
+def ffn_step_bytes(m):
+    """Algorithmic bytes of one expert FFN: weight-side bytes of the three layers plus fp16 activations in and out."""
+    weights = 2 * layer_bytes(FFN, HIDDEN) + layer_bytes(HIDDEN, FFN)
+    acts = 2 * m * HIDDEN + 2 * m * FFN + 2 * m * FFN + 2 * m * HIDDEN  # x, h written, h read, y
+    return weights + acts
+
+
+def gate_up_bytes(m):
+    return 2 * layer_bytes(FFN, HIDDEN) + 2 * m * HIDDEN + 2 * m * FFN
+
+
+def make_expert(seed, device):
+    """Random-init expert, quantised on the GPU by the package's own HQQ quantiser (W ~ N(0, 0.02))."""
+    import torch
+    from torch import nn
+
+    from mixtral_offloading_amd.custom_layers import HQQLinearTritonSavable
+    from mixtral_offloading_amd.hqq_core import BaseQuantizeConfig
+
+    cfg = BaseQuantizeConfig(nbits=NBITS, group_size=GROUP, quant_zero=True, quant_scale=True)
+    cfg["weight_quant_params"]["optimize"] = False  # min/max quantisation: the speed of the path does not depend on it
+    g = torch.Generator(device=device).manual_seed(seed)
+    layers = []
+    for n, k in ((FFN, HIDDEN), (HIDDEN, FFN), (FFN, HIDDEN)):
+        lin = nn.Linear(k, n, bias=False, device=device, dtype=torch.float16)
+        lin.weight.data = (torch.randn((n, k), device=device, generator=g) * 0.02).half()
+        layers.append(HQQLinearTritonSavable(lin, cfg))
+        del lin
+    return layers
+
+
+def cpu_baseline(budget_s=15.0):
+    import torch
+
+    from oracle import torch_path as tp
+
+    gen = torch.Generator().manual_seed(0)
+    w1 = tp.random_layer(gen, FFN, HIDDEN, NBITS, GROUP, META_GROUP)
+    w2 = tp.random_layer(gen, HIDDEN, FFN, NBITS, GROUP, META_GROUP)
+    w3 = tp.random_layer(gen, FFN, HIDDEN, NBITS, GROUP, META_GROUP)
+    x = torch.randn((1, HIDDEN), generator=gen).half()
+    with torch.inference_mode():
+        tp.expert_ffn(x, w1, w2, w3)  # warm up
+        t0 = time.perf_counter()
+        n = 0
+        while n < 3 or (time.perf_counter() - t0 < budget_s and n < 200):
+            tp.expert_ffn(x, w1, w2, w3)
+            n += 1
+        dt = (time.perf_counter() - t0) / n
+    return {"value": round(ffn_step_bytes(1) / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port", "ms_per_step": round(dt * 1e3, 2),
+            "sample": f"{n} steps of the same batch-1 2-bit expert FFN (one expert, host-resident), torch CPU half ops, "
+                      f"meta expansion + dequantize + matmul per call as the reference does"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--batch", type=int, default=1, help="tokens per step (1 is the headline; 4 and 16 are parity-test sizes)")
+    ap.add_argument("--experts", type=int, default=8, help="distinct experts the steps rotate over")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build runs on a single MI355X (--gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from mixtral_offloading_amd import _lib, hip_kernels
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    m = args.batch
+    experts = [make_expert(i, dev) for i in range(args.experts)]
+    descs = [(e[0]._desc(), e[1]._desc(), e[2]._desc()) for e in experts]
+    gx = torch.Generator(device=dev).manual_seed(1234)
+    x = torch.randn((m, HIDDEN), device=dev, generator=gx).half()
+    y = torch.empty((m, HIDDEN), device=dev, dtype=torch.float16)
+    h = torch.empty((m, FFN), device=dev, dtype=torch.float16)
+    lib = _lib.lib
+    need = lib.hqq_expert_ffn_workspace_bytes(descs[0][0].ref, descs[0][1].ref, descs[0][2].ref, m)
+    ws = torch.empty(max(int(need), 256), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.Stream(device=dev)
+    sp = stream.cuda_stream
+
+    def ffn_step(i):
+        w1, w2, w3 = descs[i % len(descs)]
+        rc = lib.hqq_expert_ffn(w1.ref, w2.ref, w3.ref, x.data_ptr(), m, y.data_ptr(), None, 0, ws.data_ptr(),
+                                ws.numel(), sp)
+        if rc != 0:
+            raise _lib.HqqError(rc, "hqq_expert_ffn")
+
+    def gate_up_step(i):
+        w1, _, w3 = descs[i % len(descs)]
+        rc = lib.hqq_gate_up(w1.ref, w3.ref, x.data_ptr(), m, h.data_ptr(), ws.data_ptr(), ws.numel(), sp)
+        if rc != 0:
+            raise _lib.HqqError(rc, "hqq_gate_up")
+
+    def timed(fn, warmup, steps):
+        with torch.cuda.stream(stream):
+            for i in range(warmup):
+                fn(i)
+            torch.cuda.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for i in range(steps):
+                fn(warmup + i)
+            e1.record(stream)
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps  # ms per step
+
+    ms_step = timed(ffn_step, args.warmup, args.steps)
+    ms_gate = timed(gate_up_step, args.warmup, args.steps)
+
+    value = ffn_step_bytes(m) / (ms_step * 1e-3) / 1e9
+    achieved = gate_up_bytes(m) / (ms_gate * 1e-3) / 1e9
+    out = {
+        "metric": "dequant-GEMV HBM GB/s (% of peak); Mixtral-8x7B mixed-quant decode tok/s",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"configs[1]: 2-bit g16 expert FFN GEMV at Mixtral shapes (w1,w3 14336x4096, w2 4096x14336), "
+                               f"batch {m}, 8-bit meta-quantised scale/zero (meta group 128), rotating over "
+                               f"{args.experts} experts ({args.experts * 66.4:.0f} MB of weights)",
+                   "bytes_per_step": ffn_step_bytes(m), "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "smallbatch_kernel<2,1,16,4,1> as launched by hqq_gate_up (w1 and w3 in one grid)",
+                     "bytes_per_launch": gate_up_bytes(m), "us_per_launch": round(ms_gate * 1e3, 3)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

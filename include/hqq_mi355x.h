@@ -114,6 +114,11 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
                    void *y_f16, const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
                    void *stream);
 
+/* ---- h = silu(w1 x) * (w3 x), fp16 (M, ffn): the first half of the expert FFN as one fused pass over both weight
+ *      matrices (src/custom_layers.py:254).  Workspace: 2 * hqq_matmul_workspace_bytes(w1, M).                        */
+int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, int64_t M, void *h_f16, void *workspace,
+                size_t workspace_bytes, void *stream);
+
 /* ---- which kernel family a call would use (for tests and profiles): 0 general, 1 MFMA small-batch, 2 MFMA tile,
  *      3 three-bit vector kernel.                                                                                     */
 int hqq_matmul_kernel_family(const hqq_linear *l, int64_t M);

@@ -170,6 +170,27 @@ size_t hqq_expert_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2
     return 3 * align256((size_t)M * w1->N * 2) + align256((size_t)M * w2->N * 2) + mm;
 }
 
+int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, int64_t M, void *h_f16, void *workspace,
+                size_t workspace_bytes, void *stream)
+{
+    int rc;
+    if ((rc = validate_linear(w1)) != HQQ_OK || (rc = validate_linear(w3)) != HQQ_OK)
+        return rc;
+    if (M < 0 || w1->N != w3->N || w1->K != w3->K)
+        return HQQ_E_SHAPE;
+    if (M == 0)
+        return HQQ_OK;
+    if (!x_f16 || !h_f16)
+        return HQQ_E_NULL;
+    if (!smallbatch_supported(w1, M) || !smallbatch_supported(w3, M) || w1->bias || w3->bias ||
+        w1->nbits != w3->nbits || w1->group_size != w3->group_size)
+        return HQQ_E_UNSUPPORTED;
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return HQQ_E_WORKSPACE;
+    return launch_smallbatch_gate_up(w1, w3, (const f16 *)x_f16, M, (f16 *)h_f16, workspace, workspace_bytes,
+                                     (hipStream_t)stream);
+}
+
 int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *x_f16, int64_t M,
                    void *y_f16, const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
                    void *stream)

@@ -1,0 +1,119 @@
+"""CPU-side tests: the C ABI library loads and exports every symbol the header declares, the host-only LRU policy
+agrees with the oracle model, and the torch restatement of the reference's PyTorch path agrees with the numpy oracle.
+No GPU compute is called here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import hqq_oracle as o
+from oracle import torch_path as tp
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    from mixtral_offloading_amd import _lib
+    header = open(os.path.join(ROOT, "include", "hqq_mi355x.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(hqq_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 25
+    for name in sorted(declared):
+        assert hasattr(_lib.lib, name), f"{name} is declared in include/hqq_mi355x.h but not exported"
+    assert declared == set(_lib.EXPORTED), (declared ^ set(_lib.EXPORTED))
+    assert _lib.lib.hqq_abi_version() == 1
+    assert b"NULL" in _lib.lib.hqq_error_string(-1)
+
+
+def test_argument_errors_without_touching_the_gpu():
+    from mixtral_offloading_amd import _lib
+    lin = _lib.HqqLinear()
+    assert _lib.lib.hqq_dequantize(ctypes.byref(lin), None, None) == -1  # NULL codes
+    lin.codes = 1 << 20
+    lin.nbits = 5
+    assert _lib.lib.hqq_matmul_kernel_family(ctypes.byref(lin), 1) == -2  # nbits
+    lin.nbits, lin.N, lin.K, lin.group_size = 4, 100, 64, 64
+    assert _lib.lib.hqq_matmul_kernel_family(ctypes.byref(lin), 1) == -3  # N % group_size
+    assert _lib.lib.hqq_pack_4bit_u8(1 << 20, 3, 4, 1 << 21, None) == -3  # odd height (reference src/packing.py:12)
+    assert _lib.lib.hqq_pack_4bit_u8(None, 2, 4, 1 << 21, None) == -1
+    assert _lib.lib.hqq_pack_4bit_u8(1 << 20, 0, 4, 1 << 21, None) == 0  # empty input
+
+
+def _plan(lib, c, experts):
+    n = len(experts)
+    arr = (ctypes.c_int32 * n)(*experts)
+    order, slot, victim = (ctypes.c_int32 * n)(), (ctypes.c_int32 * n)(), (ctypes.c_int32 * n)()
+    rc = lib.hqq_lru_plan(c, arr, n, order, slot, victim)
+    return rc, list(order), list(slot), list(victim)
+
+
+def test_lru_policy_against_the_oracle_model():
+    from mixtral_offloading_amd import _lib
+    lib = _lib.lib
+    rng = np.random.default_rng(0)
+    for slots in (2, 4):
+        c = lib.hqq_lru_create(8, slots)
+        resident = list(range(8 - slots, 8))  # build_model keeps experts >= offload_per_layer on the device
+        for e in resident:
+            assert lib.hqq_lru_add_resident(c, e) >= 0
+        assert lib.hqq_lru_add_resident(c, 0) == -7  # "Cache is full"
+        model = o.LruModel(resident, [e for e in range(8) if e not in resident])
+        slot_of = {e: lib.hqq_lru_slot_of(c, e) for e in resident}
+        for _ in range(300):
+            req = rng.choice(8, size=2, replace=False).tolist()
+            rc, order, slot, victim = _plan(lib, c, req)
+            assert rc == 0
+            m_order, m_ev = model.load(req)
+            assert order == m_order
+            assert [(e, v) for e, v in zip(order, victim) if v >= 0] == m_ev
+            for e, s, v in zip(order, slot, victim):
+                if v >= 0:
+                    assert slot_of.pop(v) == s  # the miss takes over its victim's slot
+                    slot_of[e] = s
+                else:
+                    assert slot_of[e] == s
+            assert sorted(slot_of) == sorted(model.main)
+            assert lib.hqq_lru_hits(c) == model.hits and lib.hqq_lru_misses(c) == model.misses
+        rc, *_ = _plan(lib, c, [1, 1])
+        assert rc == -7  # duplicates (reference src/expert_cache.py:133)
+        rc, *_ = _plan(lib, c, [9])
+        assert rc == -7  # unknown expert
+        lib.hqq_lru_destroy(c)
+
+
+def test_lru_hand_trace_through_the_c_abi():
+    from mixtral_offloading_amd import _lib
+    lib = _lib.lib
+    c = lib.hqq_lru_create(8, 4)
+    for e in (4, 5, 6, 7):
+        lib.hqq_lru_add_resident(c, e)
+    assert _plan(lib, c, [5, 0])[1:] == ([5, 0], [1, 0], [-1, 4])
+    assert _plan(lib, c, [1, 6])[1:] == ([6, 1], [2, 3], [-1, 7])
+    assert _plan(lib, c, [2, 3])[1:] == ([2, 3], [1, 0], [5, 0])
+    assert (lib.hqq_lru_hits(c), lib.hqq_lru_misses(c)) == (2, 4)
+    lib.hqq_lru_destroy(c)
+
+
+@pytest.mark.parametrize("nbits,n,k,gs,mgs", [(4, 64, 32, 16, 8), (2, 64, 32, 16, 8), (3, 40, 16, 8, 16)])
+def test_torch_path_matches_numpy_oracle(nbits, n, k, gs, mgs):
+    rng = np.random.default_rng(nbits)
+    layer, _ = o.random_layer(rng, n, k, nbits, gs, meta_group_size=mgs)
+    tl = tp.layer_from_numpy(layer)
+    w = tp.dequantize(tl).numpy()
+    np.testing.assert_array_equal(w.view(np.uint16), o.dequantize(layer).view(np.uint16))
+    x = rng.standard_normal((3, k)).astype(np.float16)
+    y = tp.forward(torch.from_numpy(x), tl).numpy().astype(np.float64)
+    ref = o.matmul_transpose(x, layer).astype(np.float64)
+    assert np.abs(y - ref).max() <= 1e-2 * np.abs(ref).max() + 1e-3
+
+
+def test_torch_path_random_layer_is_in_kernel_layout():
+    g = torch.Generator().manual_seed(0)
+    for nbits, n in ((2, 32), (4, 32), (3, 24)):
+        layer = tp.random_layer(g, n, 128, nbits, 8, 8)
+        u = tp.unpack(layer["W_q"], nbits)[:n]
+        assert int(u.max()) < 2 ** nbits
+        np.testing.assert_array_equal(o.PACK[nbits](u.numpy()), layer["W_q"].numpy())
