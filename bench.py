@@ -120,7 +120,7 @@ def main():
     h = torch.empty((m, FFN), device=dev, dtype=torch.float16)
     lib = _lib.lib
     need = lib.hqq_expert_ffn_workspace_bytes(descs[0][0].ref, descs[0][1].ref, descs[0][2].ref, m)
-    ws = torch.empty(max(int(need), 256), dtype=torch.uint8, device=dev)
+    ws = torch.zeros(max(int(need), 256), dtype=torch.uint8, device=dev)  # counters in its head start at zero
     stream = torch.cuda.Stream(device=dev)
     sp = stream.cuda_stream
 

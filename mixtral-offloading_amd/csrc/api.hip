@@ -122,6 +122,15 @@ size_t hqq_matmul_workspace_bytes(const hqq_linear *l, int64_t M)
     return align256(a > b ? a : b);
 }
 
+int hqq_workspace_init(void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!workspace)
+        return HQQ_E_NULL;
+    if (reinterpret_cast<uintptr_t>(workspace) & 255u)
+        return HQQ_E_WORKSPACE;
+    return launch_zero_workspace_head(workspace, workspace_bytes, (hipStream_t)stream);
+}
+
 int hqq_matmul_transpose_ex(const hqq_linear *l, const void *x_f16, int64_t M, void *y_f16, void *workspace,
                             size_t workspace_bytes, int family, void *stream)
 {
@@ -155,19 +164,24 @@ int hqq_matmul_transpose(const hqq_linear *l, const void *x_f16, int64_t M, void
     return hqq_matmul_transpose_ex(l, x_f16, M, y_f16, workspace, workspace_bytes, -1, stream);
 }
 
-// workspace of the FFN: [h: M x ffn fp16][t: M x hidden fp16][a, b: M x ffn fp16 each (unfused path)][matmul scratch]
-size_t hqq_expert_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, int64_t M)
+// workspace of the FFN: [matmul scratch, counters first][h: M x ffn fp16][t: M x hidden fp16][a, b: M x ffn fp16
+// each (unfused path only)]
+static size_t ffn_matmul_scratch(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, int64_t M)
 {
-    if (validate_linear(w1) != HQQ_OK || validate_linear(w2) != HQQ_OK || validate_linear(w3) != HQQ_OK || M <= 0)
-        return 0;
-    size_t mm = hqq_matmul_workspace_bytes(w1, M);
-    size_t m2 = hqq_matmul_workspace_bytes(w2, M);
-    size_t m3 = 2 * hqq_matmul_workspace_bytes(w3, M); // fused gate/up pass keeps two sets of partial sums
+    size_t mm = hqq_matmul_workspace_bytes(w1, M); // already sized for the fused gate pass over two layers
+    const size_t m2 = hqq_matmul_workspace_bytes(w2, M), m3 = hqq_matmul_workspace_bytes(w3, M);
     if (m2 > mm)
         mm = m2;
     if (m3 > mm)
         mm = m3;
-    return 3 * align256((size_t)M * w1->N * 2) + align256((size_t)M * w2->N * 2) + mm;
+    return align256(mm);
+}
+
+size_t hqq_expert_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, int64_t M)
+{
+    if (validate_linear(w1) != HQQ_OK || validate_linear(w2) != HQQ_OK || validate_linear(w3) != HQQ_OK || M <= 0)
+        return 0;
+    return ffn_matmul_scratch(w1, w2, w3, M) + 3 * align256((size_t)M * w1->N * 2) + align256((size_t)M * w2->N * 2);
 }
 
 int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, int64_t M, void *h_f16, void *workspace,
@@ -211,12 +225,12 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
     hipStream_t s = (hipStream_t)stream;
     char *p = static_cast<char *>(workspace);
     const size_t mid = align256((size_t)M * w1->N * 2), outb = align256((size_t)M * w2->N * 2);
-    f16 *h = (f16 *)p;
-    f16 *t = (f16 *)(p + mid);
-    f16 *a = (f16 *)(p + mid + outb);
-    f16 *b = (f16 *)(p + 2 * mid + outb);
-    void *mm = p + 3 * mid + outb;
-    const size_t mm_bytes = workspace_bytes - (3 * mid + outb);
+    const size_t mm_bytes = ffn_matmul_scratch(w1, w2, w3, M);
+    void *mm = p; // first, so that hqq_workspace_init finds the counters at the head of the workspace
+    f16 *h = (f16 *)(p + mm_bytes);
+    f16 *t = (f16 *)(p + mm_bytes + mid);
+    f16 *a = (f16 *)(p + mm_bytes + mid + outb);
+    f16 *b = (f16 *)(p + mm_bytes + 2 * mid + outb);
     const f16 *x = (const f16 *)x_f16;
     f16 *y = (f16 *)y_f16;
 

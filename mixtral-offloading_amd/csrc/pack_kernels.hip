@@ -218,12 +218,12 @@ inline int grid_for(int64_t total)
 template <int NBITS>
 int unpack_u8(const uint8_t *in, int64_t prows, int64_t cols, uint8_t *out, hipStream_t s)
 {
-    if (!in || !out)
-        return HQQ_E_NULL;
     if (prows < 0 || cols < 0)
         return HQQ_E_SHAPE;
-    if (prows == 0 || cols == 0)
+    if (prows == 0 || cols == 0) // empty input: nothing to do, and an empty tensor may well have no address
         return HQQ_OK;
+    if (!in || !out)
+        return HQQ_E_NULL;
     if (cols % 16 == 0 && aligned16(in) && aligned16(out))
         unpack_u8_kernel<NBITS, u32x4><<<grid_for(prows * cols / 16), kThreads, 0, s>>>(in, prows, cols, out);
     else
@@ -235,12 +235,12 @@ template <int NBITS>
 int pack_u8(const uint8_t *q, int64_t rows, int64_t cols, uint8_t *out, hipStream_t s)
 {
     constexpr int F = 8 / NBITS;
-    if (!q || !out)
-        return HQQ_E_NULL;
     if (rows < 0 || cols < 0 || rows % F != 0) // reference asserts an even height for 4 bit (src/packing.py:12)
         return HQQ_E_SHAPE;
     if (rows == 0 || cols == 0)
         return HQQ_OK;
+    if (!q || !out)
+        return HQQ_E_NULL;
     const int64_t prows = rows / F;
     if (cols % 16 == 0 && aligned16(q) && aligned16(out))
         pack_u8_kernel<NBITS, u32x4><<<grid_for(prows * cols / 16), kThreads, 0, s>>>(q, prows, cols, out);
@@ -293,12 +293,12 @@ int hqq_unpack_2bit_u8(const uint8_t *in, int64_t rows, int64_t cols, uint8_t *q
 
 int hqq_pack_3bit_i32(const uint8_t *q, int64_t rows, int64_t cols, int32_t *out, void *stream)
 {
-    if (!q || !out)
-        return HQQ_E_NULL;
     if (rows < 0 || cols < 0)
         return HQQ_E_SHAPE;
     if (rows == 0 || cols == 0)
         return HQQ_OK;
+    if (!q || !out)
+        return HQQ_E_NULL;
     const int64_t words = (rows + 9) / 10;
     hipStream_t s = (hipStream_t)stream;
     if (cols % 4 == 0 && aligned16(out) && (reinterpret_cast<uintptr_t>(q) & 3u) == 0)
@@ -310,12 +310,12 @@ int hqq_pack_3bit_i32(const uint8_t *q, int64_t rows, int64_t cols, int32_t *out
 
 int hqq_unpack_3bit_i32(const int32_t *in, int64_t rows, int64_t cols, uint8_t *q, void *stream)
 {
-    if (!in || !q)
-        return HQQ_E_NULL;
     if (rows < 0 || cols < 0)
         return HQQ_E_SHAPE;
     if (rows == 0 || cols == 0)
         return HQQ_OK;
+    if (!in || !q)
+        return HQQ_E_NULL;
     hipStream_t s = (hipStream_t)stream;
     if (cols % 4 == 0 && aligned16(in) && (reinterpret_cast<uintptr_t>(q) & 3u) == 0)
         unpack3_kernel<4><<<grid_for(rows * cols / 4), kThreads, 0, s>>>((const uint32_t *)in, rows, cols, q);

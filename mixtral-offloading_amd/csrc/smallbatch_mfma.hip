@@ -581,15 +581,18 @@ int finish_grid(int64_t M, int64_t N)
 bool smallbatch_supported(const hqq_linear *l, int64_t M)
 {
     SBPlan pl;
-    return make_plan(l, M, pl);
+    return slab_supported(l, M) || make_plan(l, M, pl);
 }
 
+// the first workspace_head_bytes() of a workspace belong to the slab kernel's arrival counters
 size_t smallbatch_workspace_bytes(const hqq_linear *l, int64_t M)
 {
+    if (slab_supported(l, M))
+        return slab_workspace_bytes(l, M);
     SBPlan pl;
     if (!make_plan(l, M, pl))
         return 0;
-    return (size_t)pl.NSG * (size_t)M * (size_t)l->N * sizeof(float);
+    return workspace_head_bytes() + (size_t)pl.NSG * (size_t)M * (size_t)l->N * sizeof(float);
 }
 
 static void fill_params(SBParams &p, const SBPlan &pl, const hqq_linear *l, int which, float *part)
@@ -607,13 +610,15 @@ static void fill_params(SBParams &p, const SBPlan &pl, const hqq_linear *l, int 
 int launch_smallbatch_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
                              const SmallBatchEpilogue &ep, hipStream_t s)
 {
+    if (slab_supported(l, M))
+        return launch_slab_matmul(l, x, M, y, ws, ws_bytes, ep, s);
     SBPlan pl;
     if (!make_plan(l, M, pl))
         return HQQ_E_UNSUPPORTED;
     if (pl.NSG > 1 && ws_bytes < smallbatch_workspace_bytes(l, M))
         return HQQ_E_WORKSPACE;
     SBParams p = {};
-    fill_params(p, pl, l, 0, static_cast<float *>(ws));
+    fill_params(p, pl, l, 0, reinterpret_cast<float *>(static_cast<char *>(ws) + workspace_head_bytes()));
     p.layer[1] = p.layer[0];
     p.x = x, p.M = (int)M;
     p.probe = env_int("HQQ_SB_PROBE", 0);
@@ -635,17 +640,20 @@ int launch_smallbatch_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *
 int launch_smallbatch_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
                               size_t ws_bytes, hipStream_t s)
 {
+    if (slab_supported(w1, M) && slab_supported(w3, M))
+        return launch_slab_gate_up(w1, w3, x, M, h, ws, ws_bytes, s);
     SBPlan pl, pl3;
     if (!make_plan(w1, M, pl) || !make_plan(w3, M, pl3) || w1->N != w3->N || w1->K != w3->K ||
         w1->nbits != w3->nbits || w1->group_size != w3->group_size)
         return HQQ_E_UNSUPPORTED;
     // the gate needs both projections of an output, which different blocks compute: always via partial sums
     const size_t one = (size_t)pl.NSG * (size_t)M * (size_t)w1->N * sizeof(float);
-    if (ws_bytes < 2 * one)
+    const size_t head = workspace_head_bytes();
+    if (ws_bytes < head + 2 * one)
         return HQQ_E_WORKSPACE;
     SBParams p = {};
-    fill_params(p, pl, w1, 0, static_cast<float *>(ws));
-    fill_params(p, pl, w3, 1, reinterpret_cast<float *>(static_cast<char *>(ws) + one));
+    fill_params(p, pl, w1, 0, reinterpret_cast<float *>(static_cast<char *>(ws) + head));
+    fill_params(p, pl, w3, 1, reinterpret_cast<float *>(static_cast<char *>(ws) + head + one));
     p.x = x, p.M = (int)M;
     p.NSG = pl.NSG;
     p.force_partial = 1;

@@ -45,6 +45,7 @@ _SIGNATURES = {
     "hqq_table_to_f16": (c_int, [_P(HqqTable), c_int64, c_void_p, c_void_p]),
     "hqq_dequantize": (c_int, [_P(HqqLinear), c_void_p, c_void_p]),
     "hqq_matmul_workspace_bytes": (c_size_t, [_P(HqqLinear), c_int64]),
+    "hqq_workspace_init": (c_int, [c_void_p, c_size_t, c_void_p]),
     "hqq_matmul_transpose": (c_int, [_P(HqqLinear), c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hqq_matmul_transpose_ex": (c_int, [_P(HqqLinear), c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "hqq_matmul_kernel_family": (c_int, [_P(HqqLinear), c_int64]),
