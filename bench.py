@@ -99,6 +99,9 @@ def main():
     ap.add_argument("--batch", type=int, default=1, help="tokens per step (1 is the headline; 4 and 16 are parity-test sizes)")
     ap.add_argument("--experts", type=int, default=8, help="distinct experts the steps rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run plain 256 MiB device copies, so that a counter run can scale FETCH_SIZE / WRITE_SIZE "
+                         "by what the same counters read for a copy of known size")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build runs on a single MI355X (--gpus 1)", file=sys.stderr)
@@ -153,6 +156,14 @@ def main():
 
     ms_step = timed(ffn_step, args.warmup, args.steps)
     ms_gate = timed(gate_up_step, args.warmup, args.steps)
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(f"calibration: 4 device copies of {src.numel()} bytes (reads {src.numel()}, writes {src.numel()} each)",
+              file=sys.stderr)
 
     value = ffn_step_bytes(m) / (ms_step * 1e-3) / 1e9
     achieved = gate_up_bytes(m) / (ms_gate * 1e-3) / 1e9
@@ -166,8 +177,11 @@ def main():
                                f"{args.experts} experts ({args.experts * 66.4:.0f} MB of weights)",
                    "bytes_per_step": ffn_step_bytes(m), "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "smallbatch_kernel<2,1,16,4,1> as launched by hqq_gate_up (w1 and w3 in one grid)",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this command, scaled by a
+                     # 256 MiB copy (profiles/gemv_slab_kernel_ffn_2bit_g16_m1.txt); measured at batch 1 only
+                     "traffic": 46793113 if m == 1 else None,
+                     "kernel": "gemv_slab_kernel<2,1,16,1,2,1> as launched by hqq_gate_up (w1 and w3 in one grid, one launch)",
                      "bytes_per_launch": gate_up_bytes(m), "us_per_launch": round(ms_gate * 1e3, 3)},
     }
     if not args.no_cpu_baseline:
