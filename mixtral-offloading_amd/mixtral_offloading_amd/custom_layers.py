@@ -214,3 +214,51 @@ class MixtralBLockSparseTop2MLP_HQQ(nn.Module):
         y = hip_kernels.expert_ffn(self.w1._desc(), self.w2._desc(), self.w3._desc(), x, out=out,
                                    row_scale=row_scale, accumulate=accumulate)
         return y.view(hidden_states.shape[:-1] + (y.shape[-1],)) if out is None else out
+
+
+class SparseMoeWrapper(nn.Module):
+    """Router + expert dispatch over an ``ExpertCache`` (reference src/custom_layers.py:259-314).
+
+    Returns ``(hidden_states, router_logits)`` like the reference.  Each expert's FFN runs as the fused library
+    call with the routing weight and the accumulation into the output folded in (reference :307-312 gathers,
+    multiplies and ``index_add_``s with separate kernels)."""
+
+    def __init__(self, config, layer_id, gate, expert_cache):
+        super().__init__()
+        self.hidden_dim = config.hidden_size
+        self.ffn_dim = config.intermediate_size
+        self.num_experts = config.num_local_experts
+        self.top_k = config.num_experts_per_tok
+        self.layer_id = layer_id
+        self.gate = gate
+        self.experts = expert_cache
+
+    @torch.inference_mode()
+    def forward(self, hidden_states: torch.Tensor):
+        batch_size, sequence_length, hidden_dim = hidden_states.shape
+        hidden_states = hidden_states.reshape(-1, hidden_dim)
+        router_logits = self.gate(hidden_states)  # (tokens, n_experts)
+        routing_weights = F.softmax(router_logits, dim=1, dtype=torch.float)
+        routing_weights, selected_experts = torch.topk(routing_weights, self.top_k, dim=-1)
+        routing_weights /= routing_weights.sum(dim=-1, keepdim=True)
+        routing_weights = routing_weights.to(hidden_states.dtype)
+
+        tokens = hidden_states.shape[0]
+        final_hidden_states = torch.zeros((tokens, hidden_dim), dtype=hidden_states.dtype, device=hidden_states.device)
+        selected = selected_experts.tolist()  # one host sync per layer: the cache is driven from the host
+        active_experts = sorted({e for row in selected for e in row})
+
+        for (_layer_index, expert_idx), expert_layer in self.experts.load_experts(
+                *((self.layer_id, expert_idx) for expert_idx in active_experts), unordered=True):
+            if tokens == 1:
+                k = selected[0].index(expert_idx)
+                expert_layer(hidden_states, out=final_hidden_states, row_scale=routing_weights[0, k:k + 1],
+                             accumulate=True)
+                continue
+            rows = [(t, row.index(expert_idx)) for t, row in enumerate(selected) if expert_idx in row]
+            top_x = torch.tensor([t for t, _ in rows], device=hidden_states.device)
+            idx = torch.tensor([k for _, k in rows], device=hidden_states.device)
+            current_state = hidden_states.index_select(0, top_x)
+            current_hidden_states = expert_layer(current_state, row_scale=routing_weights[top_x, idx])
+            final_hidden_states.index_add_(0, top_x, current_hidden_states.to(hidden_states.dtype))
+        return final_hidden_states.reshape(batch_size, sequence_length, hidden_dim), router_logits

@@ -1,0 +1,159 @@
+"""Minimal Mixtral decoder used as the harness around the quantized-linear hot path.
+
+The reference builds on HF ``MixtralForCausalLM`` (transformers 4.36.1,
+``src/build_model.py:182-190``); this is the same architecture written with plain
+torch ops -- RMSNorm, rotary embedding (theta 1e6), grouped-query attention with a
+KV cache, sparse top-2 MoE -- with the same module names (``model.layers[i].self_attn.q_proj``,
+``.block_sparse_moe.gate`` ...) so that ``replace_attn_layers`` and ``build_model``
+read like the reference.  The four attention projections and the expert FFNs are the
+HIP library's kernels; everything else here is plumbing, not the measured path."""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+from torch import nn
+from torch.nn import functional as F
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, hidden_size, eps=1e-5, device=None):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(hidden_size, dtype=torch.float16, device=device), requires_grad=False)
+        self.variance_epsilon = eps
+
+    def forward(self, x):
+        xf = x.float()
+        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
+        return self.weight * xf.to(x.dtype)
+
+
+class Rotary:
+    def __init__(self, head_dim, max_positions, theta, device):
+        inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32, device=device) / head_dim))
+        t = torch.arange(max_positions, dtype=torch.float32, device=device)
+        freqs = torch.outer(t, inv_freq)
+        emb = torch.cat((freqs, freqs), dim=-1)
+        self.cos, self.sin = emb.cos().half(), emb.sin().half()
+
+    @staticmethod
+    def rotate_half(x):
+        h = x.shape[-1] // 2
+        return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
+
+    def apply(self, q, k, positions):
+        cos, sin = self.cos[positions][:, None, :], self.sin[positions][:, None, :]  # (T, 1, hd)
+        return q * cos + self.rotate_half(q) * sin, k * cos + self.rotate_half(k) * sin
+
+
+class Attention(nn.Module):
+    def __init__(self, config, device):
+        super().__init__()
+        self.num_heads = config.num_attention_heads
+        self.num_kv_heads = config.num_key_value_heads
+        self.head_dim = config.hidden_size // config.num_attention_heads
+        hs = config.hidden_size
+        mk = dict(bias=False, dtype=torch.float16, device=device)
+        # fp16 placeholders; replace_attn_layers swaps in the quantized linears
+        self.q_proj = nn.Linear(hs, self.num_heads * self.head_dim, **mk)
+        self.k_proj = nn.Linear(hs, self.num_kv_heads * self.head_dim, **mk)
+        self.v_proj = nn.Linear(hs, self.num_kv_heads * self.head_dim, **mk)
+        self.o_proj = nn.Linear(self.num_heads * self.head_dim, hs, **mk)
+
+    def forward(self, x, rotary: Rotary, cache_k, cache_v, start: int):
+        """x (T, hidden) for one sequence; cache_k / cache_v (kv_heads, max_len, hd); start = tokens already cached."""
+        T = x.shape[0]
+        q = self.q_proj(x).view(T, self.num_heads, self.head_dim)
+        k = self.k_proj(x).view(T, self.num_kv_heads, self.head_dim)
+        v = self.v_proj(x).view(T, self.num_kv_heads, self.head_dim)
+        positions = torch.arange(start, start + T, device=x.device)
+        q, k = rotary.apply(q, k, positions)
+        cache_k[:, start:start + T] = k.transpose(0, 1)
+        cache_v[:, start:start + T] = v.transpose(0, 1)
+        keys, values = cache_k[:, :start + T], cache_v[:, :start + T]  # (kv, L, hd)
+        g = self.num_heads // self.num_kv_heads
+        qh = q.transpose(0, 1).reshape(self.num_kv_heads, g * T, self.head_dim)  # heads of a kv group, then tokens
+        scores = torch.bmm(qh, keys.transpose(1, 2)).float() / math.sqrt(self.head_dim)  # (kv, g*T, L)
+        if T > 1:
+            tok = torch.arange(T, device=x.device).repeat(g)  # row -> token index
+            allowed = torch.arange(start + T, device=x.device)[None, :] <= (start + tok)[:, None]
+            scores = scores.masked_fill(~allowed[None], float("-inf"))
+        probs = torch.softmax(scores, dim=-1).to(x.dtype)
+        out = torch.bmm(probs, values)  # (kv, g*T, hd)
+        out = out.view(self.num_kv_heads, g, T, self.head_dim).permute(2, 0, 1, 3).reshape(T, -1)
+        return self.o_proj(out)
+
+
+class MoePlaceholder(nn.Module):
+    """Holds the router until build_model installs the SparseMoeWrapper (reference src/build_model.py:212-217)."""
+
+    def __init__(self, config, device):
+        super().__init__()
+        self.gate = nn.Linear(config.hidden_size, config.num_local_experts, bias=False, dtype=torch.float16,
+                              device=device)
+
+
+class DecoderLayer(nn.Module):
+    def __init__(self, config, device):
+        super().__init__()
+        self.input_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps, device)
+        self.self_attn = Attention(config, device)
+        self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps, device)
+        self.block_sparse_moe = MoePlaceholder(config, device)
+
+    def forward(self, x, rotary, cache_k, cache_v, start):
+        x = x + self.self_attn(self.input_layernorm(x), rotary, cache_k, cache_v, start)
+        moe_out, _ = self.block_sparse_moe(self.post_attention_layernorm(x)[None])
+        return x + moe_out[0]
+
+
+class MixtralModel(nn.Module):
+    def __init__(self, config, device):
+        super().__init__()
+        self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size, dtype=torch.float16, device=device)
+        self.layers = nn.ModuleList([DecoderLayer(config, device) for _ in range(config.num_hidden_layers)])
+        self.norm = RMSNorm(config.hidden_size, config.rms_norm_eps, device)
+
+
+class MixtralForCausalLM(nn.Module):
+    def __init__(self, config, device, max_positions: int = 4096):
+        super().__init__()
+        self.config = config
+        self.model = MixtralModel(config, device)
+        self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False, dtype=torch.float16, device=device)
+        head_dim = config.hidden_size // config.num_attention_heads
+        self.rotary = Rotary(head_dim, max_positions, config.rope_theta, device)
+        self.max_positions = max_positions
+        self.device = device
+
+    def new_cache(self, max_len: Optional[int] = None):
+        cfg = self.config
+        hd = cfg.hidden_size // cfg.num_attention_heads
+        L = max_len or self.max_positions
+        mk = dict(dtype=torch.float16, device=self.device)
+        return [(torch.zeros((cfg.num_key_value_heads, L, hd), **mk), torch.zeros((cfg.num_key_value_heads, L, hd), **mk))
+                for _ in range(cfg.num_hidden_layers)]
+
+    @torch.inference_mode()
+    def forward(self, input_ids: torch.Tensor, cache, start: int) -> torch.Tensor:
+        """input_ids (T,), one sequence; returns logits (T, vocab)."""
+        x = self.model.embed_tokens(input_ids)
+        for layer, (ck, cv) in zip(self.model.layers, cache):
+            x = layer(x, self.rotary, ck, cv, start)
+        return self.lm_head(self.model.norm(x))
+
+    @torch.inference_mode()
+    def generate(self, prompt_ids: torch.Tensor, max_new_tokens: int, cache=None):
+        """Greedy decoding, batch 1; returns the generated ids (max_new_tokens,)."""
+        cache = cache or self.new_cache(prompt_ids.numel() + max_new_tokens)
+        logits = self.forward(prompt_ids, cache, 0)
+        tok = logits[-1].argmax()
+        out = [tok]
+        pos = prompt_ids.numel()
+        for _ in range(max_new_tokens - 1):
+            logits = self.forward(tok.view(1), cache, pos)
+            tok = logits[-1].argmax()
+            out.append(tok)
+            pos += 1
+        return torch.stack(out)

@@ -28,6 +28,9 @@ class PackedTensor(torch.Tensor):
     def __init__(self, t: torch.Tensor):
         pass
 
+    def __deepcopy__(self, memo):
+        return PackedTensor(torch.Tensor.as_subclass(self, torch.Tensor).clone())
+
     @classmethod
     def __torch_function__(cls, func, types, args=(), kwargs=None):
         # plain tensors come out of every op; only explicit construction tags
