@@ -40,6 +40,11 @@ int validate_linear(const hqq_linear *l)
 static inline size_t align256(size_t v) { return (v + 255u) & ~(size_t)255u; }
 
 enum { FAM_GENERAL = 0, FAM_SMALLBATCH = 1, FAM_TILE = 2, FAM_VEC3 = 3 };
+constexpr int64_t kSmallBatchMax = 16;
+
+// a batch wider than the small-batch kernels take, run as slices of 16 rows (the weights of the later slices come
+// from L2 / Infinity Cache); used where the tile kernel does not take the shape
+static bool sliced_supported(const hqq_linear *l, int64_t M) { return M > kSmallBatchMax && smallbatch_supported(l, kSmallBatchMax); }
 
 static int pick_family(const hqq_linear *l, int64_t M)
 {
@@ -49,13 +54,15 @@ static int pick_family(const hqq_linear *l, int64_t M)
         return FAM_VEC3;
     if (tile_supported(l, M))
         return FAM_TILE;
+    if (sliced_supported(l, M))
+        return FAM_SMALLBATCH;
     return FAM_GENERAL;
 }
 
 static size_t family_workspace(const hqq_linear *l, int64_t M, int fam)
 {
     if (fam == FAM_SMALLBATCH)
-        return smallbatch_workspace_bytes(l, M);
+        return smallbatch_workspace_bytes(l, M > kSmallBatchMax ? kSmallBatchMax : M);
     if (fam == FAM_VEC3)
         return vec3_workspace_bytes(l, M);
     return 0;
@@ -68,6 +75,15 @@ static int run_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void
         return HQQ_OK;
     switch (fam) {
     case FAM_SMALLBATCH:
+        if (M > kSmallBatchMax) {
+            for (int64_t m0 = 0; m0 < M; m0 += kSmallBatchMax) {
+                const int64_t mb = M - m0 < kSmallBatchMax ? M - m0 : kSmallBatchMax;
+                int rc = launch_smallbatch_matmul(l, x + m0 * l->K, mb, y + m0 * l->N, ws, ws_bytes, SmallBatchEpilogue{}, s);
+                if (rc != HQQ_OK)
+                    return rc;
+            }
+            return HQQ_OK;
+        }
         return launch_smallbatch_matmul(l, x, M, y, ws, ws_bytes, SmallBatchEpilogue{}, s);
     case FAM_VEC3:
         return launch_vec3_matmul(l, x, M, y, ws, ws_bytes, s);
@@ -117,7 +133,8 @@ size_t hqq_matmul_workspace_bytes(const hqq_linear *l, int64_t M)
     if (validate_linear(l) != HQQ_OK || M <= 0)
         return 0;
     // large enough for whichever family is chosen or forced
-    size_t a = smallbatch_supported(l, M) ? 2 * smallbatch_workspace_bytes(l, M) : 0;
+    const int64_t Ms = M > kSmallBatchMax ? kSmallBatchMax : M;
+    size_t a = smallbatch_supported(l, Ms) ? 2 * smallbatch_workspace_bytes(l, Ms) : 0;
     size_t b = vec3_supported(l, M) ? vec3_workspace_bytes(l, M) : 0;
     return align256(a > b ? a : b);
 }
@@ -144,7 +161,7 @@ int hqq_matmul_transpose_ex(const hqq_linear *l, const void *x_f16, int64_t M, v
     if (!x_f16 || !y_f16)
         return HQQ_E_NULL;
     int fam = family < 0 ? pick_family(l, M) : family;
-    if (fam == FAM_SMALLBATCH && !smallbatch_supported(l, M))
+    if (fam == FAM_SMALLBATCH && !smallbatch_supported(l, M) && !sliced_supported(l, M))
         return HQQ_E_UNSUPPORTED;
     if (fam == FAM_VEC3 && !vec3_supported(l, M))
         return HQQ_E_UNSUPPORTED;
@@ -248,7 +265,7 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
         if ((rc = launch_silu_mul(a, b, h, M * w1->N, s)) != HQQ_OK)
             return rc;
     }
-    if (smallbatch_supported(w2, M)) {
+    if (M <= kSmallBatchMax && smallbatch_supported(w2, M)) {
         SmallBatchEpilogue ep;
         ep.row_scale = (const f16 *)row_scale_f16;
         ep.accumulate = accumulate;

@@ -1,0 +1,272 @@
+// Multi-token (prefill) unpack-dequantise-matmul for 2- and 4-bit codes on the matrix cores.
+//
+// Above ~16 batch rows folding the scale into the activations costs more than it saves, so here the weights
+// themselves are rebuilt, bit-exactly as the reference does (w = fp16(fp16(q - z) * s)), and fed to
+// v_mfma_f32_16x16x32_f16 with fp32 accumulation.
+//
+// A block is four wavefronts; wave w owns the 16 x F output rows of one packed table row jp = 4*blockIdx.x + w
+// (rows n = F*(jp + r*GP) + i, r = 16*rb .. 16*rb+15: they share scale and zero), for BM batch columns, and
+// walks all of K in 64-column steps.  Per step
+//   * the block copies the x tile (BM x 64 fp16) to LDS once, in B-operand order, for all four waves;
+//   * each wave de-quantises its 8-bit (or fp16) scale / zero entries once (F x 64 of each) into LDS;
+//   * each lane builds its A operands in registers: 16 code bytes -> for every field i and each half of the
+//     step, eight exact fp16 weights (mask-and-insert into 2^e, subtract, subtract z, multiply s);
+//   * 2 * F * BM/16 MFMAs per wave.
+// Weight bytes come from HBM once; the x tile is re-read by N / (64*F) blocks, from L2.
+#include "hqq_common.hpp"
+#include "table_reader.hpp"
+
+namespace hqq {
+namespace {
+
+constexpr int kStepK = 64;
+constexpr int kWaves = 4;
+
+struct TileParams {
+    const uint8_t *codes;
+    Table sc, zr;
+    uint32_t sc_inv, zr_inv;
+    const f16 *x;
+    const f16 *bias;
+    f16 *y;
+    int M, N, K, GP, KT;
+};
+
+template <int NBITS> struct WField {
+    static constexpr int F = 8 / NBITS;
+    static constexpr int pos(int i) { return NBITS * (F - 1 - i); }
+    static constexpr uint32_t mask(int i) { return (((1u << NBITS) - 1u) * 0x00010001u) << pos(i); }
+    // the masked field OR-ed into the mantissa of 2^e (e = 10 - pos) reads as 2^e + q
+    static constexpr uint32_t expo(int i) { return (uint32_t)((10 - pos(i) + 15) << 10) * 0x00010001u; }
+    static constexpr float offset(int i) { return (float)(1 << (10 - pos(i))); }
+};
+
+template <int NBITS, int BM>
+__global__ __launch_bounds__(kWaves * 64) void gemm_tile_kernel(TileParams p)
+{
+    constexpr int F = 8 / NBITS;
+    constexpr int MB = BM / 16;
+    // x tile: [k block of 8 (8 per step)][batch column][8 halves in B-operand order]
+    __shared__ __attribute__((aligned(16))) f16 x_lds[8 * BM * 8];
+    // per wave: scale and zero of the step, entry ((i*2 + h)*4 + kg) of 8 halves, same order
+    __shared__ __attribute__((aligned(16))) f16 s_lds[kWaves][F * 2 * 4 * 8];
+    __shared__ __attribute__((aligned(16))) f16 z_lds[kWaves][F * 2 * 4 * 8];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int jp = blockIdx.x * kWaves + wave;
+    const int rb = blockIdx.y;
+    const int m0 = blockIdx.z * BM;
+    const int K = p.K;
+    const int rr = lane & 15, kg = lane >> 4;
+    const int ti = lane >> 4, kq = lane & 15;
+    const bool tlane = ti < F;
+
+    const uint32_t prow = (uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)p.GP;
+    const uint8_t *cptr = p.codes + (size_t)prow * K + 16 * kg;
+    TableCursor<0> sc, zr;
+    {
+        const uint32_t c0 = (uint32_t)(F * jp + (tlane ? ti : 0)) * (uint32_t)K + (uint32_t)(4 * kq);
+        sc.init(p.sc, c0, p.sc_inv);
+        zr.init(p.zr, c0, p.zr_inv);
+    }
+    // x tile copy: thread t moves chunks (column m, k block kb) = (c / 8, c % 8) for c = t, t + 256, ...
+    constexpr int XCHUNKS = BM * 8 / (kWaves * 64);
+
+    f32x4 acc[F][MB];
+#pragma unroll
+    for (int i = 0; i < F; ++i)
+#pragma unroll
+        for (int b = 0; b < MB; ++b)
+            acc[i][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    u32x4 cw_n = {0, 0, 0, 0};
+    TableRaw sraw_n, zraw_n;
+    u32x4 xr_n[XCHUNKS];
+    auto issue = [&](int s) {
+        const int k0 = s * kStepK;
+        cw_n = *reinterpret_cast<const u32x4 *>(cptr + k0);
+        if (tlane) {
+            sraw_n = table_load(sc);
+            zraw_n = table_load(zr);
+        }
+        sc.advance(kStepK);
+        zr.advance(kStepK);
+#pragma unroll
+        for (int c = 0; c < XCHUNKS; ++c) {
+            const int ch = threadIdx.x + c * kWaves * 64;
+            const int m = m0 + ch / 8, kb = ch % 8;
+            xr_n[c] = (u32x4){0, 0, 0, 0};
+            // k block kb = h*4 + kg holds the columns half h of lane group kg works on: 16*kg + 8*h .. +7
+            if (m < p.M)
+                xr_n[c] = *reinterpret_cast<const u32x4 *>(p.x + (size_t)m * K + k0 + 16 * (kb & 3) + 8 * (kb >> 2));
+        }
+    };
+    issue(0);
+
+    f16 *s_w = &s_lds[wave][(((ti * 2 + ((kq >> 1) & 1)) * 4 + (kq >> 2)) * 8) + 4 * (kq & 1)];
+    f16 *z_w = &z_lds[wave][(((ti * 2 + ((kq >> 1) & 1)) * 4 + (kq >> 2)) * 8) + 4 * (kq & 1)];
+
+    for (int s = 0; s < p.KT; ++s) {
+        const u32x4 cw = cw_n;
+        const TableRaw sraw = sraw_n, zraw = zraw_n;
+        u32x4 xr[XCHUNKS];
+#pragma unroll
+        for (int c = 0; c < XCHUNKS; ++c)
+            xr[c] = xr_n[c];
+        if (s + 1 < p.KT)
+            issue(s + 1);
+
+        __syncthreads(); // everyone is done reading the previous step's tiles
+#pragma unroll
+        for (int c = 0; c < XCHUNKS; ++c) {
+            const int ch = threadIdx.x + c * kWaves * 64;
+            const int m = ch / 8, kb = ch % 8;
+            // eight columns (0..7) stored in B-operand order (0,2,1,3,4,6,5,7)
+            const f16x8 v = __builtin_bit_cast(f16x8, xr[c]);
+            const f16x8 o = {v[0], v[2], v[1], v[3], v[4], v[6], v[5], v[7]};
+            *reinterpret_cast<f16x8 *>(&x_lds[(kb * BM + m) * 8]) = o;
+        }
+        if (tlane) {
+            f16x2 s01, s23, z01, z23;
+            table_decode(sc, sraw, s01, s23);
+            table_decode(zr, zraw, z01, z23);
+            *reinterpret_cast<f16x4 *>(s_w) = (f16x4){s01.x, s23.x, s01.y, s23.y};
+            *reinterpret_cast<f16x4 *>(z_w) = (f16x4){z01.x, z23.x, z01.y, z23.y};
+        }
+        __syncthreads();
+
+        const uint32_t d[4] = {cw.x, cw.y, cw.z, cw.w};
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t d0 = d[2 * h], d1 = d[2 * h + 1];
+            const uint32_t d0s = d0 >> 8, d1s = d1 >> 8;
+            f16x8 B[MB];
+#pragma unroll
+            for (int b = 0; b < MB; ++b)
+                B[b] = *reinterpret_cast<const f16x8 *>(&x_lds[(((h * 4 + kg) * BM) + b * 16 + (lane & 15)) * 8]);
+#pragma unroll
+            for (int i = 0; i < F; ++i) {
+                const f16x8 S = *reinterpret_cast<const f16x8 *>(&s_lds[wave][((i * 2 + h) * 4 + kg) * 8]);
+                const f16x8 Z = *reinterpret_cast<const f16x8 *>(&z_lds[wave][((i * 2 + h) * 4 + kg) * 8]);
+                const uint32_t mk = WField<NBITS>::mask(i), ex = WField<NBITS>::expo(i);
+                const f16 offv = (f16)WField<NBITS>::offset(i);
+                const f16x2 off = {offv, offv};
+                const uint32_t src[4] = {d0, d0s, d1, d1s};
+                f16x8 A;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const f16x2 q = as_f16x2((src[t] & mk) | ex) - off;          // exact code
+                    const f16x2 zz = {Z[2 * t], Z[2 * t + 1]}, ss = {S[2 * t], S[2 * t + 1]};
+                    const f16x2 w = (q - zz) * ss;                                // two fp16 roundings, as the reference
+                    A[2 * t] = w.x;
+                    A[2 * t + 1] = w.y;
+                }
+#pragma unroll
+                for (int b = 0; b < MB; ++b)
+                    acc[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B[b], acc[i][b], 0, 0, 0);
+            }
+        }
+    }
+
+    // D layout: column = batch column (lane & 15) of block b, rows r = 4*(lane>>4) + v
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+        const int m = m0 + b * 16 + (lane & 15);
+        if (m >= p.M)
+            continue;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int r = 16 * rb + 4 * kg + v;
+            const int64_t n = (int64_t)F * (jp + (int64_t)r * p.GP);
+            f16 o[F];
+#pragma unroll
+            for (int i = 0; i < F; ++i) {
+                o[i] = (f16)acc[i][b][v];
+                if (p.bias)
+                    o[i] = o[i] + p.bias[n + i];
+            }
+            f16 *dst = p.y + (int64_t)m * p.N + n;
+            if constexpr (F == 4)
+                *reinterpret_cast<f16x4 *>(dst) = (f16x4){o[0], o[1], o[2], o[3]};
+            else
+                *reinterpret_cast<f16x2 *>(dst) = (f16x2){o[0], o[1]};
+        }
+    }
+}
+
+struct TilePlan {
+    int F, GP, RB, KT, BM;
+};
+
+bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl)
+{
+    if ((l->nbits != 2 && l->nbits != 4) || M < 1)
+        return false;
+    const int F = 8 / l->nbits;
+    const int64_t G = l->N / l->group_size;
+    if (l->group_size % 16 != 0 || G % F != 0 || l->K % kStepK != 0 || l->N % 4 != 0 || (G / F) % kWaves != 0)
+        return false;
+    if (l->N * l->K / l->group_size >= (1ll << 31) || G / F > 65535 * (int64_t)kWaves || l->group_size / 16 > 65535)
+        return false;
+    if (!aligned16(l->codes))
+        return false;
+    for (const hqq_table *t : {&l->scale, &l->zero}) {
+        if (t->kind == HQQ_TABLE_U8) {
+            if (reinterpret_cast<uintptr_t>(t->data) & 3u)
+                return false;
+            if (t->meta_cols != 1 && (t->meta_cols % 4 != 0 || t->meta_cols < kStepK ||
+                                      (reinterpret_cast<uintptr_t>(t->meta_scale) & 7u) ||
+                                      (reinterpret_cast<uintptr_t>(t->meta_zero) & 7u)))
+                return false;
+        } else if (reinterpret_cast<uintptr_t>(t->data) & 7u) {
+            return false;
+        }
+    }
+    pl.F = F;
+    pl.GP = (int)(G / F);
+    pl.RB = l->group_size / 16;
+    pl.KT = (int)(l->K / kStepK);
+    // narrower batch tiles when there would otherwise be fewer blocks than compute units
+    const int64_t blocks64 = (int64_t)(pl.GP / kWaves) * pl.RB * ((M + 63) / 64);
+    pl.BM = (M <= 32 || blocks64 < 256) ? 32 : 64;
+    if ((M + pl.BM - 1) / pl.BM > 65535)
+        return false;
+    return true;
+}
+
+} // namespace
+
+bool tile_supported(const hqq_linear *l, int64_t M)
+{
+    TilePlan pl;
+    return M > 16 && make_plan(l, M, pl);
+}
+
+int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, hipStream_t s)
+{
+    TilePlan pl;
+    if (!make_plan(l, M, pl) || (reinterpret_cast<uintptr_t>(x) & 15u))
+        return HQQ_E_UNSUPPORTED;
+    TileParams p = {};
+    p.codes = static_cast<const uint8_t *>(l->codes);
+    p.sc = make_table(l->scale), p.zr = make_table(l->zero);
+    p.sc_inv = l->scale.meta_cols > 0 ? (uint32_t)(0xFFFFFFFFull / (uint64_t)l->scale.meta_cols) : 0;
+    p.zr_inv = l->zero.meta_cols > 0 ? (uint32_t)(0xFFFFFFFFull / (uint64_t)l->zero.meta_cols) : 0;
+    p.x = x, p.bias = static_cast<const f16 *>(l->bias), p.y = y;
+    p.M = (int)M, p.N = (int)l->N, p.K = (int)l->K, p.GP = pl.GP, p.KT = pl.KT;
+    const dim3 grid((unsigned)(pl.GP / kWaves), (unsigned)pl.RB, (unsigned)((M + pl.BM - 1) / pl.BM));
+    if (l->nbits == 2) {
+        if (pl.BM == 32)
+            gemm_tile_kernel<2, 32><<<grid, kWaves * 64, 0, s>>>(p);
+        else
+            gemm_tile_kernel<2, 64><<<grid, kWaves * 64, 0, s>>>(p);
+    } else {
+        if (pl.BM == 32)
+            gemm_tile_kernel<4, 32><<<grid, kWaves * 64, 0, s>>>(p);
+        else
+            gemm_tile_kernel<4, 64><<<grid, kWaves * 64, 0, s>>>(p);
+    }
+    return launch_status();
+}
+
+} // namespace hqq

@@ -24,6 +24,9 @@ SHAPES = [
     (3, 448, 256, 64, 128, True, True),
     (3, 40, 24, 8, 4, False, False),
     (3, 1280, 192, 64, 128, True, True),
+    (2, 1024, 1024, 16, 128, True, True),   # every tuned family takes these two (G/F a multiple of 4, K of 256)
+    (4, 512, 1024, 64, 128, True, True),
+    (4, 512, 512, 64, 128, False, False),
 ]
 BATCHES = [1, 2, 4, 8, 16, 17, 33, 128]
 
@@ -66,6 +69,9 @@ def test_matmul_forced_family(shape, family):
             assert e.code == -6  # HQQ_E_UNSUPPORTED is the only acceptable refusal
     if family == 0:
         assert ran == 4
+    if shape[1:3] in ((1024, 1024), (512, 1024), (512, 512)) and family in (1, 2):
+        # the tuned kernels must really have run here, not refused (the tile family only takes batches above 16)
+        assert ran >= (2 if family == 1 else 1)
 
 
 def test_bias_leading_dims_and_empty():
