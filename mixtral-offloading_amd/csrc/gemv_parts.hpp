@@ -1,0 +1,95 @@
+// Pieces shared by the decode GEMV kernels: table decoding (16 entries per lane, 128-bit loads), the in-place
+// "code as fp16 subnormal" fields and the 16-lane DPP sum.
+#pragma once
+
+#include "hqq_common.hpp"
+
+namespace hqq {
+namespace gemv {
+
+constexpr int kSlab = 256;           // columns per wave
+constexpr float kXsScale = 32.0f;    // xs = 32 * s * x keeps small activations out of the fp16 subnormal range
+constexpr size_t kCounterBytes = 64 * 1024; // head of the workspace: one arrival counter per tile
+
+enum { TK_U8_COLS = 1, TK_U8_SCALAR = 2, TK_F16 = 3 };
+
+__device__ __forceinline__ f16x2 as_h2(uint32_t v) { return __builtin_bit_cast(f16x2, v); }
+__device__ __forceinline__ uint32_t as_u32(f16x2 v) { return __builtin_bit_cast(uint32_t, v); }
+
+__device__ __forceinline__ float row16_sum(float v)
+{
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+    return v;
+}
+
+// 16 table entries of a lane, raw
+template <int KIND> struct Raw16 {
+    u32x4 q;       // 16 bytes (u8 kinds) / first 8 halves (fp16)
+    u32x4 q_hi;    // fp16 only: last 8 halves
+    u32x4 ms[2], mz[2]; // per-column meta, 16 halves each
+};
+
+template <int KIND>
+__device__ __forceinline__ void load16(Raw16<KIND> &r, const uint8_t *tab, const f16 *ms, const f16 *mz, uint32_t c,
+                                       uint32_t cm)
+{
+    if constexpr (KIND == TK_F16) {
+        const u32x4 *p = reinterpret_cast<const u32x4 *>(reinterpret_cast<const f16 *>(tab) + c);
+        r.q = p[0];
+        r.q_hi = p[1];
+    } else {
+        r.q = *reinterpret_cast<const u32x4 *>(tab + c);
+        if constexpr (KIND == TK_U8_COLS) {
+            const u32x4 *a = reinterpret_cast<const u32x4 *>(ms + cm);
+            const u32x4 *b = reinterpret_cast<const u32x4 *>(mz + cm);
+            r.ms[0] = a[0], r.ms[1] = a[1];
+            r.mz[0] = b[0], r.mz[1] = b[1];
+        }
+    }
+}
+
+// decode to 8 fp16 pairs: pair t holds columns (2t, 2t+1) of the lane's 16
+template <int KIND>
+__device__ __forceinline__ void decode16(const Raw16<KIND> &r, f16x2 ms_s, f16x2 mz_s, f16x2 (&out)[8])
+{
+    if constexpr (KIND == TK_F16) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            out[t] = as_h2(r.q[t]);
+            out[4 + t] = as_h2(r.q_hi[t]);
+        }
+    } else {
+        const f16x2 k1024 = {(f16)1024.0f, (f16)1024.0f};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            // bytes -> fp16 exactly: 0x6400 | b is 1024 + b
+            const f16x2 lo = as_h2(__builtin_amdgcn_perm(0x64646464u, r.q[w], 0x04010400u)) - k1024;
+            const f16x2 hi = as_h2(__builtin_amdgcn_perm(0x64646464u, r.q[w], 0x04030402u)) - k1024;
+            if constexpr (KIND == TK_U8_COLS) {
+                out[2 * w] = (lo - as_h2(r.mz[w >> 1][2 * (w & 1)])) * as_h2(r.ms[w >> 1][2 * (w & 1)]);
+                out[2 * w + 1] = (hi - as_h2(r.mz[w >> 1][2 * (w & 1) + 1])) * as_h2(r.ms[w >> 1][2 * (w & 1) + 1]);
+            } else {
+                out[2 * w] = (lo - mz_s) * ms_s;
+                out[2 * w + 1] = (hi - mz_s) * ms_s;
+            }
+        }
+    }
+}
+
+template <int NBITS> struct Field {
+    static constexpr int F = 8 / NBITS;
+    static constexpr int pos(int i) { return NBITS * (F - 1 - i); }
+    // field i of the byte in the low half of each 16-bit word; masked in place it is the fp16 subnormal
+    // q * 2^(pos - 24), which the matrix cores multiply exactly
+    static constexpr uint32_t mask(int i) { return (((1u << NBITS) - 1u) * 0x00010001u) << pos(i); }
+    static constexpr float unscale(int i) { return (float)(1u << (24 - pos(i))) / kXsScale; }
+};
+
+
+inline int table_kind(const hqq_table &t) { return t.kind == HQQ_TABLE_F16 ? TK_F16 : (t.meta_cols == 1 ? TK_U8_SCALAR : TK_U8_COLS); }
+
+} // namespace gemv
+} // namespace hqq

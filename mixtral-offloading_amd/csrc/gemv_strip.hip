@@ -1,0 +1,639 @@
+// Decode-time GEMV (batch M <= 4) for 2- and 4-bit codes, one launch per matmul or per fused w1/w3 gate.
+//
+// Algebra (shared with the small-batch kernel): the 16 output rows n = F*(jp + r*GP) + i, r = 16*rb .. 16*rb+15,
+// of field i use the same scale and zero in every column, so the scale is folded into the activations,
+//     y[n, m] = sum_k q[n, k] * xs[i, k, m]  -  sum_k z[i, k] * xs[i, k, m],      xs = 32 * s[i, k] * x[m, k]  (fp16),
+// and the only per-weight work left is to present the code as an fp16 number.  That takes one v_and: the field,
+// masked in place, is the fp16 subnormal q * 2^(pos - 24), which v_mfma_f32_16x16x32_f16 multiplies exactly.
+//
+// Work split.  A block owns one tile (jp, rb) of every layer of the launch (two for the gate).  Its waves split K:
+// wave (layer, ks) walks S consecutive slabs of 256 columns and keeps the MFMA accumulators in registers across
+// them, so partial sums meet only once per wave, in LDS.  All loads of a slab are 128 bits wide -- four code loads
+// per lane, and for the table lanes 16 scale bytes, 16 zero bytes, their fp16 meta values and x -- and the loads of
+// up to D slabs are in flight before the first arithmetic.  When the block holds all of K (BK == 1: every Mixtral
+// projection with K = 4096, gate included) it applies the epilogue itself: no workspace, no atomics.  Otherwise
+// (K = 14336) the BK blocks of a tile store fp32 partial sums with device-scope stores and the block that arrives
+// last at the tile's counter adds them in a fixed order.
+//
+// Lane roles inside a slab.  Code lanes: (rr = lane & 15, kg = lane >> 4) own packed row jp + (16*rb + rr)*GP,
+// bytes 64*s + 16*kg .. +15 for step s.  Table lanes: (ti = lane >> 4 < F, kq = lane & 15) own table row F*jp + ti,
+// columns 16*kq .. 16*kq+15, i.e. step kq >> 2, MFMA lane group kq & 3.
+#include "gemv_parts.hpp"
+#include "hqq_common.hpp"
+
+#include <cstdlib>
+
+namespace hqq {
+using namespace gemv;
+namespace {
+
+struct StripLayer {
+    const uint8_t *codes;
+    const uint8_t *sq, *zq; // 8-bit tables, or fp16 tables
+    const f16 *s_ms, *s_mz; // meta of the scale table
+    const f16 *z_ms, *z_mz; // meta of the zero table
+    uint32_t s_cols, z_cols, s_inv, z_inv;
+    float *part; // [BK][M][N]
+};
+
+struct StripParams {
+    StripLayer layer[2];
+    const f16 *x;
+    int M, N, K;
+    int GP, RB;
+    int NS;       // K / 256
+    int KS;       // waves per layer in a block
+    int BK;       // blocks along K per tile
+    int NL;       // layers in this launch (2 = fused gate)
+    int *counter; // one per tile, zero between launches
+    f16 *y;
+    const f16 *bias, *row_scale;
+    int accumulate;
+};
+
+template <int MT, int SKIND, int ZKIND> struct SlabRegs {
+    Raw16<SKIND> s;
+    Raw16<ZKIND> z;
+    u32x4 xv[MT][2];
+    u32x4 cw[4];
+    uint32_t sms, smz, zms, zmz; // whole-tensor meta values, raw fp16 bits
+};
+
+template <int NBITS, int MT, int S, int D, int WAVES, int SKIND, int ZKIND, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
+{
+    constexpr int F = 8 / NBITS;
+    constexpr int ENTRY = 8; // halves per B-operand entry (16 bytes)
+    constexpr int STEP_HALVES = F * 2 * 4 * MT * ENTRY;
+    constexpr int XS_HALVES = 4 * STEP_HALVES;
+    __shared__ __attribute__((aligned(16))) f16 xs_lds[WAVES][XS_HALVES];
+    __shared__ float bias_lds[WAVES][F][MT];
+    __shared__ __attribute__((aligned(16))) float red_lds[WAVES][16][MT][F];
+    __shared__ __attribute__((aligned(16))) float fin_lds[2][16][MT][F];
+    __shared__ int ticket_lds;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int kb = blockIdx.x, rb = blockIdx.y, jp = blockIdx.z;
+    const int layer = wave >= p.KS ? 1 : 0;
+    const int ks = wave - layer * p.KS;
+    const bool wave_on = wave < p.KS * p.NL;
+    // both layer records come from the kernel arguments and are selected in registers: no dependent loads
+    StripLayer L;
+    {
+        const StripLayer &A = p.layer[0], &B = p.layer[1];
+        L.codes = layer ? B.codes : A.codes;
+        L.sq = layer ? B.sq : A.sq;
+        L.zq = layer ? B.zq : A.zq;
+        L.s_ms = layer ? B.s_ms : A.s_ms;
+        L.s_mz = layer ? B.s_mz : A.s_mz;
+        L.z_ms = layer ? B.z_ms : A.z_ms;
+        L.z_mz = layer ? B.z_mz : A.z_mz;
+        L.s_cols = layer ? B.s_cols : A.s_cols;
+        L.z_cols = layer ? B.z_cols : A.z_cols;
+        L.s_inv = layer ? B.s_inv : A.s_inv;
+        L.z_inv = layer ? B.z_inv : A.z_inv;
+    }
+    const int slab0 = (kb * p.KS + ks) * S;
+    const int K = p.K;
+    const int M = MT == 1 ? 1 : p.M;
+
+    const int rr = lane & 15, kg = lane >> 4;
+    const int ti = lane >> 4, kq = lane & 15;
+    const bool tlane = ti < F;     // lanes that own table entries (all of them for 2-bit codes)
+    const int ti_l = ti & (F - 1); // the other lanes repeat a table lane's loads, so that issuing loads never diverges
+
+    const uint32_t trow = (uint32_t)(F * jp + ti_l) * (uint32_t)K + (uint32_t)(16 * kq);
+    const uint32_t crow = ((uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)p.GP) * (uint32_t)K + (uint32_t)(16 * kg);
+
+    auto issue = [&](SlabRegs<MT, SKIND, ZKIND> &r, int slab) __attribute__((always_inline)) {
+        const uint32_t k0 = (uint32_t)slab * kSlab;
+        const uint32_t c = trow + k0;
+        uint32_t scm = 0, zcm = 0;
+        if constexpr (SKIND == TK_U8_COLS) {
+            scm = c - __umulhi(c, L.s_inv) * L.s_cols; // c mod cols; the quotient estimate is at most 2 short
+            scm -= scm >= L.s_cols ? L.s_cols : 0;
+            scm -= scm >= L.s_cols ? L.s_cols : 0;
+        }
+        if constexpr (ZKIND == TK_U8_COLS) {
+            zcm = c - __umulhi(c, L.z_inv) * L.z_cols;
+            zcm -= zcm >= L.z_cols ? L.z_cols : 0;
+            zcm -= zcm >= L.z_cols ? L.z_cols : 0;
+        }
+        load16<SKIND>(r.s, L.sq, L.s_ms, L.s_mz, c, scm);
+        load16<ZKIND>(r.z, L.zq, L.z_ms, L.z_mz, c, zcm);
+        const uint32_t xo = k0 + (uint32_t)(16 * kq);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            if (m < M) {
+                const u32x4 *xp = reinterpret_cast<const u32x4 *>(p.x + (xo + (uint32_t)(m * K)));
+                r.xv[m][0] = xp[0];
+                r.xv[m][1] = xp[1];
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+            r.cw[s] = *reinterpret_cast<const u32x4 *>(L.codes + (crow + k0 + 64 * s));
+        // Whole-tensor meta values ride with the slab, after its weight loads.  Their address is the same in every
+        // lane, but it is written so that the compiler does not see that (lane >> 6 is zero): a load it knows to be
+        // uniform is moved to scalar registers at once, and that move waits for it before any weight load is issued.
+        const int zero_off = lane >> 6;
+        r.sms = r.smz = r.zms = r.zmz = 0;
+        if constexpr (SKIND == TK_U8_SCALAR) {
+            r.sms = reinterpret_cast<const uint16_t *>(L.s_ms)[zero_off];
+            r.smz = reinterpret_cast<const uint16_t *>(L.s_mz)[zero_off];
+        }
+        if constexpr (ZKIND == TK_U8_SCALAR) {
+            r.zms = reinterpret_cast<const uint16_t *>(L.z_ms)[zero_off];
+            r.zmz = reinterpret_cast<const uint16_t *>(L.z_mz)[zero_off];
+        }
+    };
+
+    // B operand of lane (mcol, kg) for (step s, field i, half h): entry ((s*F + i)*2 + h)*4 + kg, batch column mcol.
+    // Column m of the MFMA result depends on column m of B only, and columns m >= M are never read back, so lanes
+    // past the batch simply re-read a valid column instead of needing zeros.
+    const int mcol = lane & 15;
+    f16 *xs_w = &xs_lds[wave][0];
+    const f16 *xs_r = xs_w + (kg * MT + (mcol < M ? mcol : 0)) * ENTRY;
+
+    f32x4 acc[F];
+#pragma unroll
+    for (int i = 0; i < F; ++i)
+        acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float bias_acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+        bias_acc[m] = 0.f;
+
+    auto compute = [&](const SlabRegs<MT, SKIND, ZKIND> &r) __attribute__((always_inline)) {
+        // ------------------------------------------------------------ table phase, once per slab
+        if (tlane) {
+            f16x2 sv[8], zv[8];
+            const f16x2 sms = as_h2(r.sms * 0x10001u), smz = as_h2(r.smz * 0x10001u);
+            const f16x2 zms = as_h2(r.zms * 0x10001u), zmz = as_h2(r.zmz * 0x10001u);
+            decode16<SKIND>(r.s, sms, smz, sv);
+            decode16<ZKIND>(r.z, zms, zmz, zv);
+            const f16x2 k32 = {(f16)kXsScale, (f16)kXsScale};
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                sv[t] = sv[t] * k32;
+            // lane's 16 columns are step kq>>2, lane group kq&3, halves h = 0 (cols 0-7) and 1 (cols 8-15)
+            f16 *dst = xs_w + (kq >> 2) * STEP_HALVES + ((ti * 2) * 4 + (kq & 3)) * MT * ENTRY;
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                if (m < M) {
+                    f16x2 a[8];
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) {
+                        a[t] = sv[t] * as_h2(r.xv[m][t >> 2][t & 3]);
+                        bias_acc[m] = __builtin_amdgcn_fdot2(zv[t], a[t], bias_acc[m], false);
+                    }
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        // B-operand order inside an 8-column block: columns (0,2,1,3,4,6,5,7)
+                        const f16x2 *q = &a[4 * h];
+                        const f16x8 o = {q[0].x, q[1].x, q[0].y, q[1].y, q[2].x, q[3].x, q[2].y, q[3].y};
+                        *reinterpret_cast<f16x8 *>(dst + (h * 4 * MT + m) * ENTRY) = o;
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+        // ------------------------------------------------------------ code phase: 4 steps x 2F MFMAs
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            f16x8 B[2][F];
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int i = 0; i < F; ++i)
+                    B[h][i] = *reinterpret_cast<const f16x8 *>(xs_r + s * STEP_HALVES + ((i * 2 + h) * 4 * MT) * ENTRY);
+            const uint32_t d[4] = {r.cw[s].x, r.cw[s].y, r.cw[s].z, r.cw[s].w};
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t d0 = d[2 * h], d1 = d[2 * h + 1];
+                const uint32_t d0s = d0 >> 8, d1s = d1 >> 8;
+#pragma unroll
+                for (int i = 0; i < F; ++i) {
+                    const uint32_t mk = Field<NBITS>::mask(i);
+                    const u32x4 Au = {d0 & mk, d0s & mk, d1 & mk, d1s & mk};
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, Au), B[h][i], acc[i], 0, 0, 0);
+                }
+            }
+        }
+        // the next slab's table phase overwrites xs: keep it behind these reads
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+
+    // ---------------------------------------------------------------- S slabs, D of them in flight
+    // A slab past the end of K is issued all the same (it re-reads the last slab and is never used): with a fixed
+    // number of loads the compiler waits for exactly the loads a slab needs and leaves the later ones in flight.
+    if (wave_on) {
+        SlabRegs<MT, SKIND, ZKIND> regs[D];
+        const int last = p.NS - 1;
+#pragma unroll
+        for (int i = 0; i < D; ++i)
+            issue(regs[i], slab0 + i < p.NS ? slab0 + i : last);
+#pragma unroll
+        for (int i = 0; i < S; ++i) {
+            if (slab0 + i < p.NS)
+                compute(regs[i % D]);
+            if (i + D < S)
+                issue(regs[i % D], slab0 + i + D < p.NS ? slab0 + i + D : last);
+        }
+    }
+
+    // ---------------------------------------------------------------- wave tile -> LDS (zero term removed, unscaled)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const float v = row16_sum(bias_acc[m]);
+        if (tlane && kq == 0)
+            bias_lds[wave][ti][m] = v * (1.0f / kXsScale);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (mcol < MT) {
+        float bz[F];
+#pragma unroll
+        for (int i = 0; i < F; ++i)
+            bz[i] = bias_lds[wave][i][mcol];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            float o[F];
+#pragma unroll
+            for (int i = 0; i < F; ++i)
+                o[i] = __builtin_fmaf(acc[i][v], Field<NBITS>::unscale(i), -bz[i]);
+            float *dst = &red_lds[wave][4 * kg + v][mcol][0];
+            if constexpr (F == 4)
+                *reinterpret_cast<f32x4 *>(dst) = (f32x4){o[0], o[1], o[2], o[3]};
+            else
+                *reinterpret_cast<float2 *>(dst) = make_float2(o[0], o[1]);
+        }
+    }
+    __syncthreads();
+
+    // ---------------------------------------------------------------- block tile: 16 lanes per (layer, row, batch row)
+    const bool alone = p.BK == 1;
+    const int tile = jp * p.RB + rb;
+    for (int t = threadIdx.x; t < p.NL * 16 * MT * 16; t += WAVES * 64) {
+        const int w = t & 15, u = t >> 4;
+        const int l_t = u / (16 * MT), r_t = (u / MT) & 15, m_t = u % MT;
+        float o[F];
+#pragma unroll
+        for (int i = 0; i < F; ++i)
+            o[i] = 0.f;
+        if (w < p.KS) {
+            const float *src = &red_lds[l_t * p.KS + w][r_t][m_t][0];
+#pragma unroll
+            for (int i = 0; i < F; ++i)
+                o[i] = src[i];
+        }
+#pragma unroll
+        for (int i = 0; i < F; ++i)
+            o[i] = row16_sum(o[i]);
+        if (w != 0 || m_t >= M)
+            continue;
+        const int r = 16 * rb + r_t;
+        const int64_t n = (int64_t)F * (jp + (int64_t)r * p.GP); // outputs n .. n+F-1
+        if (!alone) {
+            // device-scope stores: written through the (per-XCD, mutually non-coherent) L2 so that the finishing
+            // block, which may run on another XCD, can read them without any cache-wide flush
+            float *dst = (l_t ? p.layer[1].part : p.layer[0].part) + ((int64_t)kb * M + m_t) * p.N + n;
+#pragma unroll
+            for (int i = 0; i < F; ++i)
+                __hip_atomic_store(dst + i, o[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            continue;
+        }
+        if constexpr (EPI == 1) {
+            float *dst = &fin_lds[l_t][r_t][m_t][0];
+#pragma unroll
+            for (int i = 0; i < F; ++i)
+                dst[i] = o[i];
+        } else {
+            f16 *dst = p.y + (int64_t)m_t * p.N + n;
+            f16 hv[F];
+#pragma unroll
+            for (int i = 0; i < F; ++i) {
+                f16 val = (f16)o[i];
+                if (p.bias)
+                    val = val + p.bias[n + i];
+                if (p.row_scale)
+                    val = val * p.row_scale[m_t];
+                if (p.accumulate)
+                    val = dst[i] + val;
+                hv[i] = val;
+            }
+            if constexpr (F == 4)
+                *reinterpret_cast<f16x4 *>(dst) = (f16x4){hv[0], hv[1], hv[2], hv[3]};
+            else
+                *reinterpret_cast<f16x2 *>(dst) = (f16x2){hv[0], hv[1]};
+        }
+    }
+
+    // both projections rounded to fp16, SiLU in fp32 rounded once, product in fp16: as the reference's ops do
+    auto gate = [](float a, float b) __attribute__((always_inline)) -> f16 {
+        const float g = (float)(f16)a;
+        const f16 act = (f16)(g / (1.0f + __expf(-g)));
+        return act * (f16)b;
+    };
+
+    if (alone) {
+        if constexpr (EPI == 1) {
+            __syncthreads();
+            for (int u = threadIdx.x; u < 16 * MT; u += WAVES * 64) {
+                const int r_t = u / MT, m_t = u % MT;
+                if (m_t >= M)
+                    continue;
+                const int r = 16 * rb + r_t;
+                const int64_t n = (int64_t)F * (jp + (int64_t)r * p.GP);
+                f16 hv[F];
+#pragma unroll
+                for (int i = 0; i < F; ++i)
+                    hv[i] = gate(fin_lds[0][r_t][m_t][i], fin_lds[1][r_t][m_t][i]);
+                f16 *dst = p.y + (int64_t)m_t * p.N + n;
+                if constexpr (F == 4)
+                    *reinterpret_cast<f16x4 *>(dst) = (f16x4){hv[0], hv[1], hv[2], hv[3]};
+                else
+                    *reinterpret_cast<f16x2 *>(dst) = (f16x2){hv[0], hv[1]};
+            }
+        }
+        return;
+    }
+
+    // ---------------------------------------------------------------- the block that arrives last finishes the tile
+    // The partial sums were stored at device scope; once those stores are acknowledged the arrival is counted
+    // with a device-scope atomic.  No cache-wide write-back or invalidate is involved (a __threadfence here
+    // flushes the whole L2 of the XCD and costs more than the matmul).
+    __builtin_amdgcn_s_waitcnt(0); // vmcnt(0) expcnt(0) lgkmcnt(0): every store of this thread is acknowledged
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int prev = __hip_atomic_fetch_add(&p.counter[tile], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (prev == p.BK - 1) // every contributor has arrived: leave the counter ready for the next launch
+            __hip_atomic_store(&p.counter[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ticket_lds = prev;
+    }
+    __syncthreads();
+    if (ticket_lds != p.BK - 1)
+        return;
+    for (int u = threadIdx.x; u < 16 * MT; u += WAVES * 64) {
+        const int r_t = u / MT, m_t = u % MT;
+        if (m_t >= M)
+            continue;
+        const int r = 16 * rb + r_t;
+        const int64_t n = (int64_t)F * (jp + (int64_t)r * p.GP);
+        float a[F], b[F];
+#pragma unroll
+        for (int i = 0; i < F; ++i)
+            a[i] = b[i] = 0.f;
+        for (int s = 0; s < p.BK; ++s) { // fixed order: results do not depend on which block came last
+            const int64_t off = ((int64_t)s * M + m_t) * p.N + n;
+#pragma unroll
+            for (int i = 0; i < F; ++i) {
+                a[i] += __hip_atomic_load(p.layer[0].part + off + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if constexpr (EPI == 1)
+                    b[i] += __hip_atomic_load(p.layer[1].part + off + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        f16 *dst = p.y + (int64_t)m_t * p.N + n;
+        f16 hv[F];
+#pragma unroll
+        for (int i = 0; i < F; ++i) {
+            if constexpr (EPI == 1) {
+                hv[i] = gate(a[i], b[i]);
+            } else {
+                f16 val = (f16)a[i];
+                if (p.bias)
+                    val = val + p.bias[n + i];
+                if (p.row_scale)
+                    val = val * p.row_scale[m_t];
+                if (p.accumulate)
+                    val = dst[i] + val;
+                hv[i] = val;
+            }
+        }
+        if constexpr (F == 4)
+            *reinterpret_cast<f16x4 *>(dst) = (f16x4){hv[0], hv[1], hv[2], hv[3]};
+        else
+            *reinterpret_cast<f16x2 *>(dst) = (f16x2){hv[0], hv[1]};
+    }
+}
+
+__global__ void zero_words_kernel(uint32_t *p, size_t n)
+{
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        p[i] = 0;
+}
+
+int env_int(const char *name, int dflt)
+{
+    const char *v = std::getenv(name);
+    return v ? std::atoi(v) : dflt;
+}
+
+struct StripPlan {
+    int F, GP, RB, NS, MT, S, D, WAVES, KS, BK, SKIND, ZKIND;
+};
+
+bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl)
+{
+    if ((l->nbits != 2 && l->nbits != 4) || M < 1 || M > 4)
+        return false;
+    const int F = 8 / l->nbits;
+    const int64_t G = l->N / l->group_size;
+    if (l->group_size % 16 != 0 || G % F != 0 || l->K % kSlab != 0 || l->N % 4 != 0)
+        return false;
+    if (l->N * l->K / l->group_size >= (1ll << 31) || l->N * l->K / F >= (1ll << 32) || 16 * l->K >= (1ll << 31))
+        return false; // 32-bit offsets inside the kernel
+    if (!aligned16(l->codes) || !aligned16(l->scale.data) || !aligned16(l->zero.data))
+        return false;
+    pl.SKIND = table_kind(l->scale);
+    pl.ZKIND = table_kind(l->zero);
+    // instantiated table combinations: HQQ default (scale u8 per-column meta, zero u8 scalar meta) and fp16 tables
+    if (!((pl.SKIND == TK_U8_COLS && pl.ZKIND == TK_U8_SCALAR) || (pl.SKIND == TK_F16 && pl.ZKIND == TK_F16)))
+        return false;
+    if (pl.SKIND == TK_U8_COLS && (l->scale.meta_cols % 16 != 0 || !aligned16(l->scale.meta_scale) ||
+                                   !aligned16(l->scale.meta_zero)))
+        return false;
+    pl.F = F;
+    pl.GP = (int)(G / F);
+    pl.RB = l->group_size / 16;
+    pl.NS = (int)(l->K / kSlab);
+    pl.MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
+    if (pl.GP > 65535 || pl.RB > 65535 || (int64_t)pl.GP * pl.RB * sizeof(int) > kCounterBytes)
+        return false;
+    // Shape of the split: S slabs per wave, KS waves per layer, BK blocks along K.  One slab per wave (the most
+    // waves in flight) unless a block that holds all of K would then need more than 16 waves; K is split over
+    // several blocks only when a single block cannot hold it or there would be too few blocks to cover the chip.
+    const int64_t tiles = (int64_t)pl.GP * pl.RB;
+    const int max_waves = pl.MT == 1 ? 16 : 8; // wider batches need the registers and the LDS staging of a wave twice over
+    int S = 1, BK = 1;
+    int KS = pl.NS;
+    if (KS * NL > max_waves && (pl.NS + 1) / 2 * NL <= max_waves) {
+        S = 2;
+        KS = (pl.NS + 1) / 2;
+    }
+    while (KS * NL > max_waves || (tiles * BK < 200 && KS > 4 && BK < 16)) {
+        ++BK;
+        KS = ((pl.NS + S - 1) / S + BK - 1) / BK;
+    }
+    S = env_int("HQQ_STRIP_S", S);
+    KS = env_int("HQQ_STRIP_KS", KS);
+    BK = env_int("HQQ_STRIP_BK", BK);
+    if (S != 1 && S != 2)
+        return false;
+    if (KS < 1 || KS * NL > max_waves || BK < 1 || BK > 65535)
+        return false;
+    if ((int64_t)S * KS * BK < pl.NS)
+        return false;
+    pl.S = S, pl.KS = KS, pl.BK = BK;
+    pl.WAVES = KS * NL > 8 ? 16 : (KS * NL > 4 ? 8 : 4);
+    pl.D = S; // every slab of the wave in flight at once
+    return true;
+}
+
+void fill_layer(StripLayer &L, const hqq_linear *l, float *part)
+{
+    L.codes = static_cast<const uint8_t *>(l->codes);
+    L.sq = static_cast<const uint8_t *>(l->scale.data);
+    L.zq = static_cast<const uint8_t *>(l->zero.data);
+    L.s_ms = static_cast<const f16 *>(l->scale.meta_scale);
+    L.s_mz = static_cast<const f16 *>(l->scale.meta_zero);
+    L.z_ms = static_cast<const f16 *>(l->zero.meta_scale);
+    L.z_mz = static_cast<const f16 *>(l->zero.meta_zero);
+    L.s_cols = (uint32_t)l->scale.meta_cols;
+    L.z_cols = (uint32_t)l->zero.meta_cols;
+    L.s_inv = L.s_cols ? (uint32_t)(0xFFFFFFFFull / L.s_cols) : 0;
+    L.z_inv = L.z_cols ? (uint32_t)(0xFFFFFFFFull / L.z_cols) : 0;
+    L.part = part;
+}
+
+template <int NBITS, int MT, int S, int D, int WAVES, int EPI>
+void launch_kinds(const StripParams &p, const StripPlan &pl, dim3 grid, hipStream_t s)
+{
+    if (pl.SKIND == TK_F16)
+        gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_F16, TK_F16, EPI><<<grid, dim3(WAVES * 64), 0, s>>>(p);
+    else
+        gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_U8_COLS, TK_U8_SCALAR, EPI><<<grid, dim3(WAVES * 64), 0, s>>>(p);
+}
+
+template <int NBITS, int MT, int S, int D, int EPI>
+void launch_waves(const StripParams &p, const StripPlan &pl, dim3 grid, hipStream_t s)
+{
+    if constexpr (MT == 1) {
+        if (pl.WAVES == 16) {
+            launch_kinds<NBITS, MT, S, D, 16, EPI>(p, pl, grid, s);
+            return;
+        }
+    }
+    if (pl.WAVES >= 8)
+        launch_kinds<NBITS, MT, S, D, 8, EPI>(p, pl, grid, s);
+    else
+        launch_kinds<NBITS, MT, S, D, 4, EPI>(p, pl, grid, s);
+}
+
+template <int NBITS, int MT, int EPI> void launch_depth(const StripParams &p, const StripPlan &pl, dim3 grid, hipStream_t s)
+{
+    if (pl.S == 1)
+        launch_waves<NBITS, MT, 1, 1, EPI>(p, pl, grid, s);
+    else
+        launch_waves<NBITS, MT, 2, 2, EPI>(p, pl, grid, s);
+}
+
+template <int NBITS, int EPI> void launch_batch(const StripParams &p, const StripPlan &pl, dim3 grid, hipStream_t s)
+{
+    if (pl.MT == 1)
+        launch_depth<NBITS, 1, EPI>(p, pl, grid, s);
+    else if (pl.MT == 2)
+        launch_depth<NBITS, 2, EPI>(p, pl, grid, s);
+    else
+        launch_depth<NBITS, 4, EPI>(p, pl, grid, s);
+}
+
+int run(const hqq_linear *l0, const hqq_linear *l1, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
+        const SmallBatchEpilogue &ep, hipStream_t s)
+{
+    StripPlan pl;
+    const int NL = l1 ? 2 : 1;
+    if (!make_plan(l0, M, NL, pl))
+        return HQQ_E_UNSUPPORTED;
+    const size_t one = (size_t)pl.BK * (size_t)M * (size_t)l0->N * sizeof(float);
+    const bool alone = pl.BK == 1;
+    if (!alone && (!ws || ws_bytes < kCounterBytes + NL * one))
+        return HQQ_E_WORKSPACE;
+    StripParams p = {};
+    char *base = static_cast<char *>(ws);
+    fill_layer(p.layer[0], l0, alone ? nullptr : reinterpret_cast<float *>(base + kCounterBytes));
+    if (l1)
+        fill_layer(p.layer[1], l1, alone ? nullptr : reinterpret_cast<float *>(base + kCounterBytes + one));
+    else
+        p.layer[1] = p.layer[0];
+    p.x = x, p.M = (int)M, p.N = (int)l0->N, p.K = (int)l0->K;
+    p.GP = pl.GP, p.RB = pl.RB, p.NS = pl.NS, p.KS = pl.KS, p.BK = pl.BK, p.NL = NL;
+    p.counter = reinterpret_cast<int *>(base);
+    p.y = y, p.bias = static_cast<const f16 *>(l0->bias), p.row_scale = ep.row_scale, p.accumulate = ep.accumulate;
+    const dim3 grid((unsigned)pl.BK, (unsigned)pl.RB, (unsigned)pl.GP);
+    if (l1) {
+        if (l0->nbits == 2)
+            launch_batch<2, 1>(p, pl, grid, s);
+        else
+            launch_batch<4, 1>(p, pl, grid, s);
+    } else {
+        if (l0->nbits == 2)
+            launch_batch<2, 0>(p, pl, grid, s);
+        else
+            launch_batch<4, 0>(p, pl, grid, s);
+    }
+    return launch_status();
+}
+
+} // namespace
+
+bool strip_supported(const hqq_linear *l, int64_t M)
+{
+    StripPlan pl;
+    return make_plan(l, M, 1, pl);
+}
+
+size_t strip_workspace_bytes(const hqq_linear *l, int64_t M)
+{
+    StripPlan pl;
+    if (!make_plan(l, M, 1, pl))
+        return 0;
+    // sized for the worst split the planner may choose for this shape (one slab per wave and block)
+    return kCounterBytes + (size_t)pl.NS * (size_t)M * (size_t)l->N * sizeof(float);
+}
+
+int launch_strip_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
+                        const SmallBatchEpilogue &ep, hipStream_t s)
+{
+    return run(l, nullptr, x, M, y, ws, ws_bytes, ep, s);
+}
+
+int launch_strip_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
+                         size_t ws_bytes, hipStream_t s)
+{
+    StripPlan a, b;
+    if (!make_plan(w1, M, 2, a) || !make_plan(w3, M, 2, b) || w1->N != w3->N || w1->K != w3->K || w1->nbits != w3->nbits ||
+        w1->group_size != w3->group_size || a.SKIND != b.SKIND || a.ZKIND != b.ZKIND)
+        return HQQ_E_UNSUPPORTED;
+    return run(w1, w3, x, M, h, ws, ws_bytes, SmallBatchEpilogue{}, s);
+}
+
+int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s)
+{
+    const size_t n = (ws_bytes < kCounterBytes ? ws_bytes : kCounterBytes) / 4;
+    if (n == 0)
+        return HQQ_OK;
+    zero_words_kernel<<<16, 256, 0, s>>>(static_cast<uint32_t *>(ws), n);
+    return launch_status();
+}
+
+size_t workspace_head_bytes() { return kCounterBytes; }
+
+} // namespace hqq

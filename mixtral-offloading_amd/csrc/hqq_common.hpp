@@ -98,13 +98,14 @@ int launch_smallbatch_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *
 // fused w1/w3 pass: h = silu(x w1^T) * (x w3^T), fp16 (M, N)
 int launch_smallbatch_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
                               size_t ws_bytes, hipStream_t s);
-// slab kernel (M <= 4, K % 256 == 0): the decode path; part of the small-batch family
-bool slab_supported(const hqq_linear *l, int64_t M);
-size_t slab_workspace_bytes(const hqq_linear *l, int64_t M);
-int launch_slab_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
-                       const SmallBatchEpilogue &ep, hipStream_t s);
-int launch_slab_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
-                        size_t ws_bytes, hipStream_t s);
+// strip kernel (M <= 4, K % 256 == 0): the decode path; part of the small-batch family.  A block per tile, one or two
+// slabs of 256 columns per wave, in-block gate epilogue
+bool strip_supported(const hqq_linear *l, int64_t M);
+size_t strip_workspace_bytes(const hqq_linear *l, int64_t M);
+int launch_strip_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
+                        const SmallBatchEpilogue &ep, hipStream_t s);
+int launch_strip_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
+                         size_t ws_bytes, hipStream_t s);
 int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s);
 size_t workspace_head_bytes();
 bool tile_supported(const hqq_linear *l, int64_t M);

@@ -486,14 +486,14 @@ int finish_grid(int64_t M, int64_t N)
 bool smallbatch_supported(const hqq_linear *l, int64_t M)
 {
     SBPlan pl;
-    return slab_supported(l, M) || make_plan(l, M, pl);
+    return strip_supported(l, M) || make_plan(l, M, pl);
 }
 
 // the first workspace_head_bytes() of a workspace belong to the slab kernel's arrival counters
 size_t smallbatch_workspace_bytes(const hqq_linear *l, int64_t M)
 {
-    if (slab_supported(l, M))
-        return slab_workspace_bytes(l, M);
+    if (strip_supported(l, M))
+        return strip_workspace_bytes(l, M);
     SBPlan pl;
     if (!make_plan(l, M, pl))
         return 0;
@@ -515,8 +515,8 @@ static void fill_params(SBParams &p, const SBPlan &pl, const hqq_linear *l, int 
 int launch_smallbatch_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
                              const SmallBatchEpilogue &ep, hipStream_t s)
 {
-    if (slab_supported(l, M))
-        return launch_slab_matmul(l, x, M, y, ws, ws_bytes, ep, s);
+    if (strip_supported(l, M))
+        return launch_strip_matmul(l, x, M, y, ws, ws_bytes, ep, s);
     SBPlan pl;
     if (!make_plan(l, M, pl))
         return HQQ_E_UNSUPPORTED;
@@ -545,8 +545,8 @@ int launch_smallbatch_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *
 int launch_smallbatch_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
                               size_t ws_bytes, hipStream_t s)
 {
-    if (slab_supported(w1, M) && slab_supported(w3, M))
-        return launch_slab_gate_up(w1, w3, x, M, h, ws, ws_bytes, s);
+    if (strip_supported(w1, M) && strip_supported(w3, M))
+        return launch_strip_gate_up(w1, w3, x, M, h, ws, ws_bytes, s);
     SBPlan pl, pl3;
     if (!make_plan(w1, M, pl) || !make_plan(w3, M, pl3) || w1->N != w3->N || w1->K != w3->K ||
         w1->nbits != w3->nbits || w1->group_size != w3->group_size)

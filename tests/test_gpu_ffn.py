@@ -1,0 +1,115 @@
+"""GPU parity tests of the expert FFN entry point (reference src/custom_layers.py:253-256, :308-312) against the
+numpy oracle at small sizes, and against de-quantise-then-matmul on the GPU at Mixtral size."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_matmul_close, desc_of, to_dev
+from oracle import hqq_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+# (nbits, hidden, ffn, group_size, quant tables); hidden <= 4096 and batch <= 2 take the single-launch kernel
+SHAPES = [
+    (2, 256, 1024, 16, True),    # one slab in phase 1, four in phase 2
+    (2, 1024, 3584, 16, True),   # G of the gate projections = 224 (table meta period that does not divide K)
+    (2, 4096, 512, 16, True),    # sixteen slabs in phase 1: every wave busy
+    (2, 512, 8192, 16, True),    # phase 2 split over two blocks per tile
+    (4, 512, 1024, 64, True),    # four row blocks per tile
+    (4, 256, 512, 32, False),    # fp16 tables
+    (2, 768, 1280, 16, False),
+]
+
+
+def _ffn_case(rng, nbits, hidden, ffn, gs, qt):
+    w1, _ = o.random_layer(rng, ffn, hidden, nbits, gs, qt, qt)
+    w3, _ = o.random_layer(rng, ffn, hidden, nbits, gs, qt, qt)
+    w2, _ = o.random_layer(rng, hidden, ffn, nbits, gs, qt, qt)
+    return w1, w2, w3
+
+
+def _tolerance(x, w1, w2, w3):
+    a = o.matmul_transpose(x, w1)
+    b = o.matmul_transpose(x, w3)
+    h = (o.silu_f16(a).astype(np.float32) * b.astype(np.float32)).astype(np.float16)
+    # the intermediate h carries the tolerance of two matmuls already: allow 4x the single-matmul bound
+    return 4 * o.matmul_tolerance(h, w2)
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "w%d_h%d_f%d_g%d_%s" % (s[0], s[1], s[2], s[3], "q" if s[4] else "f16"))
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 16])
+def test_expert_ffn_against_oracle(shape, m):
+    from mixtral_offloading_amd import hip_kernels
+    nbits, hidden, ffn, gs, qt = shape
+    rng = np.random.default_rng(hidden + ffn + m)
+    w1, w2, w3 = _ffn_case(rng, nbits, hidden, ffn, gs, qt)
+    x = rng.standard_normal((m, hidden)).astype(np.float16)
+    d1, d2, d3 = desc_of(w1), desc_of(w2), desc_of(w3)
+    ref = o.expert_ffn(x, w1, w2, w3)
+    atol = _tolerance(x, w1, w2, w3)
+    for rep in range(3):  # the arrival counters must be left ready for the next call
+        y = hip_kernels.expert_ffn(d1, d2, d3, to_dev(x)).cpu().numpy()
+        assert_matmul_close(y, ref, atol, rtol=2e-2)
+
+
+@pytest.mark.parametrize("m", [1, 2, 4])
+def test_expert_ffn_row_scale_and_accumulate(m):
+    """Routing weight and the index_add_ of the reference (src/custom_layers.py:308-312) as the FFN's epilogue."""
+    from mixtral_offloading_amd import hip_kernels
+    rng = np.random.default_rng(7 + m)
+    w1, w2, w3 = _ffn_case(rng, 2, 512, 1792, 16, True)
+    x = rng.standard_normal((m, 512)).astype(np.float16)
+    rw = rng.uniform(0.1, 0.9, size=(m,)).astype(np.float16)
+    base = rng.standard_normal((m, 512)).astype(np.float16)
+    d1, d2, d3 = desc_of(w1), desc_of(w2), desc_of(w3)
+    plain = hip_kernels.expert_ffn(d1, d2, d3, to_dev(x))
+    out = to_dev(base.copy())
+    hip_kernels.expert_ffn(d1, d2, d3, to_dev(x), out=out, row_scale=to_dev(rw), accumulate=True)
+    # fp16 multiply by the routing weight, then fp16 add, exactly as the reference's ops would on the plain result
+    want = to_dev(base) + plain * to_dev(rw)[:, None]
+    assert torch.equal(out, want)
+
+
+@pytest.mark.parametrize("m", [1, 2])
+def test_single_launch_ffn_equals_three_kernel_path(m, monkeypatch):
+    """The persistent kernel and the gate + w2 launches round at the same places: results are identical."""
+    from mixtral_offloading_amd import hip_kernels
+    rng = np.random.default_rng(11 + m)
+    w1, w2, w3 = _ffn_case(rng, 2, 1024, 3584, 16, True)
+    x = rng.standard_normal((m, 1024)).astype(np.float16)
+    d1, d2, d3 = desc_of(w1), desc_of(w2), desc_of(w3)
+    fused = hip_kernels.expert_ffn(d1, d2, d3, to_dev(x)).cpu().numpy()
+    monkeypatch.setenv("HQQ_NO_FUSED_FFN", "1")
+    split = hip_kernels.expert_ffn(d1, d2, d3, to_dev(x)).cpu().numpy()
+    monkeypatch.delenv("HQQ_NO_FUSED_FFN")
+    atol = _tolerance(x, w1, w2, w3)
+    assert_matmul_close(fused, o.expert_ffn(x, w1, w2, w3), atol, rtol=2e-2)
+    assert_matmul_close(split, o.expert_ffn(x, w1, w2, w3), atol, rtol=2e-2)
+    # same algebra, different summation order across waves: tiny differences only
+    assert np.abs(fused.astype(np.float32) - split.astype(np.float32)).max() <= 2 * atol.max()
+
+
+@pytest.mark.parametrize("m", [1, 2, 4, 16])
+def test_full_size_ffn_against_dequantize_then_matmul(m):
+    """Mixtral shapes (2-bit g16, 4096 -> 14336 -> 4096): the library's bit-exact de-quantiser followed by torch
+    matmuls with the reference's fp16 roundings."""
+    from mixtral_offloading_amd import hip_kernels
+    from test_gpu_matmul import _full_size_layer
+    d1 = _full_size_layer(2, 14336, 4096, 16, seed=1)
+    d2 = _full_size_layer(2, 4096, 14336, 16, seed=2)
+    d3 = _full_size_layer(2, 14336, 4096, 16, seed=3)
+    g = torch.Generator(device="cuda").manual_seed(m)
+    x = torch.randn((m, 4096), device="cuda", generator=g).half()
+    wa, wb, wc = (hip_kernels.dequantize(d).float() for d in (d1, d3, d2))
+    a = (x.float() @ wa.t()).half()
+    b = (x.float() @ wb.t()).half()
+    h = torch.nn.functional.silu(a) * b
+    ref = h.float() @ wc.t()
+    for rep in range(2):
+        y = hip_kernels.expert_ffn(d1, d2, d3, x)
+        err = (y.float() - ref).abs()
+        atol = 4e-3 * h.float().norm(dim=1)[:, None] * wc.norm(dim=1)[None, :]
+        bound = 2e-2 * ref.abs() + atol
+        assert bool((err <= bound).all()), float((err / bound).max())
