@@ -54,8 +54,10 @@ struct StripParams {
 template <int MT, int SKIND, int ZKIND> struct SlabRegs {
     Raw16<SKIND> s;
     Raw16<ZKIND> z;
-    u32x4 xv[MT][2];
-    u32x4 cw[4];
+    // the slab's activations.  Staged (MT <= 2): xw[j], lanes 0..31 hold 8 columns each of batch row 2j, lanes 32..63 of
+    // row 2j+1.  Direct (MT = 4): xw[2m], xw[2m+1] are the table lane's own 16 columns of batch row m.
+    u32x4 xw[MT <= 2 ? (MT + 1) / 2 : 2 * MT];
+    u32x4 cw[4];             // codes: load i holds rows 4i .. 4i+3 of the tile, 16 lanes x 16 bytes per row
     uint32_t sms, smz, zms, zmz; // whole-tensor meta values, raw fp16 bits
 };
 
@@ -66,7 +68,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     constexpr int ENTRY = 8; // halves per B-operand entry (16 bytes)
     constexpr int STEP_HALVES = F * 2 * 4 * MT * ENTRY;
     constexpr int XS_HALVES = 4 * STEP_HALVES;
+    // Codes are staged through LDS for batches of one and two rows; at four rows the activation staging already
+    // takes most of the LDS a wave can have, and there the codes are loaded straight into the MFMA layout.
+    constexpr bool STAGE = MT <= 2;
+    constexpr int CODE_PITCH = kSlab + 16; // bytes per tile row in the staging buffer: the pad spreads the rows over the banks
     __shared__ __attribute__((aligned(16))) f16 xs_lds[WAVES][XS_HALVES];
+    __shared__ __attribute__((aligned(16))) uint8_t code_lds[STAGE ? WAVES : 1][STAGE ? 16 * CODE_PITCH : 16];
+    __shared__ __attribute__((aligned(16))) f16 xw_lds[STAGE ? WAVES : 1][STAGE ? 2 * ((MT + 1) / 2) : 1][STAGE ? kSlab : 8];
     __shared__ float bias_lds[WAVES][F][MT];
     __shared__ __attribute__((aligned(16))) float red_lds[WAVES][16][MT][F];
     __shared__ __attribute__((aligned(16))) float fin_lds[2][16][MT][F];
@@ -104,7 +112,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     const int ti_l = ti & (F - 1); // the other lanes repeat a table lane's loads, so that issuing loads never diverges
 
     const uint32_t trow = (uint32_t)(F * jp + ti_l) * (uint32_t)K + (uint32_t)(16 * kq);
-    const uint32_t crow = ((uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)p.GP) * (uint32_t)K + (uint32_t)(16 * kg);
+    // Weight loads walk the tile row by row -- four consecutive lanes read 64 consecutive bytes, which is the unit the
+    // address pipeline of the memory path handles per cycle -- and reach the MFMA layout (lane = row + 16 * k group)
+    // through an LDS staging buffer.  Loading straight into that layout puts four different rows into every group of
+    // four lanes and costs four times the address cycles; with twelve loads per slab that pipeline, not HBM, then
+    // bounds the kernel.
+    const int lrow = lane >> 4, lchunk = lane & 15;
+    const uint32_t crow = STAGE ? ((uint32_t)jp + (uint32_t)(16 * rb + lrow) * (uint32_t)p.GP) * (uint32_t)K + (uint32_t)(16 * lchunk)
+                                : ((uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)p.GP) * (uint32_t)K + (uint32_t)(16 * kg);
+    const uint32_t crow_step = STAGE ? 4u * (uint32_t)p.GP * (uint32_t)K : 64u; // four tile rows further / next step
 
     auto issue = [&](SlabRegs<MT, SKIND, ZKIND> &r, int slab) __attribute__((always_inline)) {
         const uint32_t k0 = (uint32_t)slab * kSlab;
@@ -122,18 +138,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
         }
         load16<SKIND>(r.s, L.sq, L.s_ms, L.s_mz, c, scm);
         load16<ZKIND>(r.z, L.zq, L.z_ms, L.z_mz, c, zcm);
-        const uint32_t xo = k0 + (uint32_t)(16 * kq);
+        // x: one coalesced piece per pair of batch rows (16 bytes per lane, 32 lanes per row)
+        if constexpr (STAGE) {
 #pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            if (m < M) {
-                const u32x4 *xp = reinterpret_cast<const u32x4 *>(p.x + (xo + (uint32_t)(m * K)));
-                r.xv[m][0] = xp[0];
-                r.xv[m][1] = xp[1];
+            for (int j = 0; j < (MT + 1) / 2; ++j) {
+                int m = 2 * j + (lane >> 5);
+                m = m < M ? m : 0;
+                r.xw[j] = *reinterpret_cast<const u32x4 *>(p.x + (k0 + (uint32_t)(8 * (lane & 31)) + (uint32_t)(m * K)));
+            }
+        } else {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const u32x4 *xp = reinterpret_cast<const u32x4 *>(p.x + (k0 + (uint32_t)(16 * kq) + (uint32_t)((m < M ? m : 0) * K)));
+                r.xw[2 * m] = xp[0];
+                r.xw[2 * m + 1] = xp[1];
             }
         }
 #pragma unroll
-        for (int s = 0; s < 4; ++s)
-            r.cw[s] = *reinterpret_cast<const u32x4 *>(L.codes + (crow + k0 + 64 * s));
+        for (int i = 0; i < 4; ++i)
+            r.cw[i] = *reinterpret_cast<const u32x4 *>(L.codes + (crow + k0 + (uint32_t)i * crow_step));
         // Whole-tensor meta values ride with the slab, after its weight loads.  Their address is the same in every
         // lane, but it is written so that the compiler does not see that (lane >> 6 is zero): a load it knows to be
         // uniform is moved to scalar registers at once, and that move waits for it before any weight load is issued.
@@ -165,7 +188,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     for (int m = 0; m < MT; ++m)
         bias_acc[m] = 0.f;
 
+    uint8_t *code_w = &code_lds[wave][0];
     auto compute = [&](const SlabRegs<MT, SKIND, ZKIND> &r) __attribute__((always_inline)) {
+        // ------------------------------------------------------------ staging: x and the codes change lanes through LDS
+        if constexpr (STAGE) {
+#pragma unroll
+            for (int j = 0; j < (MT + 1) / 2; ++j)
+                *reinterpret_cast<u32x4 *>(&xw_lds[wave][2 * j + (lane >> 5)][8 * (lane & 31)]) = r.xw[j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                *reinterpret_cast<u32x4 *>(code_w + (4 * i + lrow) * CODE_PITCH + 16 * lchunk) = r.cw[i];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         // ------------------------------------------------------------ table phase, once per slab
         if (tlane) {
             f16x2 sv[8], zv[8];
@@ -182,10 +218,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 if (m < M) {
+                    u32x4 x0, x1;
+                    if constexpr (STAGE) {
+                        const u32x4 *xp = reinterpret_cast<const u32x4 *>(&xw_lds[wave][m][16 * kq]);
+                        x0 = xp[0], x1 = xp[1];
+                    } else {
+                        x0 = r.xw[MT <= 2 ? 0 : 2 * m], x1 = r.xw[MT <= 2 ? 0 : 2 * m + 1];
+                    }
                     f16x2 a[8];
 #pragma unroll
                     for (int t = 0; t < 8; ++t) {
-                        a[t] = sv[t] * as_h2(r.xv[m][t >> 2][t & 3]);
+                        a[t] = sv[t] * as_h2(t < 4 ? x0[t & 3] : x1[t & 3]);
                         bias_acc[m] = __builtin_amdgcn_fdot2(zv[t], a[t], bias_acc[m], false);
                     }
 #pragma unroll
@@ -211,7 +254,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
 #pragma unroll
                 for (int i = 0; i < F; ++i)
                     B[h][i] = *reinterpret_cast<const f16x8 *>(xs_r + s * STEP_HALVES + ((i * 2 + h) * 4 * MT) * ENTRY);
-            const uint32_t d[4] = {r.cw[s].x, r.cw[s].y, r.cw[s].z, r.cw[s].w};
+            u32x4 cws = r.cw[s];
+            if constexpr (STAGE)
+                cws = *reinterpret_cast<const u32x4 *>(code_w + rr * CODE_PITCH + 16 * (4 * s + kg));
+            const uint32_t d[4] = {cws.x, cws.y, cws.z, cws.w};
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const uint32_t d0 = d[2 * h], d1 = d[2 * h + 1];
@@ -471,7 +517,7 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl)
     // waves in flight) unless a block that holds all of K would then need more than 16 waves; K is split over
     // several blocks only when a single block cannot hold it or there would be too few blocks to cover the chip.
     const int64_t tiles = (int64_t)pl.GP * pl.RB;
-    const int max_waves = pl.MT == 1 ? 16 : 8; // wider batches need the registers and the LDS staging of a wave twice over
+    const int max_waves = pl.MT == 1 ? 16 : 8; // wider batches need more registers and LDS staging per wave
     int S = 1, BK = 1;
     int KS = pl.NS;
     if (KS * NL > max_waves && (pl.NS + 1) / 2 * NL <= max_waves) {
