@@ -48,12 +48,14 @@ static bool sliced_supported(const hqq_linear *l, int64_t M) { return M > kSmall
 
 static int pick_family(const hqq_linear *l, int64_t M)
 {
-    if (smallbatch_supported(l, M))
+    if (strip_supported(l, M)) // decode batches: part of the small-batch family
         return FAM_SMALLBATCH;
     if (vec3_supported(l, M))
         return FAM_VEC3;
-    if (tile_supported(l, M))
+    if (tile_supported(l, M)) // five rows and more: weights rebuilt once per batch tile on the matrix cores
         return FAM_TILE;
+    if (smallbatch_supported(l, M))
+        return FAM_SMALLBATCH;
     if (sliced_supported(l, M))
         return FAM_SMALLBATCH;
     return FAM_GENERAL;
@@ -65,6 +67,8 @@ static size_t family_workspace(const hqq_linear *l, int64_t M, int fam)
         return smallbatch_workspace_bytes(l, M > kSmallBatchMax ? kSmallBatchMax : M);
     if (fam == FAM_VEC3)
         return vec3_workspace_bytes(l, M);
+    if (fam == FAM_TILE)
+        return tile_workspace_bytes(l, M);
     return 0;
 }
 
@@ -88,7 +92,7 @@ static int run_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void
     case FAM_VEC3:
         return launch_vec3_matmul(l, x, M, y, ws, ws_bytes, s);
     case FAM_TILE:
-        return launch_tile_matmul(l, x, M, y, s);
+        return launch_tile_matmul(l, x, M, y, ws, ws_bytes, s);
     default:
         return launch_general_matmul(l, x, M, y, s);
     }
@@ -136,6 +140,9 @@ size_t hqq_matmul_workspace_bytes(const hqq_linear *l, int64_t M)
     const int64_t Ms = M > kSmallBatchMax ? kSmallBatchMax : M;
     size_t a = smallbatch_supported(l, Ms) ? 2 * smallbatch_workspace_bytes(l, Ms) : 0;
     size_t b = vec3_supported(l, M) ? vec3_workspace_bytes(l, M) : 0;
+    const size_t c = tile_supported(l, M) ? tile_workspace_bytes(l, M) : 0;
+    if (c > b)
+        b = c;
     return align256(a > b ? a : b);
 }
 
@@ -251,8 +258,10 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
     const f16 *x = (const f16 *)x_f16;
     f16 *y = (f16 *)y_f16;
 
-    const bool fast13 = smallbatch_supported(w1, M) && smallbatch_supported(w3, M) && !w1->bias && !w3->bias &&
-                        w1->nbits == w3->nbits && w1->group_size == w3->group_size;
+    // fused gate: decode batches always; wider ones only where the tile kernel does not take the shape
+    const bool prefer_tile = tile_supported(w1, M) && tile_supported(w3, M) && !strip_supported(w1, M);
+    const bool fast13 = !prefer_tile && smallbatch_supported(w1, M) && smallbatch_supported(w3, M) && !w1->bias &&
+                        !w3->bias && w1->nbits == w3->nbits && w1->group_size == w3->group_size;
     if (fast13) {
         rc = launch_smallbatch_gate_up(w1, w3, x, M, h, mm, mm_bytes, s);
         if (rc != HQQ_OK)
@@ -265,7 +274,7 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
         if ((rc = launch_silu_mul(a, b, h, M * w1->N, s)) != HQQ_OK)
             return rc;
     }
-    if (M <= kSmallBatchMax && smallbatch_supported(w2, M)) {
+    if (M <= kSmallBatchMax && smallbatch_supported(w2, M) && pick_family(w2, M) == FAM_SMALLBATCH) {
         SmallBatchEpilogue ep;
         ep.row_scale = (const f16 *)row_scale_f16;
         ep.accumulate = accumulate;

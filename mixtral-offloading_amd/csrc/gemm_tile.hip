@@ -29,7 +29,10 @@ struct TileParams {
     const f16 *x;
     const f16 *bias;
     f16 *y;
+    float *part; // [KSP][M][N] fp32 partial sums when K is split over several blocks, else null
     int M, N, K, GP, KT;
+    int KSP; // blocks along K
+    int KTS; // steps per block
 };
 
 template <int NBITS> struct WField {
@@ -53,7 +56,10 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile_kernel(TileParams p)
     __shared__ __attribute__((aligned(16))) f16 z_lds[kWaves][F * 2 * 4 * 8];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int jp = blockIdx.x * kWaves + wave;
+    const int jblk = blockIdx.x / p.KSP, ks = blockIdx.x - jblk * p.KSP;
+    const int jp = jblk * kWaves + wave;
+    const int s_begin = ks * p.KTS;
+    const int s_end = s_begin + p.KTS < p.KT ? s_begin + p.KTS : p.KT;
     const int rb = blockIdx.y;
     const int m0 = blockIdx.z * BM;
     const int K = p.K;
@@ -65,12 +71,12 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile_kernel(TileParams p)
     const uint8_t *cptr = p.codes + (size_t)prow * K + 16 * kg;
     TableCursor<0> sc, zr;
     {
-        const uint32_t c0 = (uint32_t)(F * jp + (tlane ? ti : 0)) * (uint32_t)K + (uint32_t)(4 * kq);
+        const uint32_t c0 = (uint32_t)(F * jp + (tlane ? ti : 0)) * (uint32_t)K + (uint32_t)(4 * kq) + (uint32_t)(s_begin * kStepK);
         sc.init(p.sc, c0, p.sc_inv);
         zr.init(p.zr, c0, p.zr_inv);
     }
     // x tile copy: thread t moves chunks (column m, k block kb) = (c / 8, c % 8) for c = t, t + 256, ...
-    constexpr int XCHUNKS = BM * 8 / (kWaves * 64);
+    constexpr int XCHUNKS = (BM * 8 + kWaves * 64 - 1) / (kWaves * 64);
 
     f32x4 acc[F][MB];
 #pragma unroll
@@ -97,23 +103,23 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile_kernel(TileParams p)
             const int m = m0 + ch / 8, kb = ch % 8;
             xr_n[c] = (u32x4){0, 0, 0, 0};
             // k block kb = h*4 + kg holds the columns half h of lane group kg works on: 16*kg + 8*h .. +7
-            if (m < p.M)
+            if (m < p.M && ch < BM * 8)
                 xr_n[c] = *reinterpret_cast<const u32x4 *>(p.x + (size_t)m * K + k0 + 16 * (kb & 3) + 8 * (kb >> 2));
         }
     };
-    issue(0);
+    issue(s_begin);
 
     f16 *s_w = &s_lds[wave][(((ti * 2 + ((kq >> 1) & 1)) * 4 + (kq >> 2)) * 8) + 4 * (kq & 1)];
     f16 *z_w = &z_lds[wave][(((ti * 2 + ((kq >> 1) & 1)) * 4 + (kq >> 2)) * 8) + 4 * (kq & 1)];
 
-    for (int s = 0; s < p.KT; ++s) {
+    for (int s = s_begin; s < s_end; ++s) {
         const u32x4 cw = cw_n;
         const TableRaw sraw = sraw_n, zraw = zraw_n;
         u32x4 xr[XCHUNKS];
 #pragma unroll
         for (int c = 0; c < XCHUNKS; ++c)
             xr[c] = xr_n[c];
-        if (s + 1 < p.KT)
+        if (s + 1 < s_end)
             issue(s + 1);
 
         __syncthreads(); // everyone is done reading the previous step's tiles
@@ -124,7 +130,8 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile_kernel(TileParams p)
             // eight columns (0..7) stored in B-operand order (0,2,1,3,4,6,5,7)
             const f16x8 v = __builtin_bit_cast(f16x8, xr[c]);
             const f16x8 o = {v[0], v[2], v[1], v[3], v[4], v[6], v[5], v[7]};
-            *reinterpret_cast<f16x8 *>(&x_lds[(kb * BM + m) * 8]) = o;
+            if (ch < BM * 8)
+                *reinterpret_cast<f16x8 *>(&x_lds[(kb * BM + m) * 8]) = o;
         }
         if (tlane) {
             f16x2 s01, s23, z01, z23;
@@ -178,6 +185,14 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile_kernel(TileParams p)
         for (int v = 0; v < 4; ++v) {
             const int r = 16 * rb + 4 * kg + v;
             const int64_t n = (int64_t)F * (jp + (int64_t)r * p.GP);
+            if (p.part) { // K is split over blocks: fp32 partial sums, added by the finishing kernel
+                float *dst = p.part + ((int64_t)ks * p.M + m) * p.N + n;
+                if constexpr (F == 4)
+                    *reinterpret_cast<f32x4 *>(dst) = (f32x4){acc[0][b][v], acc[1][b][v], acc[2][b][v], acc[3][b][v]};
+                else
+                    *reinterpret_cast<float2 *>(dst) = make_float2(acc[0][b][v], acc[1][b][v]);
+                continue;
+            }
             f16 o[F];
 #pragma unroll
             for (int i = 0; i < F; ++i) {
@@ -194,8 +209,31 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile_kernel(TileParams p)
     }
 }
 
+// y = cast(sum over the K blocks) (+ bias)
+__global__ __launch_bounds__(256) void tile_finish_kernel(const float *__restrict__ part, int KSP, int M, int N,
+                                                           const f16 *__restrict__ bias, f16 *__restrict__ y)
+{
+    const int64_t total = (int64_t)M * N / 4;
+    const int64_t stride = (int64_t)M * N;
+    for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+        const int64_t e = idx * 4;
+        f32x4 a = {0, 0, 0, 0};
+        for (int s = 0; s < KSP; ++s)
+            a += *reinterpret_cast<const f32x4 *>(part + s * stride + e);
+        f16x4 out;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            f16 v = (f16)a[t];
+            if (bias)
+                v = v + bias[(e + t) % N];
+            out[t] = v;
+        }
+        *reinterpret_cast<f16x4 *>(y + e) = out;
+    }
+}
+
 struct TilePlan {
-    int F, GP, RB, KT, BM;
+    int F, GP, RB, KT, BM, KSP, KTS;
 };
 
 bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl)
@@ -226,10 +264,21 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl)
     pl.GP = (int)(G / F);
     pl.RB = l->group_size / 16;
     pl.KT = (int)(l->K / kStepK);
-    // narrower batch tiles when there would otherwise be fewer blocks than compute units
-    const int64_t blocks64 = (int64_t)(pl.GP / kWaves) * pl.RB * ((M + 63) / 64);
-    pl.BM = (M <= 32 || blocks64 < 256) ? 32 : 64;
-    if ((M + pl.BM - 1) / pl.BM > 65535)
+    // batch tile: as wide as the batch up to 64 columns, so that every weight is rebuilt as few times as possible
+    pl.BM = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
+    const int64_t mtiles = (M + pl.BM - 1) / pl.BM;
+    if (mtiles > 65535)
+        return false;
+    // K is split over blocks until about two blocks per compute unit exist (partial sums go through the workspace)
+    const int64_t blocks = (int64_t)(pl.GP / kWaves) * pl.RB * mtiles;
+    int64_t ksp = (512 + blocks - 1) / blocks;
+    if (ksp > pl.KT / 4)
+        ksp = pl.KT / 4; // at least four steps per block
+    if (ksp < 1)
+        ksp = 1;
+    pl.KTS = (int)((pl.KT + ksp - 1) / ksp);
+    pl.KSP = (pl.KT + pl.KTS - 1) / pl.KTS;
+    if ((int64_t)(pl.GP / kWaves) * pl.KSP > 0x7fffffff)
         return false;
     return true;
 }
@@ -239,14 +288,25 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl)
 bool tile_supported(const hqq_linear *l, int64_t M)
 {
     TilePlan pl;
-    return M > 16 && make_plan(l, M, pl);
+    return M > 4 && make_plan(l, M, pl);
 }
 
-int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, hipStream_t s)
+size_t tile_workspace_bytes(const hqq_linear *l, int64_t M)
+{
+    TilePlan pl;
+    if (!make_plan(l, M, pl) || pl.KSP == 1)
+        return 0;
+    // the head of a workspace holds the arrival counters of the decode kernels: partial sums go behind it
+    return workspace_head_bytes() + (size_t)pl.KSP * (size_t)M * (size_t)l->N * sizeof(float);
+}
+
+int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s)
 {
     TilePlan pl;
     if (!make_plan(l, M, pl) || (reinterpret_cast<uintptr_t>(x) & 15u))
         return HQQ_E_UNSUPPORTED;
+    if (pl.KSP > 1 && (!ws || ws_bytes < tile_workspace_bytes(l, M)))
+        return HQQ_E_WORKSPACE;
     TileParams p = {};
     p.codes = static_cast<const uint8_t *>(l->codes);
     p.sc = make_table(l->scale), p.zr = make_table(l->zero);
@@ -254,18 +314,30 @@ int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, hip
     p.zr_inv = l->zero.meta_cols > 0 ? (uint32_t)(0xFFFFFFFFull / (uint64_t)l->zero.meta_cols) : 0;
     p.x = x, p.bias = static_cast<const f16 *>(l->bias), p.y = y;
     p.M = (int)M, p.N = (int)l->N, p.K = (int)l->K, p.GP = pl.GP, p.KT = pl.KT;
-    const dim3 grid((unsigned)(pl.GP / kWaves), (unsigned)pl.RB, (unsigned)((M + pl.BM - 1) / pl.BM));
+    p.KSP = pl.KSP, p.KTS = pl.KTS;
+    p.part = pl.KSP > 1 ? reinterpret_cast<float *>(static_cast<char *>(ws) + workspace_head_bytes()) : nullptr;
+    const dim3 grid((unsigned)(pl.GP / kWaves * pl.KSP), (unsigned)pl.RB, (unsigned)((M + pl.BM - 1) / pl.BM));
     if (l->nbits == 2) {
-        if (pl.BM == 32)
+        if (pl.BM == 16)
+            gemm_tile_kernel<2, 16><<<grid, kWaves * 64, 0, s>>>(p);
+        else if (pl.BM == 32)
             gemm_tile_kernel<2, 32><<<grid, kWaves * 64, 0, s>>>(p);
         else
             gemm_tile_kernel<2, 64><<<grid, kWaves * 64, 0, s>>>(p);
     } else {
-        if (pl.BM == 32)
+        if (pl.BM == 16)
+            gemm_tile_kernel<4, 16><<<grid, kWaves * 64, 0, s>>>(p);
+        else if (pl.BM == 32)
             gemm_tile_kernel<4, 32><<<grid, kWaves * 64, 0, s>>>(p);
         else
             gemm_tile_kernel<4, 64><<<grid, kWaves * 64, 0, s>>>(p);
     }
+    int rc = launch_status();
+    if (rc != HQQ_OK || pl.KSP == 1)
+        return rc;
+    const int64_t quads = M * l->N / 4;
+    const int fgrid = (int)(quads / 256 < 1 ? 1 : (quads / 256 > 4096 ? 4096 : quads / 256));
+    tile_finish_kernel<<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, p.bias, y);
     return launch_status();
 }
 
