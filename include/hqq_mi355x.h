@@ -123,6 +123,31 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
 int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, int64_t M, void *h_f16, void *workspace,
                 size_t workspace_bytes, void *stream);
 
+/* ---- expert FFN whose expert is chosen on the device: the same computation as hqq_expert_ffn, but the weights come
+ *      from record expert_index[0] of a device-resident table, so that the router's choice (src/custom_layers.py:
+ *      276-296: topk, then a host-side list of active experts) needs no host synchronisation when every expert of
+ *      the layer is resident.  The table holds 3 records per expert in the order w1, w3, w2, each
+ *      hqq_expert_record_bytes() long and written by hqq_expert_record_fill into HOST memory (the caller copies the
+ *      table to the device once).  w1 / w2 / w3 describe the common shape of all experts (any one expert's
+ *      descriptors).  Batches of at most 4 rows.  Workspace as for hqq_expert_ffn.                                  */
+size_t hqq_expert_record_bytes(void);
+int hqq_expert_record_fill(const hqq_linear *l, void *host_record);
+int hqq_expert_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *device_table,
+                           const int32_t *expert_index, const void *x_f16, int64_t M, void *y_f16,
+                           const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
+                           void *stream);
+
+/* ---- router of one token: logits = fp16(x W^T), fp32 softmax, the two largest probabilities renormalised and cast
+ *      to fp16 (src/custom_layers.py:276-282), written to device memory: sel_out[2] expert indices (largest
+ *      first), weights_f16_out[2]; logits_f16_out[n_experts] when not NULL.  n_experts <= 16.                       */
+int hqq_router_top2(const void *x_f16, const void *gate_w_f16, int32_t n_experts, int64_t hidden, int32_t *sel_out,
+                    void *weights_f16_out, void *logits_f16_out, void *stream);
+
+/* ---- residual add and RMSNorm of one token (the reference takes both from HF transformers' Mixtral decoder layer):
+ *      x += delta in fp16 when delta is not NULL (x is written back), y = weight * fp16(x * rsqrt(mean(x^2) + eps)). */
+int hqq_add_rmsnorm(void *x_f16, const void *delta_f16, const void *weight_f16, float eps, void *y_f16, int64_t hidden,
+                    void *stream);
+
 /* ---- which kernel family a call would use (for tests and profiles): 0 general, 1 MFMA small-batch, 2 MFMA tile,
  *      3 three-bit vector kernel.                                                                                     */
 int hqq_matmul_kernel_family(const hqq_linear *l, int64_t M);

@@ -287,4 +287,69 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
     return launch_scale_store(t, y, (const f16 *)row_scale_f16, accumulate, M, w2->N, s);
 }
 
+size_t hqq_expert_record_bytes(void) { return strip_record_bytes(); }
+
+int hqq_expert_record_fill(const hqq_linear *l, void *host_record)
+{
+    int rc = validate_linear(l);
+    if (rc != HQQ_OK)
+        return rc;
+    if (!host_record)
+        return HQQ_E_NULL;
+    if (!strip_supported(l, 1))
+        return HQQ_E_UNSUPPORTED;
+    strip_fill_record(host_record, l);
+    return HQQ_OK;
+}
+
+int hqq_expert_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *device_table,
+                           const int32_t *expert_index, const void *x_f16, int64_t M, void *y_f16,
+                           const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes, void *stream)
+{
+    int rc;
+    if ((rc = validate_linear(w1)) != HQQ_OK || (rc = validate_linear(w2)) != HQQ_OK ||
+        (rc = validate_linear(w3)) != HQQ_OK)
+        return rc;
+    if (M < 0 || w1->N != w3->N || w1->K != w3->K || w2->K != w1->N || w2->N != w1->K)
+        return HQQ_E_SHAPE;
+    if (M == 0)
+        return HQQ_OK;
+    if (!x_f16 || !y_f16 || !device_table || !expert_index)
+        return HQQ_E_NULL;
+    if (!strip_supported(w1, M) || !strip_supported(w3, M) || !strip_supported(w2, M))
+        return HQQ_E_UNSUPPORTED;
+    const size_t need = hqq_expert_ffn_workspace_bytes(w1, w2, w3, M);
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return HQQ_E_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    char *p = static_cast<char *>(workspace);
+    const size_t mm_bytes = ffn_matmul_scratch(w1, w2, w3, M);
+    f16 *h = (f16 *)(p + mm_bytes);
+    const StripIndex gate = {device_table, expert_index, 3, 0}, down = {device_table, expert_index, 3, 2};
+    if ((rc = launch_strip_gate_up(w1, w3, (const f16 *)x_f16, M, h, p, mm_bytes, s, &gate)) != HQQ_OK)
+        return rc;
+    SmallBatchEpilogue ep;
+    ep.row_scale = (const f16 *)row_scale_f16;
+    ep.accumulate = accumulate;
+    return launch_strip_matmul(w2, h, M, (f16 *)y_f16, p, mm_bytes, ep, s, &down);
+}
+
+int hqq_router_top2(const void *x_f16, const void *gate_w_f16, int32_t n_experts, int64_t hidden, int32_t *sel_out,
+                    void *weights_f16_out, void *logits_f16_out, void *stream)
+{
+    if (!x_f16 || !gate_w_f16 || !sel_out || !weights_f16_out)
+        return HQQ_E_NULL;
+    return launch_router_top2((const f16 *)x_f16, (const f16 *)gate_w_f16, n_experts, hidden, sel_out,
+                              (f16 *)weights_f16_out, (f16 *)logits_f16_out, (hipStream_t)stream);
+}
+
+int hqq_add_rmsnorm(void *x_f16, const void *delta_f16, const void *weight_f16, float eps, void *y_f16, int64_t hidden,
+                    void *stream)
+{
+    if (!x_f16 || !weight_f16 || !y_f16)
+        return HQQ_E_NULL;
+    return launch_add_rmsnorm((f16 *)x_f16, (const f16 *)delta_f16, (const f16 *)weight_f16, eps, (f16 *)y_f16, hidden,
+                              (hipStream_t)stream);
+}
+
 } // extern "C"

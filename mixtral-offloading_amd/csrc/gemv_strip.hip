@@ -33,11 +33,17 @@ struct StripLayer {
     const f16 *s_ms, *s_mz; // meta of the scale table
     const f16 *z_ms, *z_mz; // meta of the zero table
     uint32_t s_cols, z_cols, s_inv, z_inv;
-    float *part; // [BK][M][N]
 };
+static_assert(sizeof(StripLayer) == 72, "the record is read as 18 words");
 
 struct StripParams {
     StripLayer layer[2];
+    // Indexed launch (table != null): the layer records are read from a device table, record
+    // table[sel[0] * table_stride + table_first + layer], so that which expert runs is decided on the device.
+    const StripLayer *table;
+    const int *sel;
+    int table_stride, table_first;
+    float *part[2]; // [BK][M][N] per layer
     const f16 *x;
     int M, N, K;
     int GP, RB;
@@ -88,7 +94,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     const bool wave_on = wave < p.KS * p.NL;
     // both layer records come from the kernel arguments and are selected in registers: no dependent loads
     StripLayer L;
-    {
+    if (p.table) {
+        // one word of the record per lane, then broadcast: the record's address is known only now
+        const int e = __builtin_amdgcn_readfirstlane(p.sel[0]);
+        const uint32_t *src = reinterpret_cast<const uint32_t *>(p.table + (e * p.table_stride + p.table_first + layer));
+        const uint32_t word = src[lane < 18 ? lane : 0];
+        uint32_t rec[18];
+#pragma unroll
+        for (int i = 0; i < 18; ++i)
+            rec[i] = __builtin_amdgcn_readlane(word, i);
+        __builtin_memcpy(&L, rec, sizeof(L));
+    } else {
         const StripLayer &A = p.layer[0], &B = p.layer[1];
         L.codes = layer ? B.codes : A.codes;
         L.sq = layer ? B.sq : A.sq;
@@ -350,7 +366,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
         if (!alone) {
             // device-scope stores: written through the (per-XCD, mutually non-coherent) L2 so that the finishing
             // block, which may run on another XCD, can read them without any cache-wide flush
-            float *dst = (l_t ? p.layer[1].part : p.layer[0].part) + ((int64_t)kb * M + m_t) * p.N + n;
+            float *dst = (l_t ? p.part[1] : p.part[0]) + ((int64_t)kb * M + m_t) * p.N + n;
 #pragma unroll
             for (int i = 0; i < F; ++i)
                 __hip_atomic_store(dst + i, o[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -441,9 +457,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
             const int64_t off = ((int64_t)s * M + m_t) * p.N + n;
 #pragma unroll
             for (int i = 0; i < F; ++i) {
-                a[i] += __hip_atomic_load(p.layer[0].part + off + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                a[i] += __hip_atomic_load(p.part[0] + off + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if constexpr (EPI == 1)
-                    b[i] += __hip_atomic_load(p.layer[1].part + off + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    b[i] += __hip_atomic_load(p.part[1] + off + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
         f16 *dst = p.y + (int64_t)m_t * p.N + n;
@@ -543,7 +559,7 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl)
     return true;
 }
 
-void fill_layer(StripLayer &L, const hqq_linear *l, float *part)
+void fill_layer(StripLayer &L, const hqq_linear *l)
 {
     L.codes = static_cast<const uint8_t *>(l->codes);
     L.sq = static_cast<const uint8_t *>(l->scale.data);
@@ -556,7 +572,6 @@ void fill_layer(StripLayer &L, const hqq_linear *l, float *part)
     L.z_cols = (uint32_t)l->zero.meta_cols;
     L.s_inv = L.s_cols ? (uint32_t)(0xFFFFFFFFull / L.s_cols) : 0;
     L.z_inv = L.z_cols ? (uint32_t)(0xFFFFFFFFull / L.z_cols) : 0;
-    L.part = part;
 }
 
 template <int NBITS, int MT, int S, int D, int WAVES, int EPI>
@@ -601,8 +616,8 @@ template <int NBITS, int EPI> void launch_batch(const StripParams &p, const Stri
         launch_depth<NBITS, 4, EPI>(p, pl, grid, s);
 }
 
-int run(const hqq_linear *l0, const hqq_linear *l1, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
-        const SmallBatchEpilogue &ep, hipStream_t s)
+int run(const hqq_linear *l0, const hqq_linear *l1, const StripIndex *ix, const f16 *x, int64_t M, f16 *y, void *ws,
+        size_t ws_bytes, const SmallBatchEpilogue &ep, hipStream_t s)
 {
     StripPlan pl;
     const int NL = l1 ? 2 : 1;
@@ -614,11 +629,18 @@ int run(const hqq_linear *l0, const hqq_linear *l1, const f16 *x, int64_t M, f16
         return HQQ_E_WORKSPACE;
     StripParams p = {};
     char *base = static_cast<char *>(ws);
-    fill_layer(p.layer[0], l0, alone ? nullptr : reinterpret_cast<float *>(base + kCounterBytes));
+    fill_layer(p.layer[0], l0);
     if (l1)
-        fill_layer(p.layer[1], l1, alone ? nullptr : reinterpret_cast<float *>(base + kCounterBytes + one));
+        fill_layer(p.layer[1], l1);
     else
         p.layer[1] = p.layer[0];
+    p.part[0] = alone ? nullptr : reinterpret_cast<float *>(base + kCounterBytes);
+    p.part[1] = alone ? nullptr : reinterpret_cast<float *>(base + kCounterBytes + one);
+    if (ix) {
+        p.table = static_cast<const StripLayer *>(ix->table);
+        p.sel = ix->sel;
+        p.table_stride = ix->stride, p.table_first = ix->first;
+    }
     p.x = x, p.M = (int)M, p.N = (int)l0->N, p.K = (int)l0->K;
     p.GP = pl.GP, p.RB = pl.RB, p.NS = pl.NS, p.KS = pl.KS, p.BK = pl.BK, p.NL = NL;
     p.counter = reinterpret_cast<int *>(base);
@@ -656,19 +678,23 @@ size_t strip_workspace_bytes(const hqq_linear *l, int64_t M)
 }
 
 int launch_strip_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
-                        const SmallBatchEpilogue &ep, hipStream_t s)
+                        const SmallBatchEpilogue &ep, hipStream_t s, const StripIndex *ix)
 {
-    return run(l, nullptr, x, M, y, ws, ws_bytes, ep, s);
+    return run(l, nullptr, ix, x, M, y, ws, ws_bytes, ep, s);
 }
 
+size_t strip_record_bytes() { return sizeof(StripLayer); }
+
+void strip_fill_record(void *dst, const hqq_linear *l) { fill_layer(*static_cast<StripLayer *>(dst), l); }
+
 int launch_strip_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
-                         size_t ws_bytes, hipStream_t s)
+                         size_t ws_bytes, hipStream_t s, const StripIndex *ix)
 {
     StripPlan a, b;
     if (!make_plan(w1, M, 2, a) || !make_plan(w3, M, 2, b) || w1->N != w3->N || w1->K != w3->K || w1->nbits != w3->nbits ||
         w1->group_size != w3->group_size || a.SKIND != b.SKIND || a.ZKIND != b.ZKIND)
         return HQQ_E_UNSUPPORTED;
-    return run(w1, w3, x, M, h, ws, ws_bytes, SmallBatchEpilogue{}, s);
+    return run(w1, w3, ix, x, M, h, ws, ws_bytes, SmallBatchEpilogue{}, s);
 }
 
 int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s)

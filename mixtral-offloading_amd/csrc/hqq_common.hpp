@@ -102,10 +102,20 @@ int launch_smallbatch_gate_up(const hqq_linear *w1, const hqq_linear *w3, const 
 // slabs of 256 columns per wave, in-block gate epilogue
 bool strip_supported(const hqq_linear *l, int64_t M);
 size_t strip_workspace_bytes(const hqq_linear *l, int64_t M);
+// Indexed launch: the layer records come from a device table of strip_record_bytes() records, record
+// sel[0] * stride + first (+ 1 for the second projection of the gate); the descriptors passed alongside only give
+// the shape, which every record of the table must share.
+struct StripIndex {
+    const void *table;
+    const int *sel;
+    int stride, first;
+};
+size_t strip_record_bytes();
+void strip_fill_record(void *dst, const hqq_linear *l);
 int launch_strip_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
-                        const SmallBatchEpilogue &ep, hipStream_t s);
+                        const SmallBatchEpilogue &ep, hipStream_t s, const StripIndex *ix = nullptr);
 int launch_strip_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
-                         size_t ws_bytes, hipStream_t s);
+                         size_t ws_bytes, hipStream_t s, const StripIndex *ix = nullptr);
 int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s);
 size_t workspace_head_bytes();
 bool tile_supported(const hqq_linear *l, int64_t M);
@@ -114,6 +124,9 @@ int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, voi
 bool vec3_supported(const hqq_linear *l, int64_t M);
 size_t vec3_workspace_bytes(const hqq_linear *l, int64_t M);
 int launch_vec3_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s);
+int launch_router_top2(const f16 *x, const f16 *w, int n_experts, int64_t hidden, int *sel, f16 *weights, f16 *logits,
+                       hipStream_t s);
+int launch_add_rmsnorm(f16 *x, const f16 *delta, const f16 *weight, float eps, f16 *y, int64_t hidden, hipStream_t s);
 int launch_silu_mul(const f16 *a, const f16 *b, f16 *h, int64_t count, hipStream_t s);
 int launch_scale_store(const f16 *src, f16 *dst, const f16 *row_scale, int accumulate, int64_t M, int64_t N,
                        hipStream_t s);

@@ -53,6 +53,12 @@ _SIGNATURES = {
     "hqq_expert_ffn": (c_int, [_P(HqqLinear), _P(HqqLinear), _P(HqqLinear), c_void_p, c_int64, c_void_p, c_void_p,
                                c_int, c_void_p, c_size_t, c_void_p]),
     "hqq_gate_up": (c_int, [_P(HqqLinear), _P(HqqLinear), c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hqq_expert_record_bytes": (c_size_t, []),
+    "hqq_expert_record_fill": (c_int, [_P(HqqLinear), c_void_p]),
+    "hqq_expert_ffn_indexed": (c_int, [_P(HqqLinear), _P(HqqLinear), _P(HqqLinear), c_void_p, c_void_p, c_void_p, c_int64,
+                                       c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
+    "hqq_router_top2": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "hqq_add_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, ctypes.c_float, c_void_p, c_int64, c_void_p]),
     "hqq_slab_h2d_async": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
     "hqq_stream_wait_event": (c_int, [c_void_p, c_void_p]),
     "hqq_lru_create": (c_void_p, [c_int32, c_int32]),

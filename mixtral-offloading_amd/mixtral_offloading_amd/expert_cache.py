@@ -231,6 +231,20 @@ class ExpertCache:
             self.ready[slot].record(self.copy_stream)
         self.bytes_copied += self.module_size
 
+    def resident_group(self, eviction_group: int) -> Optional[List[MixtralExpertWrapper]]:
+        """The device modules of every expert of a group, in expert order, when all of them are resident and none
+        can be evicted (no expert of the cache is offloaded); else None."""
+        if self.n_offloaded > 0 or eviction_group not in self.group_infos:
+            return None
+        group = self.group_infos[eviction_group]
+        out = []
+        for info in group.members:
+            local = _lib.lib.hqq_lru_slot_of(group._lru, info.index)
+            if local < 0:
+                return None
+            out.append(self.slots[group.global_slot[local]])
+        return out
+
     # convenience counters (the reference keeps hits / misses per EvictionGroupInfo)
     def stats(self) -> Dict[str, int]:
         return {"hits": sum(g.hits for g in self.group_infos.values()),

@@ -195,3 +195,63 @@ def expert_ffn(w1: LinearDesc, w2: LinearDesc, w3: LinearDesc, x: torch.Tensor, 
                                            int(accumulate), ws.data_ptr(), ws.numel(),
                                            _lib.current_stream_ptr(x.device)), "hqq_expert_ffn")
     return out
+
+
+class ExpertTable:
+    """Device-resident table of the experts of one MoE layer for ``expert_ffn_indexed``: three records per expert
+    (w1, w3, w2).  ``experts`` is a list of (w1, w2, w3) ``LinearDesc`` triples that all share one shape."""
+
+    def __init__(self, experts):
+        rec = _lib.lib.hqq_expert_record_bytes()
+        host = (ctypes.c_uint8 * (rec * 3 * len(experts)))()
+        base = ctypes.addressof(host)
+        for e, (w1, w2, w3) in enumerate(experts):
+            for j, d in enumerate((w1, w3, w2)):
+                _lib.check(_lib.lib.hqq_expert_record_fill(d.ref, base + (3 * e + j) * rec), "hqq_expert_record_fill")
+        self.shape = experts[0]
+        self.device = experts[0][0].device
+        self.table = torch.frombuffer(host, dtype=torch.uint8).clone().to(self.device)
+        self._keep = list(experts)
+
+
+def expert_ffn_indexed(table: ExpertTable, expert_index: torch.Tensor, x: torch.Tensor, out: torch.Tensor,
+                       row_scale: Optional[torch.Tensor] = None, accumulate: bool = False) -> torch.Tensor:
+    """``expert_ffn`` of expert ``expert_index[0]`` (an int32 device tensor) of the table: no host synchronisation."""
+    w1, w2, w3 = table.shape
+    assert x.dtype == torch.float16 and x.is_contiguous() and x.shape[-1] == w1.K
+    assert expert_index.dtype == torch.int32 and expert_index.is_cuda
+    M = x.numel() // w1.K
+    assert out.is_contiguous() and out.numel() == M * w2.N and out.dtype == torch.float16
+    with torch.cuda.device(x.device):
+        need = _lib.lib.hqq_expert_ffn_workspace_bytes(w1.ref, w2.ref, w3.ref, M)
+        ws = workspace(x.device, need)
+        _lib.check(_lib.lib.hqq_expert_ffn_indexed(w1.ref, w2.ref, w3.ref, table.table.data_ptr(),
+                                                   expert_index.data_ptr(), x.data_ptr(), M, out.data_ptr(),
+                                                   row_scale.data_ptr() if row_scale is not None else None,
+                                                   int(accumulate), ws.data_ptr(), ws.numel(),
+                                                   _lib.current_stream_ptr(x.device)), "hqq_expert_ffn_indexed")
+    return out
+
+
+def router_top2(x: torch.Tensor, gate_weight: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
+                logits: Optional[torch.Tensor] = None) -> None:
+    """Router of one token into device tensors ``sel`` (int32[2]) and ``weights`` (fp16[2])
+    (reference src/custom_layers.py:276-282)."""
+    n_experts, hidden = gate_weight.shape
+    assert x.dtype == torch.float16 and gate_weight.dtype == torch.float16 and x.numel() == hidden
+    assert sel.dtype == torch.int32 and sel.numel() >= 2 and weights.dtype == torch.float16 and weights.numel() >= 2
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib.hqq_router_top2(x.data_ptr(), gate_weight.data_ptr(), n_experts, hidden, sel.data_ptr(),
+                                            weights.data_ptr(), logits.data_ptr() if logits is not None else None,
+                                            _lib.current_stream_ptr(x.device)), "hqq_router_top2")
+
+
+def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out: torch.Tensor) -> torch.Tensor:
+    """``x += delta`` (when given) then ``out = weight * rmsnorm(x)`` for one token."""
+    assert x.dtype == torch.float16 and x.is_contiguous() and out.dtype == torch.float16 and x.numel() == weight.numel()
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib.hqq_add_rmsnorm(x.data_ptr(), delta.data_ptr() if delta is not None else None,
+                                            weight.data_ptr(), float(eps), out.data_ptr(), x.numel(),
+                                            _lib.current_stream_ptr(x.device)), "hqq_add_rmsnorm")
+    return out

@@ -116,6 +116,115 @@ class MixtralModel(nn.Module):
         self.norm = RMSNorm(config.hidden_size, config.rms_norm_eps, device)
 
 
+class DecodeGraph:
+    """One batch-1 decode step of the whole model as a replayable HIP graph.
+
+    Usable when every expert of every layer is resident on the device: the router's choice then stays on the device
+    (``hip_kernels.router_top2`` writes the two expert indices, ``expert_ffn_indexed`` reads them), the position is a
+    device tensor, attention runs over the whole cache with the positions past the current one masked, and the next
+    token is written back into the step's own input -- nothing in a step waits for the host.  The reference drives
+    the same step from Python with one host synchronisation per MoE layer and two more per active expert
+    (src/custom_layers.py:292-302)."""
+
+    def __init__(self, model: "MixtralForCausalLM", max_len: int):
+        from . import hip_kernels
+
+        self.model, self.max_len = model, max_len
+        cfg, dev = model.config, model.device
+        self.tables = []
+        for layer_id, layer in enumerate(model.model.layers):
+            mods = layer.block_sparse_moe.experts.resident_group(layer_id)
+            if mods is None:
+                raise RuntimeError("the graph path needs every expert of every layer resident on the device")
+            self.tables.append(hip_kernels.ExpertTable(
+                [(m._expert[0].w1._desc(), m._expert[0].w2._desc(), m._expert[0].w3._desc()) for m in mods]))
+        self.cache = model.new_cache(max_len)
+        mk = dict(device=dev)
+        self.tok = torch.zeros(1, dtype=torch.int64, **mk)
+        self.pos = torch.zeros(1, dtype=torch.int64, **mk)
+        self.arange = torch.arange(max_len, **mk)
+        self.x = torch.zeros((1, cfg.hidden_size), dtype=torch.float16, **mk)
+        self.xn = torch.zeros_like(self.x)
+        self.moe = torch.zeros_like(self.x)
+        self.sel = torch.zeros(2, dtype=torch.int32, **mk)
+        self.rw = torch.zeros(2, dtype=torch.float16, **mk)
+        self.logits = torch.zeros((1, cfg.vocab_size), dtype=torch.float16, **mk)
+        self.graph = None
+
+    @torch.inference_mode()
+    def _step(self):
+        from . import hip_kernels
+
+        m, cfg = self.model, self.model.config
+        H, KV = cfg.num_attention_heads, cfg.num_key_value_heads
+        hd = cfg.hidden_size // H
+        g = H // KV
+        eps = cfg.rms_norm_eps
+        x = self.x
+        x.copy_(m.model.embed_tokens(self.tok))
+        cos = m.rotary.cos.index_select(0, self.pos)[:, None, :]
+        sin = m.rotary.sin.index_select(0, self.pos)[:, None, :]
+        future = (self.arange > self.pos)[None, None, :]
+        delta = None
+        for layer, (ck, cv), table in zip(m.model.layers, self.cache, self.tables):
+            attn = layer.self_attn
+            hip_kernels.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps, self.xn)
+            q = attn.q_proj(self.xn).view(1, H, hd)
+            k = attn.k_proj(self.xn).view(1, KV, hd)
+            v = attn.v_proj(self.xn).view(1, KV, hd)
+            q = q * cos + Rotary.rotate_half(q) * sin
+            k = k * cos + Rotary.rotate_half(k) * sin
+            ck.index_copy_(1, self.pos, k.transpose(0, 1))
+            cv.index_copy_(1, self.pos, v.transpose(0, 1))
+            qh = q.transpose(0, 1).reshape(KV, g, hd)
+            scores = torch.bmm(qh, ck.transpose(1, 2)).float() / math.sqrt(hd)
+            probs = torch.softmax(scores.masked_fill(future, float("-inf")), dim=-1).to(torch.float16)
+            out = torch.bmm(probs, cv).reshape(1, H * hd)
+            attn_out = attn.o_proj(out)
+            hip_kernels.add_rmsnorm(x, attn_out, layer.post_attention_layernorm.weight, eps, self.xn)
+            hip_kernels.router_top2(self.xn, layer.block_sparse_moe.gate.weight, self.sel, self.rw)
+            hip_kernels.expert_ffn_indexed(table, self.sel[0:1], self.xn, self.moe, row_scale=self.rw[0:1])
+            hip_kernels.expert_ffn_indexed(table, self.sel[1:2], self.xn, self.moe, row_scale=self.rw[1:2], accumulate=True)
+            delta = self.moe
+        hip_kernels.add_rmsnorm(x, delta, m.model.norm.weight, eps, self.xn)
+        self.logits.copy_(m.lm_head(self.xn))
+        self.tok.copy_(self.logits.argmax(-1))
+        self.pos.add_(1)
+
+    def capture(self):
+        """Warm up on a side stream (workspaces and allocator pools get their final size), then record the step."""
+        keep = (self.tok.clone(), self.pos.clone())
+        side = torch.cuda.Stream(device=self.model.device)
+        side.wait_stream(torch.cuda.current_stream(self.model.device))
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                self._step()
+        torch.cuda.current_stream(self.model.device).wait_stream(side)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self._step()
+        # the warm-up and the capture wrote cache entries at and after `pos`: every one is rewritten by the real
+        # steps before a query can see it (positions past the current one are masked)
+        self.tok.copy_(keep[0])
+        self.pos.copy_(keep[1])
+
+    @torch.inference_mode()
+    def prefill(self, prompt_ids: torch.Tensor) -> torch.Tensor:
+        """Runs the prompt through the eager path into this graph's cache; returns the first generated token."""
+        logits = self.model.forward(prompt_ids, self.cache, 0)
+        tok = logits[-1].argmax()
+        self.tok.copy_(tok.view(1))
+        self.pos.fill_(prompt_ids.numel())
+        return tok
+
+    def step(self):
+        """One decode step; afterwards ``self.tok`` holds the next token and ``self.logits`` its logits."""
+        if self.graph is None:
+            self._step()
+        else:
+            self.graph.replay()
+
+
 class MixtralForCausalLM(nn.Module):
     def __init__(self, config, device, max_positions: int = 4096):
         super().__init__()
@@ -142,6 +251,20 @@ class MixtralForCausalLM(nn.Module):
         for layer, (ck, cv) in zip(self.model.layers, cache):
             x = layer(x, self.rotary, ck, cv, start)
         return self.lm_head(self.model.norm(x))
+
+    @torch.inference_mode()
+    def generate_graph(self, prompt_ids: torch.Tensor, max_new_tokens: int, decode: Optional[DecodeGraph] = None):
+        """Greedy decoding, batch 1, with the decode steps replayed from a HIP graph (all experts resident)."""
+        total = prompt_ids.numel() + max_new_tokens + 2  # the warm-up of the capture writes two positions ahead
+        if decode is None or decode.max_len < total:
+            decode = DecodeGraph(self, total)
+        out = [decode.prefill(prompt_ids).view(1)]
+        if decode.graph is None:
+            decode.capture()
+        for _ in range(max_new_tokens - 1):
+            decode.step()
+            out.append(decode.tok.clone())
+        return torch.cat(out), decode
 
     @torch.inference_mode()
     def generate(self, prompt_ids: torch.Tensor, max_new_tokens: int, cache=None):
