@@ -352,4 +352,15 @@ int hqq_add_rmsnorm(void *x_f16, const void *delta_f16, const void *weight_f16, 
                               (hipStream_t)stream);
 }
 
+int hqq_attention_decode(const void *q_f16, const void *k_f16, const void *v_f16, const void *cos_f16, const void *sin_f16,
+                         const int64_t *pos, void *cache_k_f16, void *cache_v_f16, int64_t max_len, int32_t n_heads,
+                         int32_t n_kv_heads, int32_t head_dim, void *out_f16, void *stream)
+{
+    if (!q_f16 || !k_f16 || !v_f16 || !cos_f16 || !sin_f16 || !pos || !cache_k_f16 || !cache_v_f16 || !out_f16)
+        return HQQ_E_NULL;
+    return launch_attention_decode((const f16 *)q_f16, (const f16 *)k_f16, (const f16 *)v_f16, (const f16 *)cos_f16,
+                                   (const f16 *)sin_f16, pos, (f16 *)cache_k_f16, (f16 *)cache_v_f16, max_len, n_heads,
+                                   n_kv_heads, head_dim, (f16 *)out_f16, (hipStream_t)stream);
+}
+
 } // extern "C"

@@ -94,7 +94,124 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(f16 *__restrict__ x, c
     }
 }
 
+// Rotary embedding, KV-cache append and attention of ONE new token (the reference takes them from HF transformers'
+// Mixtral attention): one block per query head.  Roundings follow the fp16 torch ops they replace: rope terms
+// rounded separately, scores = fp16(q . k) then / sqrt(hd) in fp32, softmax in fp32, probabilities cast to fp16,
+// output accumulated in fp32.  The current position is read from device memory, so the launch can be replayed
+// from a graph; positions 0 .. pos are attended (the new key and value are taken from registers, and also
+// written to the cache by the first head of each KV group).
+template <int HD>
+__global__ __launch_bounds__(256) void attention_decode_kernel(const f16 *__restrict__ q_in, const f16 *__restrict__ k_in,
+                                                               const f16 *__restrict__ v_in, const f16 *__restrict__ cos_t,
+                                                               const f16 *__restrict__ sin_t, const int64_t *__restrict__ pos_p,
+                                                               f16 *__restrict__ cache_k, f16 *__restrict__ cache_v,
+                                                               int64_t max_len, int group, f16 *__restrict__ out)
+{
+    extern __shared__ float score_lds[]; // [pos + 1]
+    __shared__ __attribute__((aligned(16))) f16 q_lds[HD];
+    __shared__ __attribute__((aligned(16))) f16 k_lds[HD];
+    __shared__ float red_lds[8];
+    __shared__ float acc_lds[4][HD];
+    const int h = blockIdx.x, kv = h / group;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t pos = pos_p[0];
+    const f16 *cs = cos_t + pos * HD, *sn = sin_t + pos * HD;
+    if (tid < HD) {
+        const int d = tid, o = d < HD / 2 ? d + HD / 2 : d - HD / 2;
+        const f16 qa = q_in[h * HD + d], qb = q_in[h * HD + o];
+        const f16 ka = k_in[kv * HD + d], kb = k_in[kv * HD + o];
+        const f16 qr = d < HD / 2 ? -qb : qb, kr = d < HD / 2 ? -kb : kb;
+        const f16 qrot = (f16)(qa * cs[d]) + (f16)(qr * sn[d]);
+        const f16 krot = (f16)(ka * cs[d]) + (f16)(kr * sn[d]);
+        q_lds[d] = qrot;
+        k_lds[d] = krot;
+        if (h % group == 0) {
+            cache_k[((int64_t)kv * max_len + pos) * HD + d] = krot;
+            cache_v[((int64_t)kv * max_len + pos) * HD + d] = v_in[kv * HD + d];
+        }
+    }
+    __syncthreads();
+
+    // scores: one position per thread, the key row read as 16-byte pieces, q broadcast from LDS
+    const float inv = 1.0f / __builtin_sqrtf((float)HD);
+    float mx = -3.0e38f;
+    for (int64_t l = tid; l <= pos; l += 256) {
+        const f16 *krow = l == pos ? k_lds : cache_k + ((int64_t)kv * max_len + l) * HD;
+        float acc = 0.f;
+#pragma unroll
+        for (int c = 0; c < HD / 8; ++c) {
+            const f16x8 kk = *reinterpret_cast<const f16x8 *>(krow + 8 * c);
+            const f16x8 qq = *reinterpret_cast<const f16x8 *>(q_lds + 8 * c);
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                acc += (float)kk[t] * (float)qq[t];
+        }
+        const float sc = (float)(f16)acc * inv;
+        score_lds[l] = sc;
+        mx = fmaxf(mx, sc);
+    }
+    // block max
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1)
+        mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    if (lane == 0)
+        red_lds[wave] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red_lds[0], red_lds[1]), fmaxf(red_lds[2], red_lds[3]));
+    float sum = 0.f;
+    for (int64_t l = tid; l <= pos; l += 256) {
+        const float e = __expf(score_lds[l] - mx);
+        score_lds[l] = e;
+        sum += e;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0)
+        red_lds[4 + wave] = sum;
+    __syncthreads();
+    sum = red_lds[4] + red_lds[5] + red_lds[6] + red_lds[7];
+    const float rs = 1.0f / sum;
+
+    // output: wave w takes positions w, w+4, ...; lane owns HD/64 consecutive dimensions
+    constexpr int PER = HD / 64;
+    float o[PER];
+#pragma unroll
+    for (int t = 0; t < PER; ++t)
+        o[t] = 0.f;
+    for (int64_t l = wave; l <= pos; l += 4) {
+        const float pr = (float)(f16)(score_lds[l] * rs);
+        const f16 *vrow = l == pos ? v_in + kv * HD : cache_v + ((int64_t)kv * max_len + l) * HD;
+#pragma unroll
+        for (int t = 0; t < PER; ++t)
+            o[t] += pr * (float)vrow[lane * PER + t];
+    }
+#pragma unroll
+    for (int t = 0; t < PER; ++t)
+        acc_lds[wave][lane * PER + t] = o[t];
+    __syncthreads();
+    if (tid < HD)
+        out[h * HD + tid] = (f16)(acc_lds[0][tid] + acc_lds[1][tid] + acc_lds[2][tid] + acc_lds[3][tid]);
+}
+
 } // namespace
+
+int launch_attention_decode(const f16 *q, const f16 *k, const f16 *v, const f16 *cos_t, const f16 *sin_t, const int64_t *pos,
+                            f16 *cache_k, f16 *cache_v, int64_t max_len, int n_heads, int n_kv_heads, int head_dim, f16 *out,
+                            hipStream_t s)
+{
+    if (n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads != 0 || max_len < 1 || max_len > 16000)
+        return HQQ_E_SHAPE;
+    if (head_dim != 64 && head_dim != 128)
+        return HQQ_E_UNSUPPORTED;
+    if (!aligned16(cache_k) || !aligned16(cache_v))
+        return HQQ_E_ALIGN;
+    const size_t lds = (size_t)max_len * sizeof(float);
+    const int group = n_heads / n_kv_heads;
+    if (head_dim == 128)
+        attention_decode_kernel<128><<<n_heads, 256, lds, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len, group, out);
+    else
+        attention_decode_kernel<64><<<n_heads, 256, lds, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len, group, out);
+    return launch_status();
+}
 
 int launch_router_top2(const f16 *x, const f16 *w, int n_experts, int64_t hidden, int *sel, f16 *weights, f16 *logits,
                        hipStream_t s)

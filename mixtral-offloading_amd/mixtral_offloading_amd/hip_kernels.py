@@ -255,3 +255,19 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
                                             weight.data_ptr(), float(eps), out.data_ptr(), x.numel(),
                                             _lib.current_stream_ptr(x.device)), "hqq_add_rmsnorm")
     return out
+
+
+def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                     pos: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """Rope, cache append and attention of one new token; ``pos`` is an int64 device tensor with the position."""
+    n_kv, max_len, hd = cache_k.shape
+    n_heads = q.numel() // hd
+    assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous() and cache_k.is_contiguous() and cache_v.is_contiguous()
+    assert pos.dtype == torch.int64 and pos.is_cuda and cos.shape[-1] == hd and cos.is_contiguous() and sin.is_contiguous()
+    assert out.numel() == n_heads * hd and k.numel() == n_kv * hd == v.numel()
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.lib.hqq_attention_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+                                                 pos.data_ptr(), cache_k.data_ptr(), cache_v.data_ptr(), max_len, n_heads,
+                                                 n_kv, hd, out.data_ptr(), _lib.current_stream_ptr(q.device)),
+                   "hqq_attention_decode")
+    return out

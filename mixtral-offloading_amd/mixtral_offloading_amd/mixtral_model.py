@@ -146,6 +146,7 @@ class DecodeGraph:
         self.x = torch.zeros((1, cfg.hidden_size), dtype=torch.float16, **mk)
         self.xn = torch.zeros_like(self.x)
         self.moe = torch.zeros_like(self.x)
+        self.att = torch.zeros((1, cfg.num_attention_heads * (cfg.hidden_size // cfg.num_attention_heads)), dtype=torch.float16, **mk)
         self.sel = torch.zeros(2, dtype=torch.int32, **mk)
         self.rw = torch.zeros(2, dtype=torch.float16, **mk)
         self.logits = torch.zeros((1, cfg.vocab_size), dtype=torch.float16, **mk)
@@ -162,24 +163,14 @@ class DecodeGraph:
         eps = cfg.rms_norm_eps
         x = self.x
         x.copy_(m.model.embed_tokens(self.tok))
-        cos = m.rotary.cos.index_select(0, self.pos)[:, None, :]
-        sin = m.rotary.sin.index_select(0, self.pos)[:, None, :]
-        future = (self.arange > self.pos)[None, None, :]
         delta = None
         for layer, (ck, cv), table in zip(m.model.layers, self.cache, self.tables):
             attn = layer.self_attn
             hip_kernels.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps, self.xn)
-            q = attn.q_proj(self.xn).view(1, H, hd)
-            k = attn.k_proj(self.xn).view(1, KV, hd)
-            v = attn.v_proj(self.xn).view(1, KV, hd)
-            q = q * cos + Rotary.rotate_half(q) * sin
-            k = k * cos + Rotary.rotate_half(k) * sin
-            ck.index_copy_(1, self.pos, k.transpose(0, 1))
-            cv.index_copy_(1, self.pos, v.transpose(0, 1))
-            qh = q.transpose(0, 1).reshape(KV, g, hd)
-            scores = torch.bmm(qh, ck.transpose(1, 2)).float() / math.sqrt(hd)
-            probs = torch.softmax(scores.masked_fill(future, float("-inf")), dim=-1).to(torch.float16)
-            out = torch.bmm(probs, cv).reshape(1, H * hd)
+            q = attn.q_proj(self.xn)
+            k = attn.k_proj(self.xn)
+            v = attn.v_proj(self.xn)
+            out = hip_kernels.attention_decode(q, k, v, m.rotary.cos, m.rotary.sin, self.pos, ck, cv, self.att)
             attn_out = attn.o_proj(out)
             hip_kernels.add_rmsnorm(x, attn_out, layer.post_attention_layernorm.weight, eps, self.xn)
             hip_kernels.router_top2(self.xn, layer.block_sparse_moe.gate.weight, self.sel, self.rw)

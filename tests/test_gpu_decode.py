@@ -117,3 +117,35 @@ def test_graph_decode_refuses_offloaded_experts():
                            max_positions=64)
     with pytest.raises(RuntimeError):
         DecodeGraph(model, 32)
+
+
+@pytest.mark.parametrize("heads,kv,hd,pos", [(32, 8, 128, 0), (32, 8, 128, 37), (32, 8, 128, 511), (4, 2, 64, 5), (8, 8, 64, 300)])
+def test_attention_decode_against_torch_ops(heads, kv, hd, pos):
+    """Same roundings as the harness's torch attention (rope terms, fp16 scores, fp32 softmax, fp16 probabilities)."""
+    import math
+    from mixtral_offloading_amd import hip_kernels
+    from mixtral_offloading_amd.mixtral_model import Rotary
+    g = torch.Generator(device="cuda").manual_seed(heads + pos)
+    L = 512
+    rot = Rotary(hd, L, 1e6, torch.device("cuda"))
+    q = torch.randn((1, heads * hd), device="cuda", generator=g).half()
+    k = torch.randn((1, kv * hd), device="cuda", generator=g).half()
+    v = torch.randn((1, kv * hd), device="cuda", generator=g).half()
+    ck = torch.randn((kv, L, hd), device="cuda", generator=g).half()
+    cv = torch.randn((kv, L, hd), device="cuda", generator=g).half()
+    ck2, cv2 = ck.clone(), cv.clone()
+    # torch path (the harness's Attention.forward for T = 1)
+    positions = torch.tensor([pos], device="cuda")
+    qr, kr = rot.apply(q.view(1, heads, hd), k.view(1, kv, hd), positions)
+    ck[:, pos:pos + 1] = kr.transpose(0, 1)
+    cv[:, pos:pos + 1] = v.view(1, kv, hd).transpose(0, 1)
+    grp = heads // kv
+    qh = qr.transpose(0, 1).reshape(kv, grp, hd)
+    scores = torch.bmm(qh, ck[:, :pos + 1].transpose(1, 2)).float() / math.sqrt(hd)
+    probs = torch.softmax(scores, dim=-1).half()
+    want = torch.bmm(probs, cv[:, :pos + 1]).view(kv, grp, 1, hd).permute(2, 0, 1, 3).reshape(1, -1)
+    out = torch.empty((1, heads * hd), dtype=torch.float16, device="cuda")
+    hip_kernels.attention_decode(q, k, v, rot.cos, rot.sin, torch.tensor([pos], device="cuda"), ck2, cv2, out)
+    assert torch.equal(ck2, ck) and torch.equal(cv2, cv)  # the rotated key and the value landed in the cache, bit-exact
+    err = (out.float() - want.float()).abs().max()
+    assert float(err) <= 4e-3 * max(1.0, float(want.float().abs().max()))
