@@ -12,7 +12,11 @@ Prints ONE JSON line.  ``value`` is algorithmic bytes per step / time per step.
 ``roofline`` is the dominant kernel alone (the fused w1/w3 pass), timed with HIP
 events on the stream it is launched on.  ``cpu_baseline`` times the reference's
 PyTorch dequantise-then-matmul path (restated in oracle/torch_path.py) on the
-host cores for a bounded sample of the same steps."""
+host cores for a bounded sample of the same steps.  ``decode`` is the second half
+of the metric: greedy batch-1 decoding of the 32-layer random-init Mixtral-8x7B
+(attention 4-bit g64, experts 2-bit g16) from a 64-token random prompt, with every
+expert resident (graph-replayed and eager) and with a per-layer expert cache of 4
+and 2 slots fed by pinned host-to-device copies on a side stream."""
 from __future__ import annotations
 
 import argparse
@@ -91,6 +95,64 @@ def cpu_baseline(budget_s=15.0):
                       f"meta expansion + dequantize + matmul per call as the reference does"}
 
 
+def decode_section(dev, tokens_resident=256, tokens_offload=48):
+    """Tokens per second of the whole model (BASELINE configs[4]); every figure is measured between synchronisations
+    around the decode loop, prompt processing excluded."""
+    import gc
+
+    import torch
+
+    from mixtral_offloading_amd import build_model as bm
+    from mixtral_offloading_amd.mixtral_model import DecodeGraph
+
+    out = {"model": "Mixtral-8x7B architecture, 32 layers, random-init, attention 4-bit g64, experts 2-bit g16, "
+                    "64-token prompt, greedy, batch 1"}
+    cfg = bm.mixtral_config()
+    gen = torch.Generator(device=dev).manual_seed(1)
+    prompt = torch.randint(0, cfg.vocab_size, (64,), device=dev, generator=gen)
+
+    def timed_eager(model, n):
+        cache = model.new_cache(64 + n + 1)
+        tok = model.forward(prompt, cache, 0)[-1].argmax()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n):
+            tok = model.forward(tok.view(1), cache, 64 + i)[-1].argmax()
+        torch.cuda.synchronize()
+        return n / (time.perf_counter() - t0)
+
+    for per_layer in (8, 4, 2):
+        off = bm.OffloadConfig(main_size=32 * per_layer, offload_size=32 * (8 - per_layer), buffer_size=4,
+                               offload_per_layer=8 - per_layer)
+        model = bm.build_model(dev, bm.default_quant_config(), off, model_config=cfg, seed=0, max_positions=512)
+        model.generate(prompt, 2)  # workspaces, allocator pools
+        if per_layer == 8:
+            dec = DecodeGraph(model, 64 + tokens_resident + 4)
+            dec.prefill(prompt)
+            dec.capture()
+            dec.prefill(prompt)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(tokens_resident):
+                dec.step()
+            torch.cuda.synchronize()
+            out["all_experts_resident_graph_tok_s"] = round(tokens_resident / (time.perf_counter() - t0), 1)
+            out["all_experts_resident_graph_tokens"] = tokens_resident
+            del dec
+            out["all_experts_resident_eager_tok_s"] = round(timed_eager(model, 48), 1)
+        else:
+            before = model.expert_cache.stats()
+            out[f"expert_cache_{per_layer}_per_layer_tok_s"] = round(timed_eager(model, tokens_offload), 2)
+            st = model.expert_cache.stats()
+            out[f"expert_cache_{per_layer}_per_layer_detail"] = {
+                "tokens": tokens_offload, "hits": st["hits"] - before["hits"], "misses": st["misses"] - before["misses"],
+                "GB_copied_host_to_device": round((st["bytes_copied"] - before["bytes_copied"]) / 1e9, 2)}
+        del model
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -99,6 +161,7 @@ def main():
     ap.add_argument("--batch", type=int, default=1, help="tokens per step (1 is the headline; 4 and 16 are parity-test sizes)")
     ap.add_argument("--experts", type=int, default=8, help="distinct experts the steps rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-decode", action="store_true", help="skip the whole-model decode section")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain 256 MiB device copies, so that a counter run can scale FETCH_SIZE / WRITE_SIZE "
                          "by what the same counters read for a copy of known size")
@@ -179,13 +242,17 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this command, scaled by a
-                     # 256 MiB copy (profiles/gemv_slab_kernel_ffn_2bit_g16_m1.txt); measured at batch 1 only
-                     "traffic": 46793113 if m == 1 else None,
-                     "kernel": "gemv_slab_kernel<2,1,16,1,2,1> as launched by hqq_gate_up (w1 and w3 in one grid, one launch)",
+                     # 256 MiB copy (profiles/gemv_strip_kernel_ffn_2bit_g16_m1.txt); measured at batch 1 only
+                     "traffic": 46231757 if m == 1 else None,
+                     "kernel": "gemv_strip_kernel<2,1,2,2,16,1,2,1> as launched by hqq_gate_up (w1 and w3 in one grid, one launch)",
                      "bytes_per_launch": gate_up_bytes(m), "us_per_launch": round(ms_gate * 1e3, 3)},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+    if not args.no_decode:
+        del experts, descs
+        torch.cuda.empty_cache()
+        out["decode"] = decode_section(dev)
     print(json.dumps(out))
 
 
