@@ -95,6 +95,99 @@ def cpu_baseline(budget_s=15.0):
                       f"meta expansion + dequantize + matmul per call as the reference does"}
 
 
+def random_desc(nbits, n, k, gs, seed, dev):
+    """Random codes and 8-bit tables of one layer in the kernel layout, built on the GPU (their values do not
+    change the speed of any kernel)."""
+    import torch
+
+    from mixtral_offloading_amd import hip_kernels, packing
+
+    g = torch.Generator(device=dev).manual_seed(seed)
+    s_cnt = n * k // gs
+    q = torch.randint(0, 2 ** nbits, (n, k), dtype=torch.uint8, device=dev, generator=g)
+    pack = {4: packing.pack_4bit_u8_common, 2: packing.pack_2bit_u8_common, 3: packing.pack_3bit_i32_common}[nbits]
+    step = 0.07 / (2 ** nbits - 1)
+    meta = {"nbits": nbits, "group_size": gs, "shape": (n, k), "quant_scale": True, "quant_zero": True,
+            "scale_q": torch.randint(0, 256, (128, s_cnt // 128), dtype=torch.uint8, device=dev, generator=g),
+            "meta_scale": {"scale": torch.full((1, s_cnt // 128), step / 255, device=dev).half(),
+                           "zero": torch.full((1, s_cnt // 128), -128.0, device=dev).half()},
+            "zero_q": torch.randint(0, 256, (1, s_cnt), dtype=torch.uint8, device=dev, generator=g),
+            "meta_zero": {"scale": torch.tensor([(2 ** nbits - 1) / 255.0], device=dev).half(),
+                          "zero": torch.tensor([0.0], device=dev).half()}}
+    return hip_kernels.LinearDesc(pack(q), meta), q
+
+
+def survey_section(dev):
+    """Every kernel of the path at the BASELINE shapes: microseconds per launch by HIP events (cache-cold: each
+    timing rotates over more than 256 MB of distinct inputs) and the rate that follows from its algorithmic bytes."""
+    import torch
+
+    from mixtral_offloading_amd import _lib, hip_kernels, packing
+
+    lib = _lib.lib
+    stream = torch.cuda.Stream(device=dev)
+    rows = []
+
+    def timed(fn, iters):
+        with torch.cuda.stream(stream):
+            for i in range(max(4, iters // 4)):
+                fn(i)
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for i in range(iters):
+                fn(i)
+            e1.record(stream)
+            stream.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / iters
+
+    def add(name, us, nbytes, flops=None):
+        r = {"kernel": name, "us": round(us, 2), "GB_s": round(nbytes / us / 1e3, 0), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)}
+        if flops:
+            r["TFLOP_s"] = round(flops / us / 1e6, 1)
+        rows.append(r)
+        print(f"{name:58s} {us:9.2f} us {r['GB_s']:8.0f} GB/s" + (f" {r['TFLOP_s']:8.1f} TFLOP/s" if flops else ""), file=sys.stderr, flush=True)
+
+    shapes = [(4, 4096, 4096, 64, (1, 4, 16, 128)), (4, 1024, 4096, 64, (1,)), (2, 14336, 4096, 16, (1, 4, 16, 128)),
+              (2, 4096, 14336, 16, (1, 4, 16, 128)), (3, 14336, 4096, 64, (1, 8)), (3, 4096, 14336, 64, (1, 8))]
+    for nbits, n, k, gs, batches in shapes:
+        wbytes = (n * k * nbits // 8 if nbits != 3 else ((n + 9) // 10) * k * 4) + 2 * (n * k // gs) + 4 * (n * k // gs // META_GROUP) + 4
+        nl = max(2, min(16, (320 << 20) // wbytes + 1))
+        layers, codes = [], []
+        for i in range(nl):
+            d, q = random_desc(nbits, n, k, gs, 100 * nbits + i, dev)
+            layers.append(d)
+            if i < 4:
+                codes.append(q)
+        tag = f"w{nbits} {n}x{k} g{gs}"
+        with torch.cuda.stream(stream):
+            # packers and the de-quantiser (one-time work at load, streaming kernels)
+            pk = {4: (packing.pack_4bit_u8_common, packing.unpack_4bit_u8_common), 2: (packing.pack_2bit_u8_common, packing.unpack_2bit_u8_common),
+                  3: (packing.pack_3bit_i32_common, packing.unpack_3bit_i32_common)}[nbits]
+            packed = [pk[0](c) for c in codes]
+        cbytes = packed[0].numel() * packed[0].element_size()
+        add(f"pack   {tag}", timed(lambda i: pk[0](codes[i % 4]), 12), n * k + cbytes)
+        add(f"unpack {tag}", timed(lambda i: pk[1](packed[i % 4]), 12), n * k + cbytes)
+        add(f"dequantize {tag}", timed(lambda i: hip_kernels.dequantize(layers[i % nl]), 12), wbytes + 2 * n * k)
+        del codes, packed
+        for m in batches:
+            x = torch.randn((m, k), device=dev).half()
+            y = torch.empty((m, n), device=dev, dtype=torch.float16)
+            need = lib.hqq_matmul_workspace_bytes(layers[0].ref, m)
+            ws = torch.zeros(max(int(need), 256), dtype=torch.uint8, device=dev)
+
+            def f(i):
+                rc = lib.hqq_matmul_transpose(layers[i % nl].ref, x.data_ptr(), m, y.data_ptr(), ws.data_ptr(), ws.numel(), stream.cuda_stream)
+                if rc != 0:
+                    raise _lib.HqqError(rc, "hqq_matmul_transpose")
+
+            fam = lib.hqq_matmul_kernel_family(layers[0].ref, m)
+            add(f"matmul {tag} M={m} (family {fam})", timed(f, 48 if m <= 16 else 16), wbytes + 2 * m * (n + k), 2.0 * m * n * k)
+        del layers
+        torch.cuda.empty_cache()
+    return rows
+
+
 def decode_section(dev, tokens_resident=256, tokens_offload=48):
     """Tokens per second of the whole model (BASELINE configs[4]); every figure is measured between synchronisations
     around the decode loop, prompt processing excluded."""
@@ -162,6 +255,9 @@ def main():
     ap.add_argument("--experts", type=int, default=8, help="distinct experts the steps rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the whole-model decode section")
+    ap.add_argument("--survey", action="store_true",
+                    help="also time every kernel of the path (packers, de-quantiser, 2/3/4-bit matmuls at the BASELINE "
+                         "shapes and batches) and add the table as 'kernels'")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain 256 MiB device copies, so that a counter run can scale FETCH_SIZE / WRITE_SIZE "
                          "by what the same counters read for a copy of known size")
@@ -249,6 +345,8 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+    if args.survey:
+        out["kernels"] = survey_section(dev)
     if not args.no_decode:
         del experts, descs
         torch.cuda.empty_cache()

@@ -4,6 +4,7 @@
 // 32-bit or 128-bit words and does its bit work on four codes per lane-op.
 // Layouts follow the reference packers (src/packing.py:10-97).
 #include "hqq_common.hpp"
+#include "table_reader.hpp"
 
 namespace hqq {
 namespace {
@@ -182,6 +183,62 @@ __global__ __launch_bounds__(kThreads) void dequantize_kernel(const void *__rest
     }
 }
 
+// The same values for the usual shapes, moving whole words: one thread owns four columns of one packed row, turns
+// the row's codes into fp16 with byte permutes (0x6400 | b is 1024 + b), reads four entries of each table per
+// weight row and stores four halves per weight row.  Needs K % 4 == 0, G*K < 2^32 and, for 8-bit tables with
+// per-column meta, meta_cols % 4 == 0 (a chunk of four columns then never wraps).
+template <int NBITS, int SKIND, int ZKIND>
+__global__ __launch_bounds__(kThreads) void dequantize_words_kernel(const void *__restrict__ codes, Table sc, Table zr,
+                                                                    uint32_t sc_inv, uint32_t zr_inv, uint32_t N,
+                                                                    uint32_t K, uint32_t G, f16 *__restrict__ w)
+{
+    constexpr uint32_t F = NBITS == 3 ? 10 : 8 / NBITS;
+    const uint32_t prows = (N + F - 1) / F;
+    const uint32_t kchunks = K / 4;
+    const uint32_t total = prows * kchunks;
+    const f16x2 k1024 = {(f16)1024.0f, (f16)1024.0f};
+    for (uint32_t idx = blockIdx.x * kThreads + threadIdx.x; idx < total; idx += gridDim.x * kThreads) {
+        const uint32_t p = idx / kchunks, k0 = (idx - p * kchunks) * 4;
+        u32x4 w3 = {0, 0, 0, 0};
+        uint32_t w8 = 0;
+        if constexpr (NBITS == 3)
+            w3 = *reinterpret_cast<const u32x4 *>(static_cast<const uint32_t *>(codes) + (size_t)p * K + k0);
+        else
+            w8 = *reinterpret_cast<const uint32_t *>(static_cast<const uint8_t *>(codes) + (size_t)p * K + k0);
+        uint32_t j = (F * p) % G;
+#pragma unroll
+        for (uint32_t i = 0; i < F; ++i) {
+            const uint32_t n = F * p + i;
+            if (n >= N)
+                break;
+            TableCursor<SKIND> cs;
+            TableCursor<ZKIND> cz;
+            cs.init(sc, j * K + k0, sc_inv);
+            cz.init(zr, j * K + k0, zr_inv);
+            f16x2 s01, s23, z01, z23;
+            table_decode(cs, table_load(cs), s01, s23);
+            table_decode(cz, table_load(cz), z01, z23);
+            uint32_t b; // the four codes of row n, one per byte
+            if constexpr (NBITS == 3) {
+                const uint32_t sh = 3 * (9 - i);
+                b = ((w3.x >> sh) & 7u) | (((w3.y >> sh) & 7u) << 8) | (((w3.z >> sh) & 7u) << 16) |
+                    (((w3.w >> sh) & 7u) << 24);
+            } else {
+                b = (w8 >> (NBITS * (F - 1 - i))) & ((1u << NBITS) - 1) * 0x01010101u;
+            }
+            const f16x2 q01 = as_f16x2(__builtin_amdgcn_perm(0x64646464u, b, 0x04010400u)) - k1024;
+            const f16x2 q23 = as_f16x2(__builtin_amdgcn_perm(0x64646464u, b, 0x04030402u)) - k1024;
+            const f16x2 d01 = q01 - z01, d23 = q23 - z23; // first rounding
+            u32x2 o;
+            o.x = __builtin_bit_cast(uint32_t, d01 * s01); // second rounding
+            o.y = __builtin_bit_cast(uint32_t, d23 * s23);
+            *reinterpret_cast<u32x2 *>(w + (size_t)n * K + k0) = o;
+            if (++j == G)
+                j = 0;
+        }
+    }
+}
+
 // ------------------------------------------------------- small elementwise
 __global__ __launch_bounds__(kThreads) void silu_mul_kernel(const f16 *__restrict__ a, const f16 *__restrict__ b,
                                                             f16 *__restrict__ h, int64_t count)
@@ -247,6 +304,66 @@ int pack_u8(const uint8_t *q, int64_t rows, int64_t cols, uint8_t *out, hipStrea
     else
         pack_u8_kernel<NBITS, uint8_t><<<grid_for(prows * cols), kThreads, 0, s>>>(q, prows, cols, out);
     return launch_status();
+}
+
+// table kinds of TableCursor: 1 u8 with per-column meta, 2 u8 with scalar meta, 3 fp16; 0 = not a word-path table
+inline int words_table_kind(const hqq_table &t)
+{
+    if (t.kind == HQQ_TABLE_F16)
+        return aligned16(t.data) ? 3 : 0;
+    if ((reinterpret_cast<uintptr_t>(t.data) & 3u) != 0)
+        return 0;
+    if (t.meta_cols == 1)
+        return 2;
+    const bool meta_ok = (reinterpret_cast<uintptr_t>(t.meta_scale) & 7u) == 0 && (reinterpret_cast<uintptr_t>(t.meta_zero) & 7u) == 0;
+    return t.meta_cols % 4 == 0 && meta_ok ? 1 : 0;
+}
+
+template <int NBITS, int SKIND>
+void dequantize_words_z(int zk, int grid, const hqq_linear *l, const Table &sc, const Table &zr, uint32_t si, uint32_t zi,
+                        uint32_t G, f16 *w, hipStream_t s)
+{
+    const uint32_t N = (uint32_t)l->N, K = (uint32_t)l->K;
+    if (zk == 1)
+        dequantize_words_kernel<NBITS, SKIND, 1><<<grid, kThreads, 0, s>>>(l->codes, sc, zr, si, zi, N, K, G, w);
+    else if (zk == 2)
+        dequantize_words_kernel<NBITS, SKIND, 2><<<grid, kThreads, 0, s>>>(l->codes, sc, zr, si, zi, N, K, G, w);
+    else
+        dequantize_words_kernel<NBITS, SKIND, 3><<<grid, kThreads, 0, s>>>(l->codes, sc, zr, si, zi, N, K, G, w);
+}
+
+template <int NBITS>
+void dequantize_words_s(int sk, int zk, int grid, const hqq_linear *l, const Table &sc, const Table &zr, uint32_t si,
+                        uint32_t zi, uint32_t G, f16 *w, hipStream_t s)
+{
+    if (sk == 1)
+        dequantize_words_z<NBITS, 1>(zk, grid, l, sc, zr, si, zi, G, w, s);
+    else if (sk == 2)
+        dequantize_words_z<NBITS, 2>(zk, grid, l, sc, zr, si, zi, G, w, s);
+    else
+        dequantize_words_z<NBITS, 3>(zk, grid, l, sc, zr, si, zi, G, w, s);
+}
+
+// launches the word-path de-quantiser when the layer fits it; false = the caller takes the per-element kernel
+bool dequantize_words(const hqq_linear *l, const Table &sc, const Table &zr, f16 *w, hipStream_t s)
+{
+    const int sk = words_table_kind(l->scale), zk = words_table_kind(l->zero);
+    const int64_t G = l->N / l->group_size;
+    const int F = l->nbits == 3 ? 10 : 8 / l->nbits;
+    const int64_t prows = (l->N + F - 1) / F;
+    if (!sk || !zk || l->K % 4 != 0 || G * l->K >= (1ll << 32) || prows * (l->K / 4) >= (1ll << 31) ||
+        (reinterpret_cast<uintptr_t>(w) & 7u) != 0 || !aligned16(l->codes))
+        return false;
+    const uint32_t si = l->scale.meta_cols > 0 ? (uint32_t)(0xFFFFFFFFull / (uint64_t)l->scale.meta_cols) : 0;
+    const uint32_t zi = l->zero.meta_cols > 0 ? (uint32_t)(0xFFFFFFFFull / (uint64_t)l->zero.meta_cols) : 0;
+    const int grid = grid_for(prows * (l->K / 4));
+    if (l->nbits == 4)
+        dequantize_words_s<4>(sk, zk, grid, l, sc, zr, si, zi, (uint32_t)G, w, s);
+    else if (l->nbits == 2)
+        dequantize_words_s<2>(sk, zk, grid, l, sc, zr, si, zi, (uint32_t)G, w, s);
+    else
+        dequantize_words_s<3>(sk, zk, grid, l, sc, zr, si, zi, (uint32_t)G, w, s);
+    return true;
 }
 
 } // namespace
@@ -350,6 +467,8 @@ int hqq_dequantize(const hqq_linear *l, void *w_out_f16, void *stream)
     const int64_t total = ((l->N + F - 1) / F) * ((l->K + 3) / 4);
     hipStream_t s = (hipStream_t)stream;
     const Table sc = make_table(l->scale), zr = make_table(l->zero);
+    if (dequantize_words(l, sc, zr, (f16 *)w_out_f16, s))
+        return launch_status();
     if (l->nbits == 4)
         dequantize_kernel<4><<<grid_for(total), kThreads, 0, s>>>(l->codes, sc, zr, l->N, l->K, G, (f16 *)w_out_f16);
     else if (l->nbits == 2)
