@@ -137,6 +137,30 @@ int hqq_expert_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq
                            const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
                            void *stream);
 
+/* ---- both experts of one token in two launches instead of four: y (+)= sum over e < 2 of
+ *      fp16(FFN_{expert_index[e]}(x)) * row_scale[e], the loop body of src/custom_layers.py:298-312 for the two
+ *      active experts of a single token, each product and the sum rounded to fp16 as index_add_ on fp16 tensors
+ *      rounds them (what two hqq_expert_ffn_indexed calls give, the second accumulating, up to the order in which the
+ *      fp32 partial sums over K are added).  One launch
+ *      computes silu(w1 x) * w3 x of both experts, one both down projections and their weighted sum.  x is one row
+ *      (hidden fp16), expert_index two device int32, row_scale two device fp16.  Table as for
+ *      hqq_expert_ffn_indexed.  HQQ_E_UNSUPPORTED when the shapes do not fit the decode kernel (the workspace query
+ *      then returns 0): call hqq_expert_ffn_indexed twice instead.                                                 */
+size_t hqq_expert_pair_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3);
+int hqq_expert_pair_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3,
+                                const void *device_table, const int32_t *expert_index, const void *x_f16, void *y_f16,
+                                const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
+                                void *stream);
+
+/* ---- up to four HQQLinearTritonSavable.forward_triton calls (src/custom_layers.py:100-118) on the same single row
+ *      in one launch: ys[i] = x @ dequant(layers[i]).T (+ bias).  The layers share K, code width, group size and
+ *      table kinds but not N -- the q, k and v projections of an attention block.  Results are those of
+ *      hqq_matmul_transpose on each layer up to the order in which the fp32 partial sums over K are added.  HQQ_E_UNSUPPORTED (workspace query 0) when the layers do not fit: call
+ *      hqq_matmul_transpose per layer instead.                                                                      */
+size_t hqq_matmul_group_workspace_bytes(const hqq_linear *const *layers, int32_t count);
+int hqq_matmul_group(const hqq_linear *const *layers, int32_t count, const void *x_f16, void *const *ys_f16,
+                     void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- router of one token: logits = fp16(x W^T), fp32 softmax, the two largest probabilities renormalised and cast
  *      to fp16 (src/custom_layers.py:276-282), written to device memory: sel_out[2] expert indices (largest
  *      first), weights_f16_out[2]; logits_f16_out[n_experts] when not NULL.  n_experts <= 16.                       */
@@ -147,6 +171,13 @@ int hqq_router_top2(const void *x_f16, const void *gate_w_f16, int32_t n_experts
  *      x += delta in fp16 when delta is not NULL (x is written back), y = weight * fp16(x * rsqrt(mean(x^2) + eps)). */
 int hqq_add_rmsnorm(void *x_f16, const void *delta_f16, const void *weight_f16, float eps, void *y_f16, int64_t hidden,
                     void *stream);
+
+/* ---- hqq_add_rmsnorm followed by hqq_router_top2 on its output y, in one launch: the post-attention norm of a
+ *      decoder layer and the router that reads it (src/custom_layers.py:276-282).  x and y as hqq_add_rmsnorm gives
+ *      them; logits as hqq_router_top2 up to the order of the fp32 sums.                                           */
+int hqq_add_rmsnorm_router(void *x_f16, const void *delta_f16, const void *weight_f16, float eps, void *y_f16,
+                           int64_t hidden, const void *gate_w_f16, int32_t n_experts, int32_t *sel_out,
+                           void *weights_f16_out, void *logits_f16_out, void *stream);
 
 /* ---- rotary embedding, KV-cache append and attention of one new token (HF transformers' Mixtral attention in the
  *      reference): q (n_heads*head_dim), k and v (n_kv_heads*head_dim) are the un-rotated projections of the token;

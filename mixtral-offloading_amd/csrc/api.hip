@@ -334,6 +334,89 @@ int hqq_expert_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq
     return launch_strip_matmul(w2, h, M, (f16 *)y_f16, p, mm_bytes, ep, s, &down);
 }
 
+// workspace of the two-expert step: [strip scratch, counters first][h of expert 0][h of expert 1]
+static size_t pair_scratch(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3)
+{
+    const hqq_linear *gate[4] = {w1, w3, w1, w3}, *down[2] = {w2, w2};
+    const size_t a = strip_job_workspace_bytes(gate, 4, 2, 1), b = strip_job_workspace_bytes(down, 2, 2, 1);
+    if (a == 0 || b == 0)
+        return 0;
+    return align256(a > b ? a : b);
+}
+
+size_t hqq_expert_pair_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3)
+{
+    if (validate_linear(w1) != HQQ_OK || validate_linear(w2) != HQQ_OK || validate_linear(w3) != HQQ_OK)
+        return 0;
+    const size_t mm = pair_scratch(w1, w2, w3);
+    return mm ? mm + 2 * align256((size_t)w1->N * 2) : 0;
+}
+
+int hqq_expert_pair_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3,
+                                const void *device_table, const int32_t *expert_index, const void *x_f16, void *y_f16,
+                                const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
+                                void *stream)
+{
+    int rc;
+    if ((rc = validate_linear(w1)) != HQQ_OK || (rc = validate_linear(w2)) != HQQ_OK ||
+        (rc = validate_linear(w3)) != HQQ_OK)
+        return rc;
+    if (w1->N != w3->N || w1->K != w3->K || w2->K != w1->N || w2->N != w1->K)
+        return HQQ_E_SHAPE;
+    if (!x_f16 || !y_f16 || !device_table || !expert_index || !row_scale_f16)
+        return HQQ_E_NULL;
+    const size_t mm_bytes = pair_scratch(w1, w2, w3);
+    if (mm_bytes == 0)
+        return HQQ_E_UNSUPPORTED;
+    if (!workspace || workspace_bytes < hqq_expert_pair_ffn_workspace_bytes(w1, w2, w3) ||
+        (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return HQQ_E_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    char *p = static_cast<char *>(workspace);
+    const size_t mid = align256((size_t)w1->N * 2);
+    f16 *h0 = (f16 *)(p + mm_bytes), *h1 = (f16 *)(p + mm_bytes + mid);
+    const StripIndex gate = {device_table, expert_index, 3, 0}, down = {device_table, expert_index, 3, 2};
+    if ((rc = launch_strip_gate_up_pair(w1, w3, (const f16 *)x_f16, h0, h1, p, mm_bytes, s, gate)) != HQQ_OK)
+        return rc;
+    return launch_strip_down_pair(w2, h0, (int64_t)(mid / 2), (f16 *)y_f16, (const f16 *)row_scale_f16, accumulate, p,
+                                  mm_bytes, s, down);
+}
+
+size_t hqq_matmul_group_workspace_bytes(const hqq_linear *const *layers, int32_t count)
+{
+    if (!layers || count < 1 || count > 4)
+        return 0;
+    for (int i = 0; i < count; ++i)
+        if (validate_linear(layers[i]) != HQQ_OK)
+            return 0;
+    return strip_job_workspace_bytes(layers, count, 1, 1);
+}
+
+int hqq_matmul_group(const hqq_linear *const *layers, int32_t count, const void *x_f16, void *const *ys_f16,
+                     void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!layers || !ys_f16 || !x_f16)
+        return HQQ_E_NULL;
+    if (count < 1 || count > 4)
+        return HQQ_E_SHAPE;
+    int rc;
+    for (int i = 0; i < count; ++i) {
+        if ((rc = validate_linear(layers[i])) != HQQ_OK)
+            return rc;
+        if (!ys_f16[i])
+            return HQQ_E_NULL;
+        if (layers[i]->K != layers[0]->K)
+            return HQQ_E_SHAPE;
+    }
+    const size_t need = strip_job_workspace_bytes(layers, count, 1, 1);
+    if (need == 0)
+        return HQQ_E_UNSUPPORTED;
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return HQQ_E_WORKSPACE;
+    return launch_strip_group(layers, count, (const f16 *)x_f16, reinterpret_cast<f16 *const *>(ys_f16), workspace,
+                              workspace_bytes, (hipStream_t)stream);
+}
+
 int hqq_router_top2(const void *x_f16, const void *gate_w_f16, int32_t n_experts, int64_t hidden, int32_t *sel_out,
                     void *weights_f16_out, void *logits_f16_out, void *stream)
 {
@@ -350,6 +433,17 @@ int hqq_add_rmsnorm(void *x_f16, const void *delta_f16, const void *weight_f16, 
         return HQQ_E_NULL;
     return launch_add_rmsnorm((f16 *)x_f16, (const f16 *)delta_f16, (const f16 *)weight_f16, eps, (f16 *)y_f16, hidden,
                               (hipStream_t)stream);
+}
+
+int hqq_add_rmsnorm_router(void *x_f16, const void *delta_f16, const void *weight_f16, float eps, void *y_f16,
+                           int64_t hidden, const void *gate_w_f16, int32_t n_experts, int32_t *sel_out,
+                           void *weights_f16_out, void *logits_f16_out, void *stream)
+{
+    if (!x_f16 || !weight_f16 || !y_f16 || !gate_w_f16 || !sel_out || !weights_f16_out)
+        return HQQ_E_NULL;
+    return launch_add_rmsnorm_router((f16 *)x_f16, (const f16 *)delta_f16, (const f16 *)weight_f16, eps, (f16 *)y_f16,
+                                     hidden, (const f16 *)gate_w_f16, n_experts, sel_out, (f16 *)weights_f16_out,
+                                     (f16 *)logits_f16_out, (hipStream_t)stream);
 }
 
 int hqq_attention_decode(const void *q_f16, const void *k_f16, const void *v_f16, const void *cos_f16, const void *sin_f16,

@@ -7,31 +7,11 @@ namespace {
 
 constexpr int kMaxExperts = 16;
 
-// logits = fp16(x W^T) (fp32 accumulation, one rounding, as a half linear does); softmax in fp32; the two largest
-// probabilities, renormalised by their sum, cast to fp16 (reference src/custom_layers.py:277-282).
-__global__ __launch_bounds__(64 * kMaxExperts) void router_top2_kernel(const f16 *__restrict__ x, const f16 *__restrict__ w,
-                                                                       int n_experts, int hidden, int *__restrict__ sel,
-                                                                       f16 *__restrict__ weights, f16 *__restrict__ logits_out)
+// softmax over the fp16-rounded logits in fp32, the two largest probabilities renormalised by their sum and cast to
+// fp16 (reference src/custom_layers.py:277-282); one thread.
+__device__ void route_top2(const float *logit_lds, int n_experts, int *__restrict__ sel, f16 *__restrict__ weights,
+                           f16 *__restrict__ logits_out)
 {
-    __shared__ float logit_lds[kMaxExperts];
-    const int lane = threadIdx.x & 63, e = threadIdx.x >> 6;
-    if (e < n_experts) {
-        const f16 *row = w + (int64_t)e * hidden;
-        float acc = 0.f;
-        for (int k = lane * 8; k < hidden; k += 64 * 8) {
-            const f16x8 a = *reinterpret_cast<const f16x8 *>(x + k);
-            const f16x8 b = *reinterpret_cast<const f16x8 *>(row + k);
-#pragma unroll
-            for (int t = 0; t < 8; ++t)
-                acc += (float)a[t] * (float)b[t];
-        }
-        acc = wave_sum(acc);
-        if (lane == 0)
-            logit_lds[e] = (float)(f16)acc;
-    }
-    __syncthreads();
-    if (threadIdx.x != 0)
-        return;
     float mx = logit_lds[0];
     for (int i = 1; i < n_experts; ++i)
         mx = fmaxf(mx, logit_lds[i]);
@@ -56,6 +36,33 @@ __global__ __launch_bounds__(64 * kMaxExperts) void router_top2_kernel(const f16
     sel[0] = b0, sel[1] = b1;
     weights[0] = (f16)(prob[b0] / tot);
     weights[1] = (f16)(prob[b1] / tot);
+}
+
+// logits = fp16(x W^T) (fp32 accumulation, one rounding, as a half linear does); softmax in fp32; the two largest
+// probabilities, renormalised by their sum, cast to fp16 (reference src/custom_layers.py:277-282).
+__global__ __launch_bounds__(64 * kMaxExperts) void router_top2_kernel(const f16 *__restrict__ x, const f16 *__restrict__ w,
+                                                                       int n_experts, int hidden, int *__restrict__ sel,
+                                                                       f16 *__restrict__ weights, f16 *__restrict__ logits_out)
+{
+    __shared__ float logit_lds[kMaxExperts];
+    const int lane = threadIdx.x & 63, e = threadIdx.x >> 6;
+    if (e < n_experts) {
+        const f16 *row = w + (int64_t)e * hidden;
+        float acc = 0.f;
+        for (int k = lane * 8; k < hidden; k += 64 * 8) {
+            const f16x8 a = *reinterpret_cast<const f16x8 *>(x + k);
+            const f16x8 b = *reinterpret_cast<const f16x8 *>(row + k);
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                acc += (float)a[t] * (float)b[t];
+        }
+        acc = wave_sum(acc);
+        if (lane == 0)
+            logit_lds[e] = (float)(f16)acc;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0)
+        route_top2(logit_lds, n_experts, sel, weights, logits_out);
 }
 
 // x += delta (fp16 add, when delta is given; x is written back), then y = weight * fp16(x * rsqrt(mean(x^2) + eps))
@@ -94,6 +101,162 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(f16 *__restrict__ x, c
     }
 }
 
+// add_rmsnorm_kernel followed by router_top2_kernel on its output, in one block: the post-attention norm of a decoder
+// layer feeds the router directly (reference src/custom_layers.py:276-282 on the normed hidden state).
+__global__ __launch_bounds__(256) void add_rmsnorm_router_kernel(f16 *__restrict__ x, const f16 *__restrict__ delta,
+                                                                 const f16 *__restrict__ weight, float eps,
+                                                                 f16 *__restrict__ y, int hidden,
+                                                                 const f16 *__restrict__ gate_w, int n_experts,
+                                                                 int *__restrict__ sel, f16 *__restrict__ weights,
+                                                                 f16 *__restrict__ logits_out)
+{
+    __shared__ float part_lds[4];
+    __shared__ float dot_lds[4][kMaxExperts];
+    __shared__ float logit_lds[kMaxExperts];
+    const int tid = threadIdx.x;
+    float ss = 0.f;
+    for (int k = tid * 8; k < hidden; k += 256 * 8) {
+        f16x8 v = *reinterpret_cast<const f16x8 *>(x + k);
+        if (delta) {
+            v = v + *reinterpret_cast<const f16x8 *>(delta + k);
+            *reinterpret_cast<f16x8 *>(x + k) = v;
+        }
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+            ss += (float)v[t] * (float)v[t];
+    }
+    ss = wave_sum(ss);
+    if ((tid & 63) == 0)
+        part_lds[tid >> 6] = ss;
+    __syncthreads();
+    const float mean = (part_lds[0] + part_lds[1] + part_lds[2] + part_lds[3]) / (float)hidden;
+    const float r = 1.0f / __builtin_sqrtf(mean + eps);
+    float dot[kMaxExperts];
+#pragma unroll
+    for (int e = 0; e < kMaxExperts; ++e)
+        dot[e] = 0.f;
+    for (int k = tid * 8; k < hidden; k += 256 * 8) {
+        const f16x8 v = *reinterpret_cast<const f16x8 *>(x + k); // this thread's own writes
+        const f16x8 w = *reinterpret_cast<const f16x8 *>(weight + k);
+        f16x8 o;
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+            o[t] = w[t] * (f16)((float)v[t] * r);
+        *reinterpret_cast<f16x8 *>(y + k) = o;
+#pragma unroll
+        for (int e = 0; e < kMaxExperts; ++e) {
+            if (e < n_experts) {
+                const f16x8 g = *reinterpret_cast<const f16x8 *>(gate_w + (int64_t)e * hidden + k);
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    dot[e] += (float)o[t] * (float)g[t];
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < kMaxExperts; ++e) {
+        if (e < n_experts) {
+            const float d = wave_sum(dot[e]);
+            if ((tid & 63) == 0)
+                dot_lds[tid >> 6][e] = d;
+        }
+    }
+    __syncthreads();
+    if (tid < n_experts)
+        logit_lds[tid] = (float)(f16)(dot_lds[0][tid] + dot_lds[1][tid] + dot_lds[2][tid] + dot_lds[3][tid]);
+    __syncthreads();
+    if (tid == 0)
+        route_top2(logit_lds, n_experts, sel, weights, logits_out);
+}
+
+// The same computation for hidden <= CH * 2048 and at most NE experts with every global load issued before the
+// first use: the token, the norm weight and the thread's pieces of all router rows travel together, so the block
+// waits for memory once.  Thread t owns elements (c * 256 + t) * 8 .. + 7 of chunk c.
+template <int CH, int NE>
+__global__ __launch_bounds__(256) void add_rmsnorm_router_once_kernel(f16 *__restrict__ x, const f16 *__restrict__ delta,
+                                                                      const f16 *__restrict__ weight, float eps,
+                                                                      f16 *__restrict__ y, int hidden,
+                                                                      const f16 *__restrict__ gate_w, int n_experts,
+                                                                      int *__restrict__ sel, f16 *__restrict__ weights,
+                                                                      f16 *__restrict__ logits_out)
+{
+    __shared__ float part_lds[4];
+    __shared__ float dot_lds[NE][256 + 4];
+    __shared__ float logit_lds[kMaxExperts];
+    const int tid = threadIdx.x;
+    f16x8 xv[CH], wv[CH], gv[CH][NE];
+    bool on[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int k = (c * 256 + tid) * 8;
+        on[c] = k < hidden;
+        const int kc = on[c] ? k : 0;
+        xv[c] = *reinterpret_cast<const f16x8 *>(x + kc);
+        if (delta)
+            xv[c] = xv[c] + *reinterpret_cast<const f16x8 *>(delta + kc);
+        wv[c] = *reinterpret_cast<const f16x8 *>(weight + kc);
+#pragma unroll
+        for (int e = 0; e < NE; ++e)
+            gv[c][e] = *reinterpret_cast<const f16x8 *>(gate_w + (int64_t)(e < n_experts ? e : 0) * hidden + kc);
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        if (on[c]) {
+            if (delta)
+                *reinterpret_cast<f16x8 *>(x + (c * 256 + tid) * 8) = xv[c];
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                ss += (float)xv[c][t] * (float)xv[c][t];
+        }
+    }
+    ss = wave_sum(ss);
+    if ((tid & 63) == 0)
+        part_lds[tid >> 6] = ss;
+    __syncthreads();
+    const float mean = (part_lds[0] + part_lds[1] + part_lds[2] + part_lds[3]) / (float)hidden;
+    const float r = 1.0f / __builtin_sqrtf(mean + eps);
+    float dot[NE];
+#pragma unroll
+    for (int e = 0; e < NE; ++e)
+        dot[e] = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        if (on[c]) {
+            f16x8 o;
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                o[t] = wv[c][t] * (f16)((float)xv[c][t] * r);
+            *reinterpret_cast<f16x8 *>(y + (c * 256 + tid) * 8) = o;
+#pragma unroll
+            for (int e = 0; e < NE; ++e)
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    dot[e] += (float)o[t] * (float)gv[c][e][t];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < NE; ++e)
+        dot_lds[e][tid] = dot[e];
+    __syncthreads();
+    // sixteen threads per expert: each adds sixteen of the 256 partial sums, then the sixteen meet by lane shuffles
+    const int e = tid >> 4, i = tid & 15;
+    if (e < NE) {
+        float a = 0.f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+            a += dot_lds[e][16 * j + i];
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1)
+            a += __shfl_xor(a, off, 64);
+        if (i == 0 && e < n_experts)
+            logit_lds[e] = (float)(f16)a;
+    }
+    __syncthreads();
+    if (tid == 0)
+        route_top2(logit_lds, n_experts, sel, weights, logits_out);
+}
+
 // Rotary embedding, KV-cache append and attention of ONE new token (the reference takes them from HF transformers'
 // Mixtral attention): one block per query head.  Roundings follow the fp16 torch ops they replace: rope terms
 // rounded separately, scores = fp16(q . k) then / sqrt(hd) in fp32, softmax in fp32, probabilities cast to fp16,
@@ -111,7 +274,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const f16 *__rest
     __shared__ __attribute__((aligned(16))) f16 q_lds[HD];
     __shared__ __attribute__((aligned(16))) f16 k_lds[HD];
     __shared__ float red_lds[8];
-    __shared__ float acc_lds[4][HD];
+    __shared__ float acc_lds[256 / (HD / 8)][HD];
     const int h = blockIdx.x, kv = h / group;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t pos = pos_p[0];
@@ -171,25 +334,42 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const f16 *__rest
     sum = red_lds[4] + red_lds[5] + red_lds[6] + red_lds[7];
     const float rs = 1.0f / sum;
 
-    // output: wave w takes positions w, w+4, ...; lane owns HD/64 consecutive dimensions
-    constexpr int PER = HD / 64;
-    float o[PER];
+    // output: LPR threads share a value row (16 bytes each), the block covers ROWS rows per pass and four passes
+    // are in flight; the ROWS partial outputs meet in LDS
+    constexpr int LPR = HD / 8, ROWS = 256 / LPR;
+    const int rsub = tid / LPR, c8 = tid % LPR;
+    float o[8];
 #pragma unroll
-    for (int t = 0; t < PER; ++t)
+    for (int t = 0; t < 8; ++t)
         o[t] = 0.f;
-    for (int64_t l = wave; l <= pos; l += 4) {
-        const float pr = (float)(f16)(score_lds[l] * rs);
-        const f16 *vrow = l == pos ? v_in + kv * HD : cache_v + ((int64_t)kv * max_len + l) * HD;
+    for (int64_t l0 = 0; l0 <= pos; l0 += 4 * ROWS) {
+        f16x8 vv[4];
+        float pr[4];
 #pragma unroll
-        for (int t = 0; t < PER; ++t)
-            o[t] += pr * (float)vrow[lane * PER + t];
+        for (int u = 0; u < 4; ++u) {
+            const int64_t l = l0 + u * ROWS + rsub;
+            const int64_t lc = l <= pos ? l : pos;
+            const f16 *vrow = lc == pos ? v_in + kv * HD : cache_v + ((int64_t)kv * max_len + lc) * HD;
+            vv[u] = *reinterpret_cast<const f16x8 *>(vrow + 8 * c8);
+            pr[u] = l <= pos ? (float)(f16)(score_lds[lc] * rs) : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                o[t] += pr[u] * (float)vv[u][t];
     }
 #pragma unroll
-    for (int t = 0; t < PER; ++t)
-        acc_lds[wave][lane * PER + t] = o[t];
+    for (int t = 0; t < 8; ++t)
+        acc_lds[rsub][8 * c8 + t] = o[t];
     __syncthreads();
-    if (tid < HD)
-        out[h * HD + tid] = (f16)(acc_lds[0][tid] + acc_lds[1][tid] + acc_lds[2][tid] + acc_lds[3][tid]);
+    if (tid < HD) {
+        float a = 0.f;
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r)
+            a += acc_lds[r][tid];
+        out[h * HD + tid] = (f16)a;
+    }
 }
 
 } // namespace
@@ -231,6 +411,28 @@ int launch_add_rmsnorm(f16 *x, const f16 *delta, const f16 *weight, float eps, f
     if (!aligned16(x) || !aligned16(weight) || !aligned16(y) || (delta && !aligned16(delta)))
         return HQQ_E_ALIGN;
     add_rmsnorm_kernel<<<1, 256, 0, s>>>(x, delta, weight, eps, y, (int)hidden);
+    return launch_status();
+}
+
+int launch_add_rmsnorm_router(f16 *x, const f16 *delta, const f16 *weight, float eps, f16 *y, int64_t hidden,
+                              const f16 *gate_w, int n_experts, int *sel, f16 *weights, f16 *logits, hipStream_t s)
+{
+    if (hidden % 8 != 0 || hidden <= 0 || hidden > (1 << 24) || n_experts < 2 || n_experts > kMaxExperts)
+        return HQQ_E_SHAPE;
+    if (!aligned16(x) || !aligned16(weight) || !aligned16(y) || (delta && !aligned16(delta)) || !aligned16(gate_w))
+        return HQQ_E_ALIGN;
+    if (n_experts <= 8 && hidden <= 2048)
+        add_rmsnorm_router_once_kernel<1, 8><<<1, 256, 0, s>>>(x, delta, weight, eps, y, (int)hidden, gate_w, n_experts, sel,
+                                                               weights, logits);
+    else if (n_experts <= 8 && hidden <= 4096)
+        add_rmsnorm_router_once_kernel<2, 8><<<1, 256, 0, s>>>(x, delta, weight, eps, y, (int)hidden, gate_w, n_experts, sel,
+                                                               weights, logits);
+    else if (hidden <= 2048)
+        add_rmsnorm_router_once_kernel<1, 16><<<1, 256, 0, s>>>(x, delta, weight, eps, y, (int)hidden, gate_w, n_experts, sel,
+                                                                weights, logits);
+    else
+        add_rmsnorm_router_kernel<<<1, 256, 0, s>>>(x, delta, weight, eps, y, (int)hidden, gate_w, n_experts, sel, weights,
+                                                    logits);
     return launch_status();
 }
 

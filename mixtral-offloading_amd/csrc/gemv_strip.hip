@@ -36,24 +36,38 @@ struct StripLayer {
 };
 static_assert(sizeof(StripLayer) == 72, "the record is read as 18 words");
 
+// A launch may hold several groups of layers: group g covers blockIdx.z = z_begin .. z_begin + GP - 1 and has its
+// own output.  Groups share K, the code width and the group size, not N (q, k and v projections in one launch;
+// the gates of two experts in one launch).
+constexpr int kMaxGroups = 4;
+struct StripGroup {
+    int z_begin, GP, N, pad;
+    f16 *y;
+    const f16 *bias;
+    float *part[2]; // [BK][M][N] per layer
+};
+
 struct StripParams {
-    StripLayer layer[2];
-    // Indexed launch (table != null): the layer records are read from a device table, record
-    // table[sel[0] * table_stride + table_first + layer], so that which expert runs is decided on the device.
+    StripLayer layer[kMaxGroups]; // record of (group g, layer l) at g * NL + l
+    // Indexed launch (table != null): the layer records are read from a device table instead, record
+    // table[sel[g * sel_gstride + l * sel_lstride] * table_stride + table_first + l * first_lstride], so that which
+    // expert runs is decided on the device.
     const StripLayer *table;
     const int *sel;
     int table_stride, table_first;
-    float *part[2]; // [BK][M][N] per layer
+    int sel_gstride, sel_lstride, first_lstride;
+    StripGroup grp[kMaxGroups];
     const f16 *x;
-    int M, N, K;
-    int GP, RB;
+    int x_lstride; // layer l reads x + l * x_lstride (0: every layer reads the same activations)
+    int M, K;
+    int RB;
     int NS;       // K / 256
     int KS;       // waves per layer in a block
     int BK;       // blocks along K per tile
-    int NL;       // layers in this launch (2 = fused gate)
+    int NL;       // layers per block (2: fused gate, or the down projections of two experts)
     int *counter; // one per tile, zero between launches
-    f16 *y;
-    const f16 *bias, *row_scale;
+    const f16 *row_scale;
+    int rs_lstride; // EPI 2: layer l scales by row_scale[l * rs_lstride + m]
     int accumulate;
 };
 
@@ -67,7 +81,8 @@ template <int MT, int SKIND, int ZKIND> struct SlabRegs {
     uint32_t sms, smz, zms, zmz; // whole-tensor meta values, raw fp16 bits
 };
 
-template <int NBITS, int MT, int S, int D, int WAVES, int SKIND, int ZKIND, int EPI>
+// EPI: 0 y = o (+ bias) (* row_scale) (+ y);  1 y = silu(o0) * o1;  2 y = (y +) o0 * row_scale[0] + o1 * row_scale[1]
+template <int NBITS, int MT, int S, int D, int WAVES, int SKIND, int ZKIND, int EPI, bool GROUPED = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
 {
     constexpr int F = 8 / NBITS;
@@ -88,7 +103,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int kb = blockIdx.x, rb = blockIdx.y, jp = blockIdx.z;
+    const int kb = blockIdx.x, rb = blockIdx.y;
+    int g = 0;
+    if constexpr (GROUPED) // absent groups begin at INT_MAX
+        g = ((int)blockIdx.z >= p.grp[1].z_begin) + ((int)blockIdx.z >= p.grp[2].z_begin) + ((int)blockIdx.z >= p.grp[3].z_begin);
+    const StripGroup &Gd = p.grp[g]; // g is uniform: the record comes from the kernel arguments by scalar loads
+    const int jp = (int)blockIdx.z - Gd.z_begin;
+    const int GP = Gd.GP, N = Gd.N;
     const int layer = wave >= p.KS ? 1 : 0;
     const int ks = wave - layer * p.KS;
     const bool wave_on = wave < p.KS * p.NL;
@@ -96,14 +117,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     StripLayer L;
     if (p.table) {
         // one word of the record per lane, then broadcast: the record's address is known only now
-        const int e = __builtin_amdgcn_readfirstlane(p.sel[0]);
-        const uint32_t *src = reinterpret_cast<const uint32_t *>(p.table + (e * p.table_stride + p.table_first + layer));
+        const int e = __builtin_amdgcn_readfirstlane(p.sel[g * p.sel_gstride + layer * p.sel_lstride]);
+        const uint32_t *src =
+            reinterpret_cast<const uint32_t *>(p.table + (e * p.table_stride + p.table_first + layer * p.first_lstride));
         const uint32_t word = src[lane < 18 ? lane : 0];
         uint32_t rec[18];
 #pragma unroll
         for (int i = 0; i < 18; ++i)
             rec[i] = __builtin_amdgcn_readlane(word, i);
         __builtin_memcpy(&L, rec, sizeof(L));
+    } else if constexpr (GROUPED) {
+        L = p.layer[__builtin_amdgcn_readfirstlane(g * p.NL + layer)];
     } else {
         const StripLayer &A = p.layer[0], &B = p.layer[1];
         L.codes = layer ? B.codes : A.codes;
@@ -134,9 +158,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     // four lanes and costs four times the address cycles; with twelve loads per slab that pipeline, not HBM, then
     // bounds the kernel.
     const int lrow = lane >> 4, lchunk = lane & 15;
-    const uint32_t crow = STAGE ? ((uint32_t)jp + (uint32_t)(16 * rb + lrow) * (uint32_t)p.GP) * (uint32_t)K + (uint32_t)(16 * lchunk)
-                                : ((uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)p.GP) * (uint32_t)K + (uint32_t)(16 * kg);
-    const uint32_t crow_step = STAGE ? 4u * (uint32_t)p.GP * (uint32_t)K : 64u; // four tile rows further / next step
+    const uint32_t crow = STAGE ? ((uint32_t)jp + (uint32_t)(16 * rb + lrow) * (uint32_t)GP) * (uint32_t)K + (uint32_t)(16 * lchunk)
+                                : ((uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)GP) * (uint32_t)K + (uint32_t)(16 * kg);
+    const uint32_t crow_step = STAGE ? 4u * (uint32_t)GP * (uint32_t)K : 64u; // four tile rows further / next step
+    const f16 *xl = p.x + layer * p.x_lstride;
 
     auto issue = [&](SlabRegs<MT, SKIND, ZKIND> &r, int slab) __attribute__((always_inline)) {
         const uint32_t k0 = (uint32_t)slab * kSlab;
@@ -160,12 +185,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
             for (int j = 0; j < (MT + 1) / 2; ++j) {
                 int m = 2 * j + (lane >> 5);
                 m = m < M ? m : 0;
-                r.xw[j] = *reinterpret_cast<const u32x4 *>(p.x + (k0 + (uint32_t)(8 * (lane & 31)) + (uint32_t)(m * K)));
+                r.xw[j] = *reinterpret_cast<const u32x4 *>(xl + (k0 + (uint32_t)(8 * (lane & 31)) + (uint32_t)(m * K)));
             }
         } else {
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
-                const u32x4 *xp = reinterpret_cast<const u32x4 *>(p.x + (k0 + (uint32_t)(16 * kq) + (uint32_t)((m < M ? m : 0) * K)));
+                const u32x4 *xp = reinterpret_cast<const u32x4 *>(xl + (k0 + (uint32_t)(16 * kq) + (uint32_t)((m < M ? m : 0) * K)));
                 r.xw[2 * m] = xp[0];
                 r.xw[2 * m + 1] = xp[1];
             }
@@ -342,7 +367,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
 
     // ---------------------------------------------------------------- block tile: 16 lanes per (layer, row, batch row)
     const bool alone = p.BK == 1;
-    const int tile = jp * p.RB + rb;
+    const int tile = (int)blockIdx.z * p.RB + rb;
     for (int t = threadIdx.x; t < p.NL * 16 * MT * 16; t += WAVES * 64) {
         const int w = t & 15, u = t >> 4;
         const int l_t = u / (16 * MT), r_t = (u / MT) & 15, m_t = u % MT;
@@ -362,29 +387,29 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
         if (w != 0 || m_t >= M)
             continue;
         const int r = 16 * rb + r_t;
-        const int64_t n = (int64_t)F * (jp + (int64_t)r * p.GP); // outputs n .. n+F-1
+        const int64_t n = (int64_t)F * (jp + (int64_t)r * GP); // outputs n .. n+F-1
         if (!alone) {
             // device-scope stores: written through the (per-XCD, mutually non-coherent) L2 so that the finishing
             // block, which may run on another XCD, can read them without any cache-wide flush
-            float *dst = (l_t ? p.part[1] : p.part[0]) + ((int64_t)kb * M + m_t) * p.N + n;
+            float *dst = (l_t ? Gd.part[1] : Gd.part[0]) + ((int64_t)kb * M + m_t) * N + n;
 #pragma unroll
             for (int i = 0; i < F; ++i)
                 __hip_atomic_store(dst + i, o[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             continue;
         }
-        if constexpr (EPI == 1) {
+        if constexpr (EPI != 0) {
             float *dst = &fin_lds[l_t][r_t][m_t][0];
 #pragma unroll
             for (int i = 0; i < F; ++i)
                 dst[i] = o[i];
         } else {
-            f16 *dst = p.y + (int64_t)m_t * p.N + n;
+            f16 *dst = Gd.y + (int64_t)m_t * N + n;
             f16 hv[F];
 #pragma unroll
             for (int i = 0; i < F; ++i) {
                 f16 val = (f16)o[i];
-                if (p.bias)
-                    val = val + p.bias[n + i];
+                if (Gd.bias)
+                    val = val + Gd.bias[n + i];
                 if (p.row_scale)
                     val = val * p.row_scale[m_t];
                 if (p.accumulate)
@@ -400,25 +425,35 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
 
     // both projections rounded to fp16, SiLU in fp32 rounded once, product in fp16: as the reference's ops do
     auto gate = [](float a, float b) __attribute__((always_inline)) -> f16 {
-        const float g = (float)(f16)a;
-        const f16 act = (f16)(g / (1.0f + __expf(-g)));
+        const float u = (float)(f16)a;
+        const f16 act = (f16)(u / (1.0f + __expf(-u)));
         return act * (f16)b;
+    };
+    // two down projections, each rounded to fp16 and scaled by its routing weight, added in layer order: the bits
+    // two launches with row_scale (the second accumulating) would give
+    auto both = [&](float a, float b, int m, f16 prev) __attribute__((always_inline)) -> f16 {
+        const f16 t0 = (f16)a * p.row_scale[m], t1 = (f16)b * p.row_scale[p.rs_lstride + m];
+        return p.accumulate ? (f16)((f16)(prev + t0) + t1) : (f16)(t0 + t1);
     };
 
     if (alone) {
-        if constexpr (EPI == 1) {
+        if constexpr (EPI != 0) {
             __syncthreads();
             for (int u = threadIdx.x; u < 16 * MT; u += WAVES * 64) {
                 const int r_t = u / MT, m_t = u % MT;
                 if (m_t >= M)
                     continue;
                 const int r = 16 * rb + r_t;
-                const int64_t n = (int64_t)F * (jp + (int64_t)r * p.GP);
+                const int64_t n = (int64_t)F * (jp + (int64_t)r * GP);
+                f16 *dst = Gd.y + (int64_t)m_t * N + n;
                 f16 hv[F];
 #pragma unroll
-                for (int i = 0; i < F; ++i)
-                    hv[i] = gate(fin_lds[0][r_t][m_t][i], fin_lds[1][r_t][m_t][i]);
-                f16 *dst = p.y + (int64_t)m_t * p.N + n;
+                for (int i = 0; i < F; ++i) {
+                    if constexpr (EPI == 1)
+                        hv[i] = gate(fin_lds[0][r_t][m_t][i], fin_lds[1][r_t][m_t][i]);
+                    else
+                        hv[i] = both(fin_lds[0][r_t][m_t][i], fin_lds[1][r_t][m_t][i], m_t, p.accumulate ? dst[i] : (f16)0);
+                }
                 if constexpr (F == 4)
                     *reinterpret_cast<f16x4 *>(dst) = (f16x4){hv[0], hv[1], hv[2], hv[3]};
                 else
@@ -448,30 +483,32 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
         if (m_t >= M)
             continue;
         const int r = 16 * rb + r_t;
-        const int64_t n = (int64_t)F * (jp + (int64_t)r * p.GP);
+        const int64_t n = (int64_t)F * (jp + (int64_t)r * GP);
         float a[F], b[F];
 #pragma unroll
         for (int i = 0; i < F; ++i)
             a[i] = b[i] = 0.f;
         for (int s = 0; s < p.BK; ++s) { // fixed order: results do not depend on which block came last
-            const int64_t off = ((int64_t)s * M + m_t) * p.N + n;
+            const int64_t off = ((int64_t)s * M + m_t) * N + n;
 #pragma unroll
             for (int i = 0; i < F; ++i) {
-                a[i] += __hip_atomic_load(p.part[0] + off + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if constexpr (EPI == 1)
-                    b[i] += __hip_atomic_load(p.part[1] + off + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                a[i] += __hip_atomic_load(Gd.part[0] + off + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if constexpr (EPI != 0)
+                    b[i] += __hip_atomic_load(Gd.part[1] + off + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        f16 *dst = p.y + (int64_t)m_t * p.N + n;
+        f16 *dst = Gd.y + (int64_t)m_t * N + n;
         f16 hv[F];
 #pragma unroll
         for (int i = 0; i < F; ++i) {
             if constexpr (EPI == 1) {
                 hv[i] = gate(a[i], b[i]);
+            } else if constexpr (EPI == 2) {
+                hv[i] = both(a[i], b[i], m_t, p.accumulate ? dst[i] : (f16)0);
             } else {
                 f16 val = (f16)a[i];
-                if (p.bias)
-                    val = val + p.bias[n + i];
+                if (Gd.bias)
+                    val = val + Gd.bias[n + i];
                 if (p.row_scale)
                     val = val * p.row_scale[m_t];
                 if (p.accumulate)
@@ -502,7 +539,8 @@ struct StripPlan {
     int F, GP, RB, NS, MT, S, D, WAVES, KS, BK, SKIND, ZKIND;
 };
 
-bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl)
+// tiles_all: tiles of the whole launch when it holds more groups than this layer's (0: this layer alone)
+bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl, int64_t tiles_all = 0)
 {
     if ((l->nbits != 2 && l->nbits != 4) || M < 1 || M > 4)
         return false;
@@ -532,7 +570,9 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl)
     // Shape of the split: S slabs per wave, KS waves per layer, BK blocks along K.  One slab per wave (the most
     // waves in flight) unless a block that holds all of K would then need more than 16 waves; K is split over
     // several blocks only when a single block cannot hold it or there would be too few blocks to cover the chip.
-    const int64_t tiles = (int64_t)pl.GP * pl.RB;
+    const int64_t tiles = tiles_all > 0 ? tiles_all : (int64_t)pl.GP * pl.RB;
+    if (tiles * sizeof(int) > kCounterBytes)
+        return false;
     const int max_waves = pl.MT == 1 ? 16 : 8; // wider batches need more registers and LDS staging per wave
     int S = 1, BK = 1;
     int KS = pl.NS;
@@ -574,88 +614,170 @@ void fill_layer(StripLayer &L, const hqq_linear *l)
     L.z_inv = L.z_cols ? (uint32_t)(0xFFFFFFFFull / L.z_cols) : 0;
 }
 
-template <int NBITS, int MT, int S, int D, int WAVES, int EPI>
+template <int NBITS, int MT, int S, int D, int WAVES, int EPI, bool GROUPED>
 void launch_kinds(const StripParams &p, const StripPlan &pl, dim3 grid, hipStream_t s)
 {
     if (pl.SKIND == TK_F16)
-        gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_F16, TK_F16, EPI><<<grid, dim3(WAVES * 64), 0, s>>>(p);
+        gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_F16, TK_F16, EPI, GROUPED><<<grid, dim3(WAVES * 64), 0, s>>>(p);
     else
-        gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_U8_COLS, TK_U8_SCALAR, EPI><<<grid, dim3(WAVES * 64), 0, s>>>(p);
+        gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_U8_COLS, TK_U8_SCALAR, EPI, GROUPED><<<grid, dim3(WAVES * 64), 0, s>>>(p);
 }
 
-template <int NBITS, int MT, int S, int D, int EPI>
+template <int NBITS, int MT, int S, int D, int EPI, bool GROUPED>
 void launch_waves(const StripParams &p, const StripPlan &pl, dim3 grid, hipStream_t s)
 {
     if constexpr (MT == 1) {
         if (pl.WAVES == 16) {
-            launch_kinds<NBITS, MT, S, D, 16, EPI>(p, pl, grid, s);
+            launch_kinds<NBITS, MT, S, D, 16, EPI, GROUPED>(p, pl, grid, s);
             return;
         }
     }
     if (pl.WAVES >= 8)
-        launch_kinds<NBITS, MT, S, D, 8, EPI>(p, pl, grid, s);
+        launch_kinds<NBITS, MT, S, D, 8, EPI, GROUPED>(p, pl, grid, s);
     else
-        launch_kinds<NBITS, MT, S, D, 4, EPI>(p, pl, grid, s);
+        launch_kinds<NBITS, MT, S, D, 4, EPI, GROUPED>(p, pl, grid, s);
 }
 
-template <int NBITS, int MT, int EPI> void launch_depth(const StripParams &p, const StripPlan &pl, dim3 grid, hipStream_t s)
+template <int NBITS, int MT, int EPI, bool GROUPED>
+void launch_depth(const StripParams &p, const StripPlan &pl, dim3 grid, hipStream_t s)
 {
     if (pl.S == 1)
-        launch_waves<NBITS, MT, 1, 1, EPI>(p, pl, grid, s);
+        launch_waves<NBITS, MT, 1, 1, EPI, GROUPED>(p, pl, grid, s);
     else
-        launch_waves<NBITS, MT, 2, 2, EPI>(p, pl, grid, s);
+        launch_waves<NBITS, MT, 2, 2, EPI, GROUPED>(p, pl, grid, s);
 }
 
-template <int NBITS, int EPI> void launch_batch(const StripParams &p, const StripPlan &pl, dim3 grid, hipStream_t s)
+// several groups in one launch and the two-expert sum exist for single-row batches only (the decode step)
+template <int NBITS, int EPI, bool GROUPED>
+void launch_batch(const StripParams &p, const StripPlan &pl, dim3 grid, hipStream_t s)
 {
-    if (pl.MT == 1)
-        launch_depth<NBITS, 1, EPI>(p, pl, grid, s);
-    else if (pl.MT == 2)
-        launch_depth<NBITS, 2, EPI>(p, pl, grid, s);
-    else
-        launch_depth<NBITS, 4, EPI>(p, pl, grid, s);
+    if (pl.MT == 1) {
+        launch_depth<NBITS, 1, EPI, GROUPED>(p, pl, grid, s);
+        return;
+    }
+    if constexpr (!GROUPED && EPI != 2) {
+        if (pl.MT == 2)
+            launch_depth<NBITS, 2, EPI, false>(p, pl, grid, s);
+        else
+            launch_depth<NBITS, 4, EPI, false>(p, pl, grid, s);
+    }
 }
 
-int run(const hqq_linear *l0, const hqq_linear *l1, const StripIndex *ix, const f16 *x, int64_t M, f16 *y, void *ws,
-        size_t ws_bytes, const SmallBatchEpilogue &ep, hipStream_t s)
+// What one launch covers: NG groups of NL layers each.  Shapes come from shape[g * NL + l]; the records come from
+// the same descriptors, or from a device table when ix is given.
+struct StripJob {
+    const hqq_linear *shape[kMaxGroups];
+    int NG, NL, EPI;
+    const StripIndex *ix;
+    int sel_gstride, sel_lstride, first_lstride;
+    const f16 *x;
+    int64_t x_lstride;
+    f16 *y[kMaxGroups];
+    const f16 *row_scale;
+    int rs_lstride, accumulate;
+};
+
+bool same_family(const hqq_linear *a, const hqq_linear *b)
 {
-    StripPlan pl;
-    const int NL = l1 ? 2 : 1;
-    if (!make_plan(l0, M, NL, pl))
+    return a->K == b->K && a->nbits == b->nbits && a->group_size == b->group_size &&
+           table_kind(a->scale) == table_kind(b->scale) && table_kind(a->zero) == table_kind(b->zero);
+}
+
+// plan of the whole job (the split along K is common to every group) and the bytes of partial sums it needs
+bool plan_job(const StripJob &j, int64_t M, StripPlan &pl, StripPlan *per_group, size_t &part_bytes)
+{
+    if (j.NG < 1 || j.NL < 1 || j.NL > 2 || j.NG * j.NL > kMaxGroups)
+        return false;
+    int64_t tiles = 0;
+    for (int g = 0; g < j.NG; ++g) {
+        StripPlan t;
+        for (int l = 0; l < j.NL; ++l) {
+            const hqq_linear *a = j.shape[g * j.NL + l];
+            if (!a || !make_plan(a, M, j.NL, t) || !same_family(a, j.shape[0]) || a->N != j.shape[g * j.NL]->N)
+                return false;
+        }
+        tiles += (int64_t)t.GP * t.RB;
+    }
+    if ((j.NG > 1 || j.EPI == 2) && M != 1)
+        return false;
+    part_bytes = 0;
+    for (int g = 0; g < j.NG; ++g) {
+        if (!make_plan(j.shape[g * j.NL], M, j.NL, per_group[g], tiles))
+            return false;
+        part_bytes += (size_t)j.NL * (size_t)per_group[g].BK * (size_t)M * (size_t)j.shape[g * j.NL]->N * sizeof(float);
+    }
+    pl = per_group[0];
+    if (pl.BK == 1)
+        part_bytes = 0;
+    return true;
+}
+
+int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
+{
+    StripPlan pl, per_group[kMaxGroups];
+    size_t part_bytes = 0;
+    if (!plan_job(j, M, pl, per_group, part_bytes))
         return HQQ_E_UNSUPPORTED;
-    const size_t one = (size_t)pl.BK * (size_t)M * (size_t)l0->N * sizeof(float);
     const bool alone = pl.BK == 1;
-    if (!alone && (!ws || ws_bytes < kCounterBytes + NL * one))
+    if (!alone && (!ws || ws_bytes < kCounterBytes + part_bytes))
         return HQQ_E_WORKSPACE;
+    if (j.EPI == 2 && !j.row_scale)
+        return HQQ_E_NULL;
     StripParams p = {};
     char *base = static_cast<char *>(ws);
-    fill_layer(p.layer[0], l0);
-    if (l1)
-        fill_layer(p.layer[1], l1);
-    else
-        p.layer[1] = p.layer[0];
-    p.part[0] = alone ? nullptr : reinterpret_cast<float *>(base + kCounterBytes);
-    p.part[1] = alone ? nullptr : reinterpret_cast<float *>(base + kCounterBytes + one);
-    if (ix) {
-        p.table = static_cast<const StripLayer *>(ix->table);
-        p.sel = ix->sel;
-        p.table_stride = ix->stride, p.table_first = ix->first;
+    char *part = base + kCounterBytes;
+    int z = 0;
+    for (int g = 0; g < kMaxGroups; ++g) {
+        StripGroup &G = p.grp[g];
+        if (g >= j.NG) {
+            G.z_begin = 0x7fffffff;
+            continue;
+        }
+        const hqq_linear *a = j.shape[g * j.NL];
+        G.z_begin = z, G.GP = per_group[g].GP, G.N = (int)a->N;
+        G.y = j.y[g];
+        G.bias = j.EPI == 0 ? static_cast<const f16 *>(a->bias) : nullptr;
+        for (int l = 0; l < j.NL; ++l) {
+            fill_layer(p.layer[g * j.NL + l], j.shape[g * j.NL + l]);
+            if (!alone) {
+                G.part[l] = reinterpret_cast<float *>(part);
+                part += (size_t)pl.BK * (size_t)M * (size_t)a->N * sizeof(float);
+            }
+        }
+        z += per_group[g].GP;
     }
-    p.x = x, p.M = (int)M, p.N = (int)l0->N, p.K = (int)l0->K;
-    p.GP = pl.GP, p.RB = pl.RB, p.NS = pl.NS, p.KS = pl.KS, p.BK = pl.BK, p.NL = NL;
+    if (j.NL == 1) // the single-group kernel picks between records 0 and 1 by the wave's layer
+        for (int g = j.NG; g < kMaxGroups; ++g)
+            p.layer[g] = p.layer[0];
+    if (z > 65535)
+        return HQQ_E_UNSUPPORTED;
+    if (j.ix) {
+        p.table = static_cast<const StripLayer *>(j.ix->table);
+        p.sel = j.ix->sel;
+        p.table_stride = j.ix->stride, p.table_first = j.ix->first;
+        p.sel_gstride = j.sel_gstride, p.sel_lstride = j.sel_lstride, p.first_lstride = j.first_lstride;
+    }
+    p.x = j.x, p.x_lstride = (int)j.x_lstride, p.M = (int)M, p.K = (int)j.shape[0]->K;
+    p.RB = pl.RB, p.NS = pl.NS, p.KS = pl.KS, p.BK = pl.BK, p.NL = j.NL;
     p.counter = reinterpret_cast<int *>(base);
-    p.y = y, p.bias = static_cast<const f16 *>(l0->bias), p.row_scale = ep.row_scale, p.accumulate = ep.accumulate;
-    const dim3 grid((unsigned)pl.BK, (unsigned)pl.RB, (unsigned)pl.GP);
-    if (l1) {
-        if (l0->nbits == 2)
-            launch_batch<2, 1>(p, pl, grid, s);
+    p.row_scale = j.row_scale, p.rs_lstride = j.rs_lstride, p.accumulate = j.accumulate;
+    const dim3 grid((unsigned)pl.BK, (unsigned)pl.RB, (unsigned)z);
+    const bool two = j.shape[0]->nbits == 2;
+    if (j.NG > 1) {
+        if (j.EPI == 0 && j.NL == 1)
+            two ? launch_batch<2, 0, true>(p, pl, grid, s) : launch_batch<4, 0, true>(p, pl, grid, s);
+        else if (j.EPI == 1 && j.NL == 2)
+            two ? launch_batch<2, 1, true>(p, pl, grid, s) : launch_batch<4, 1, true>(p, pl, grid, s);
         else
-            launch_batch<4, 1>(p, pl, grid, s);
+            return HQQ_E_UNSUPPORTED;
+    } else if (j.EPI == 0 && j.NL == 1) {
+        two ? launch_batch<2, 0, false>(p, pl, grid, s) : launch_batch<4, 0, false>(p, pl, grid, s);
+    } else if (j.EPI == 1 && j.NL == 2) {
+        two ? launch_batch<2, 1, false>(p, pl, grid, s) : launch_batch<4, 1, false>(p, pl, grid, s);
+    } else if (j.EPI == 2 && j.NL == 2) {
+        two ? launch_batch<2, 2, false>(p, pl, grid, s) : launch_batch<4, 2, false>(p, pl, grid, s);
     } else {
-        if (l0->nbits == 2)
-            launch_batch<2, 0>(p, pl, grid, s);
-        else
-            launch_batch<4, 0>(p, pl, grid, s);
+        return HQQ_E_UNSUPPORTED;
     }
     return launch_status();
 }
@@ -680,7 +802,10 @@ size_t strip_workspace_bytes(const hqq_linear *l, int64_t M)
 int launch_strip_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
                         const SmallBatchEpilogue &ep, hipStream_t s, const StripIndex *ix)
 {
-    return run(l, nullptr, ix, x, M, y, ws, ws_bytes, ep, s);
+    StripJob j = {};
+    j.shape[0] = l, j.NG = 1, j.NL = 1, j.EPI = 0, j.ix = ix, j.first_lstride = 1;
+    j.x = x, j.y[0] = y, j.row_scale = ep.row_scale, j.accumulate = ep.accumulate;
+    return run_job(j, M, ws, ws_bytes, s);
 }
 
 size_t strip_record_bytes() { return sizeof(StripLayer); }
@@ -690,11 +815,61 @@ void strip_fill_record(void *dst, const hqq_linear *l) { fill_layer(*static_cast
 int launch_strip_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
                          size_t ws_bytes, hipStream_t s, const StripIndex *ix)
 {
-    StripPlan a, b;
-    if (!make_plan(w1, M, 2, a) || !make_plan(w3, M, 2, b) || w1->N != w3->N || w1->K != w3->K || w1->nbits != w3->nbits ||
-        w1->group_size != w3->group_size || a.SKIND != b.SKIND || a.ZKIND != b.ZKIND)
+    StripJob j = {};
+    j.shape[0] = w1, j.shape[1] = w3, j.NG = 1, j.NL = 2, j.EPI = 1, j.ix = ix, j.first_lstride = 1;
+    j.x = x, j.y[0] = h;
+    return run_job(j, M, ws, ws_bytes, s);
+}
+
+// The gates of the experts sel[0] and sel[1] of a record table in one launch: h[e] = silu(w1_e x) * w3_e x.
+int launch_strip_gate_up_pair(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, f16 *h0, f16 *h1, void *ws,
+                              size_t ws_bytes, hipStream_t s, const StripIndex &ix)
+{
+    StripJob j = {};
+    j.shape[0] = j.shape[2] = w1, j.shape[1] = j.shape[3] = w3;
+    j.NG = 2, j.NL = 2, j.EPI = 1, j.ix = &ix, j.sel_gstride = 1, j.first_lstride = 1;
+    j.x = x, j.y[0] = h0, j.y[1] = h1;
+    return run_job(j, 1, ws, ws_bytes, s);
+}
+
+// y (+)= w2_{sel[0]} h0 * row_scale[0] + w2_{sel[1]} h1 * row_scale[1] in one launch; h1 = h0 + h_stride.
+int launch_strip_down_pair(const hqq_linear *w2, const f16 *h0, int64_t h_stride, f16 *y, const f16 *row_scale,
+                           int accumulate, void *ws, size_t ws_bytes, hipStream_t s, const StripIndex &ix)
+{
+    StripJob j = {};
+    j.shape[0] = j.shape[1] = w2;
+    j.NG = 1, j.NL = 2, j.EPI = 2, j.ix = &ix, j.sel_lstride = 1, j.first_lstride = 0;
+    j.x = h0, j.x_lstride = h_stride, j.y[0] = y, j.row_scale = row_scale, j.rs_lstride = 1, j.accumulate = accumulate;
+    return run_job(j, 1, ws, ws_bytes, s);
+}
+
+// Up to four projections of the same K, code width and group size applied to the same single row in one launch.
+int launch_strip_group(const hqq_linear *const *layers, int count, const f16 *x, f16 *const *ys, void *ws,
+                       size_t ws_bytes, hipStream_t s)
+{
+    if (count < 1 || count > kMaxGroups)
         return HQQ_E_UNSUPPORTED;
-    return run(w1, w3, ix, x, M, h, ws, ws_bytes, SmallBatchEpilogue{}, s);
+    StripJob j = {};
+    for (int g = 0; g < count; ++g)
+        j.shape[g] = layers[g], j.y[g] = ys[g];
+    j.NG = count, j.NL = 1, j.EPI = 0, j.x = x;
+    return run_job(j, 1, ws, ws_bytes, s);
+}
+
+// bytes of workspace the three launches above can need for these shapes (0 when the strip kernel does not take them)
+size_t strip_job_workspace_bytes(const hqq_linear *const *layers, int count, int NL, int64_t M)
+{
+    if (count < 1 || count > kMaxGroups)
+        return 0;
+    StripJob j = {};
+    for (int g = 0; g < count; ++g)
+        j.shape[g] = layers[g];
+    j.NL = NL, j.NG = count / NL;
+    StripPlan pl, per_group[kMaxGroups];
+    size_t part = 0;
+    if (!plan_job(j, M, pl, per_group, part))
+        return 0;
+    return kCounterBytes + part;
 }
 
 int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s)

@@ -116,6 +116,13 @@ int launch_strip_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, vo
                         const SmallBatchEpilogue &ep, hipStream_t s, const StripIndex *ix = nullptr);
 int launch_strip_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
                          size_t ws_bytes, hipStream_t s, const StripIndex *ix = nullptr);
+int launch_strip_gate_up_pair(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, f16 *h0, f16 *h1, void *ws,
+                              size_t ws_bytes, hipStream_t s, const StripIndex &ix);
+int launch_strip_down_pair(const hqq_linear *w2, const f16 *h0, int64_t h_stride, f16 *y, const f16 *row_scale,
+                           int accumulate, void *ws, size_t ws_bytes, hipStream_t s, const StripIndex &ix);
+int launch_strip_group(const hqq_linear *const *layers, int count, const f16 *x, f16 *const *ys, void *ws,
+                       size_t ws_bytes, hipStream_t s);
+size_t strip_job_workspace_bytes(const hqq_linear *const *layers, int count, int NL, int64_t M);
 int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s);
 size_t workspace_head_bytes();
 bool tile_supported(const hqq_linear *l, int64_t M);
@@ -127,6 +134,8 @@ int launch_vec3_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, voi
 int launch_router_top2(const f16 *x, const f16 *w, int n_experts, int64_t hidden, int *sel, f16 *weights, f16 *logits,
                        hipStream_t s);
 int launch_add_rmsnorm(f16 *x, const f16 *delta, const f16 *weight, float eps, f16 *y, int64_t hidden, hipStream_t s);
+int launch_add_rmsnorm_router(f16 *x, const f16 *delta, const f16 *weight, float eps, f16 *y, int64_t hidden,
+                              const f16 *gate_w, int n_experts, int *sel, f16 *weights, f16 *logits, hipStream_t s);
 int launch_attention_decode(const f16 *q, const f16 *k, const f16 *v, const f16 *cos_t, const f16 *sin_t, const int64_t *pos,
                             f16 *cache_k, f16 *cache_v, int64_t max_len, int n_heads, int n_kv_heads, int head_dim, f16 *out,
                             hipStream_t s);

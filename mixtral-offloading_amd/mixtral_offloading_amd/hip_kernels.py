@@ -233,6 +233,55 @@ def expert_ffn_indexed(table: ExpertTable, expert_index: torch.Tensor, x: torch.
     return out
 
 
+def expert_pair_supported(table: ExpertTable) -> bool:
+    """Whether ``expert_pair_ffn_indexed`` takes the experts of this table."""
+    w1, w2, w3 = table.shape
+    return _lib.lib.hqq_expert_pair_ffn_workspace_bytes(w1.ref, w2.ref, w3.ref) > 0
+
+
+def expert_pair_ffn_indexed(table: ExpertTable, expert_index: torch.Tensor, x: torch.Tensor, out: torch.Tensor,
+                            row_scale: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
+    """``out (+)= sum_e expert_ffn_{expert_index[e]}(x) * row_scale[e]`` over the two active experts of one token
+    (reference src/custom_layers.py:298-312) in two launches; ``expert_index`` int32[2] and ``row_scale`` fp16[2] are
+    device tensors, as ``router_top2`` writes them."""
+    w1, w2, w3 = table.shape
+    assert x.dtype == torch.float16 and x.is_contiguous() and x.numel() == w1.K
+    assert expert_index.dtype == torch.int32 and expert_index.is_cuda and expert_index.numel() >= 2
+    assert row_scale.dtype == torch.float16 and row_scale.is_cuda and row_scale.numel() >= 2
+    assert out.is_contiguous() and out.numel() == w2.N and out.dtype == torch.float16
+    with torch.cuda.device(x.device):
+        need = _lib.lib.hqq_expert_pair_ffn_workspace_bytes(w1.ref, w2.ref, w3.ref)
+        ws = workspace(x.device, need)
+        _lib.check(_lib.lib.hqq_expert_pair_ffn_indexed(w1.ref, w2.ref, w3.ref, table.table.data_ptr(),
+                                                        expert_index.data_ptr(), x.data_ptr(), out.data_ptr(),
+                                                        row_scale.data_ptr(), int(accumulate), ws.data_ptr(), ws.numel(),
+                                                        _lib.current_stream_ptr(x.device)), "hqq_expert_pair_ffn_indexed")
+    return out
+
+
+class LinearGroup:
+    """Up to four layers applied to the same single row in one launch (``hqq_matmul_group``): the q, k and v
+    projections of an attention block.  ``supported`` is False when the layers do not fit one launch."""
+
+    def __init__(self, descs):
+        self.descs = list(descs)
+        n = len(self.descs)
+        self._ptrs = (ctypes.POINTER(_lib.HqqLinear) * n)(*[ctypes.pointer(d.c) for d in self.descs])
+        self.need = int(_lib.lib.hqq_matmul_group_workspace_bytes(self._ptrs, n)) if 1 <= n <= 4 else 0
+        self.supported = self.need > 0
+
+    def __call__(self, x: torch.Tensor):
+        d0 = self.descs[0]
+        assert x.dtype == torch.float16 and x.is_contiguous() and x.numel() == d0.K and x.device == d0.device
+        outs = [torch.empty((1, d.N), device=x.device, dtype=torch.float16) for d in self.descs]
+        ys = (ctypes.c_void_p * len(outs))(*[o.data_ptr() for o in outs])
+        with torch.cuda.device(x.device):
+            ws = workspace(x.device, self.need)
+            _lib.check(_lib.lib.hqq_matmul_group(self._ptrs, len(outs), x.data_ptr(), ys, ws.data_ptr(), ws.numel(),
+                                                 _lib.current_stream_ptr(x.device)), "hqq_matmul_group")
+        return outs
+
+
 def router_top2(x: torch.Tensor, gate_weight: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
                 logits: Optional[torch.Tensor] = None) -> None:
     """Router of one token into device tensors ``sel`` (int32[2]) and ``weights`` (fp16[2])
@@ -254,6 +303,23 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
         _lib.check(_lib.lib.hqq_add_rmsnorm(x.data_ptr(), delta.data_ptr() if delta is not None else None,
                                             weight.data_ptr(), float(eps), out.data_ptr(), x.numel(),
                                             _lib.current_stream_ptr(x.device)), "hqq_add_rmsnorm")
+    return out
+
+
+def add_rmsnorm_router(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                       out: torch.Tensor, gate_weight: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
+                       logits: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``add_rmsnorm`` followed by ``router_top2`` on its output, in one launch."""
+    n_experts, hidden = gate_weight.shape
+    assert x.dtype == torch.float16 and x.is_contiguous() and out.dtype == torch.float16 and x.numel() == weight.numel()
+    assert gate_weight.dtype == torch.float16 and gate_weight.is_contiguous() and x.numel() == hidden
+    assert sel.dtype == torch.int32 and sel.numel() >= 2 and weights.dtype == torch.float16 and weights.numel() >= 2
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib.hqq_add_rmsnorm_router(x.data_ptr(), delta.data_ptr() if delta is not None else None,
+                                                   weight.data_ptr(), float(eps), out.data_ptr(), hidden,
+                                                   gate_weight.data_ptr(), n_experts, sel.data_ptr(), weights.data_ptr(),
+                                                   logits.data_ptr() if logits is not None else None,
+                                                   _lib.current_stream_ptr(x.device)), "hqq_add_rmsnorm_router")
     return out
 
 

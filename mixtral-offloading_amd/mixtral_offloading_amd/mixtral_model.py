@@ -138,6 +138,10 @@ class DecodeGraph:
                 raise RuntimeError("the graph path needs every expert of every layer resident on the device")
             self.tables.append(hip_kernels.ExpertTable(
                 [(m._expert[0].w1._desc(), m._expert[0].w2._desc(), m._expert[0].w3._desc()) for m in mods]))
+        # the two active experts in two launches, q / k / v in one, where the shapes allow
+        self.pair = all(hip_kernels.expert_pair_supported(t) for t in self.tables)
+        self.qkv = [hip_kernels.LinearGroup([p._desc() for p in (l.self_attn.q_proj, l.self_attn.k_proj, l.self_attn.v_proj)])
+                    for l in model.model.layers]
         self.cache = model.new_cache(max_len)
         mk = dict(device=dev)
         self.tok = torch.zeros(1, dtype=torch.int64, **mk)
@@ -164,18 +168,22 @@ class DecodeGraph:
         x = self.x
         x.copy_(m.model.embed_tokens(self.tok))
         delta = None
-        for layer, (ck, cv), table in zip(m.model.layers, self.cache, self.tables):
+        for layer, (ck, cv), table, qkv in zip(m.model.layers, self.cache, self.tables, self.qkv):
             attn = layer.self_attn
             hip_kernels.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps, self.xn)
-            q = attn.q_proj(self.xn)
-            k = attn.k_proj(self.xn)
-            v = attn.v_proj(self.xn)
+            if qkv.supported:
+                q, k, v = qkv(self.xn)
+            else:
+                q, k, v = attn.q_proj(self.xn), attn.k_proj(self.xn), attn.v_proj(self.xn)
             out = hip_kernels.attention_decode(q, k, v, m.rotary.cos, m.rotary.sin, self.pos, ck, cv, self.att)
             attn_out = attn.o_proj(out)
-            hip_kernels.add_rmsnorm(x, attn_out, layer.post_attention_layernorm.weight, eps, self.xn)
-            hip_kernels.router_top2(self.xn, layer.block_sparse_moe.gate.weight, self.sel, self.rw)
-            hip_kernels.expert_ffn_indexed(table, self.sel[0:1], self.xn, self.moe, row_scale=self.rw[0:1])
-            hip_kernels.expert_ffn_indexed(table, self.sel[1:2], self.xn, self.moe, row_scale=self.rw[1:2], accumulate=True)
+            hip_kernels.add_rmsnorm_router(x, attn_out, layer.post_attention_layernorm.weight, eps, self.xn,
+                                           layer.block_sparse_moe.gate.weight, self.sel, self.rw)
+            if self.pair:
+                hip_kernels.expert_pair_ffn_indexed(table, self.sel, self.xn, self.moe, self.rw)
+            else:
+                hip_kernels.expert_ffn_indexed(table, self.sel[0:1], self.xn, self.moe, row_scale=self.rw[0:1])
+                hip_kernels.expert_ffn_indexed(table, self.sel[1:2], self.xn, self.moe, row_scale=self.rw[1:2], accumulate=True)
             delta = self.moe
         hip_kernels.add_rmsnorm(x, delta, m.model.norm.weight, eps, self.xn)
         self.logits.copy_(m.lm_head(self.xn))

@@ -52,6 +52,31 @@ def test_add_rmsnorm_against_torch(hidden, with_delta):
     assert float((y.float() - want.float()).abs().max()) <= 2e-3 * float(want.float().abs().max())
 
 
+@pytest.mark.parametrize("n_experts,hidden", [(8, 4096), (8, 256), (4, 1024), (16, 5120)])
+def test_add_rmsnorm_router_equals_the_two_calls(n_experts, hidden):
+    from mixtral_offloading_amd import hip_kernels
+    g = torch.Generator(device="cuda").manual_seed(hidden + n_experts)
+    for trial in range(3):
+        x = torch.randn((1, hidden), device="cuda", generator=g).half()
+        d = torch.randn((1, hidden), device="cuda", generator=g).half() if trial else None
+        w = (1 + 0.1 * torch.randn(hidden, device="cuda", generator=g)).half()
+        gw = (0.05 * torch.randn((n_experts, hidden), device="cuda", generator=g)).half()
+        x1, y1 = x.clone(), torch.empty_like(x)
+        sel1, rw1 = torch.zeros(2, dtype=torch.int32, device="cuda"), torch.zeros(2, dtype=torch.float16, device="cuda")
+        lg1 = torch.zeros(n_experts, dtype=torch.float16, device="cuda")
+        hip_kernels.add_rmsnorm(x1, d, w, 1e-5, y1)
+        hip_kernels.router_top2(y1, gw, sel1, rw1, lg1)
+        x2, y2 = x.clone(), torch.empty_like(x)
+        sel2, rw2, lg2 = torch.zeros_like(sel1), torch.zeros_like(rw1), torch.zeros_like(lg1)
+        hip_kernels.add_rmsnorm_router(x2, d, w, 1e-5, y2, gw, sel2, rw2, lg2)
+        assert torch.equal(x1, x2) and torch.equal(y1, y2)
+        assert float((lg1.float() - lg2.float()).abs().max()) <= 4e-3 * max(1.0, float(lg1.float().abs().max()))
+        top = lg1.float().sort(descending=True).values
+        if float(top[0] - top[1]) > 0.02 and float(top[1] - top[2]) > 0.02:  # no near-tie
+            assert sel1.tolist() == sel2.tolist()
+            assert float((rw1.float() - rw2.float()).abs().max()) <= 2e-3
+
+
 @pytest.mark.parametrize("m", [1, 2, 4])
 def test_expert_ffn_indexed_equals_direct(m):
     from mixtral_offloading_amd import hip_kernels
@@ -76,6 +101,81 @@ def test_expert_ffn_indexed_equals_direct(m):
         plain = torch.empty_like(base)
         hip_kernels.expert_ffn_indexed(table, idx, x, plain)
         assert torch.equal(plain, hip_kernels.expert_ffn(*experts[e], x))
+
+
+# (nbits, hidden, ffn, group size, quantised tables): K of the down projections split over one and several blocks
+PAIR_SHAPES = [(2, 512, 1024, 16, True), (2, 1024, 3584, 16, True), (4, 512, 2048, 64, True), (2, 256, 768, 16, False),
+               (2, 4096, 14336, 16, True)]
+
+
+@pytest.mark.parametrize("shape", PAIR_SHAPES, ids=lambda s: "w%d_h%d_f%d_g%d_%s" % (s[0], s[1], s[2], s[3], "q" if s[4] else "f16"))
+def test_expert_pair_equals_two_indexed_calls(shape):
+    """Both active experts of a token in two launches against one hqq_expert_ffn_indexed call per expert: the same
+    fp16 rounding points, but K may be split over waves and blocks differently, so the fp32 sums can differ in the
+    last bit and a few outputs land on the neighbouring fp16 value."""
+    from mixtral_offloading_amd import hip_kernels
+    from test_gpu_matmul import _full_size_layer
+    nbits, hidden, ffn, gs, qt = shape
+    rng = np.random.default_rng(hidden + ffn)
+    experts = []
+    for e in range(3):
+        if hidden >= 4096:  # built on the GPU: the numpy generator takes seconds per layer at this size
+            experts.append((_full_size_layer(nbits, ffn, hidden, gs, seed=3 * e), _full_size_layer(nbits, hidden, ffn, gs, seed=3 * e + 1),
+                            _full_size_layer(nbits, ffn, hidden, gs, seed=3 * e + 2)))
+            continue
+        w1, _ = o.random_layer(rng, ffn, hidden, nbits, gs, qt, qt)
+        w3, _ = o.random_layer(rng, ffn, hidden, nbits, gs, qt, qt)
+        w2, _ = o.random_layer(rng, hidden, ffn, nbits, gs, qt, qt)
+        experts.append((desc_of(w1), desc_of(w2), desc_of(w3)))
+    table = hip_kernels.ExpertTable(experts)
+    assert hip_kernels.expert_pair_supported(table)
+    x = to_dev(rng.standard_normal((1, hidden)).astype(np.float16))
+    for pair in ((2, 0), (1, 2), (0, 1), (1, 1)):
+        sel = torch.tensor(pair, dtype=torch.int32, device="cuda")
+        rw = to_dev(rng.uniform(0.2, 0.8, size=(2,)).astype(np.float16))
+        base = to_dev(rng.standard_normal((1, hidden)).astype(np.float16))
+        for accumulate in (False, True):
+            want = base.clone()
+            hip_kernels.expert_ffn_indexed(table, sel[0:1], x, want, row_scale=rw[0:1], accumulate=accumulate)
+            hip_kernels.expert_ffn_indexed(table, sel[1:2], x, want, row_scale=rw[1:2], accumulate=True)
+            got = base.clone()
+            hip_kernels.expert_pair_ffn_indexed(table, sel, x, got, rw, accumulate=accumulate)
+            err = (got.float() - want.float()).abs()
+            # h differs by an fp16 ulp in places, which the down projection carries through
+            assert float(err.max()) <= 4e-3 * float(want.float().abs().max()), (pair, accumulate, float(err.max()))
+            assert float((err > 0).float().mean()) < 0.5
+
+
+@pytest.mark.parametrize("nbits,gs,k,ns,bias", [(4, 64, 4096, (4096, 1024, 1024), False), (4, 64, 1024, (512, 128, 128), True),
+                                                (2, 16, 512, (256, 64), False), (4, 32, 1024, (64, 64, 64, 128), True)])
+def test_matmul_group_equals_single_calls(nbits, gs, k, ns, bias):
+    """q, k and v projections in one launch against hqq_matmul_transpose on each layer: equal up to the order in which
+    the fp32 partial sums over K are added (the split of K follows the size of the whole launch)."""
+    from mixtral_offloading_amd import hip_kernels
+    rng = np.random.default_rng(k + len(ns))
+    descs = []
+    for n in ns:
+        w, _ = o.random_layer(rng, n, k, nbits, gs)
+        b = rng.standard_normal((n,)).astype(np.float16) if bias else None
+        descs.append(desc_of(w, bias=b))
+    group = hip_kernels.LinearGroup(descs)
+    assert group.supported
+    for rep in range(3):
+        x = to_dev(rng.standard_normal((1, k)).astype(np.float16))
+        outs = group(x)
+        for d, y in zip(descs, outs):
+            want = hip_kernels.matmul(d, x)
+            err = (y.float() - want.float()).abs()
+            assert float(err.max()) <= 1e-3 * float(want.float().abs().max()), float(err.max())
+            assert float((err > 0).float().mean()) < 0.2
+
+
+def test_matmul_group_refuses_mixed_layers():
+    from mixtral_offloading_amd import hip_kernels
+    rng = np.random.default_rng(3)
+    a, _ = o.random_layer(rng, 256, 512, 4, 64)
+    b, _ = o.random_layer(rng, 256, 512, 2, 16)
+    assert not hip_kernels.LinearGroup([desc_of(a), desc_of(b)]).supported
 
 
 def test_graph_decode_matches_eager_logits():
