@@ -32,21 +32,30 @@ template <int KIND> struct Raw16 {
     u32x4 ms[2], mz[2]; // per-column meta, 16 halves each
 };
 
+// Load through a pointer known to be device memory.  A pointer that reaches the kernel inside a record (selected
+// between two kernel arguments, or read from a table) has lost its address space, and the compiler then emits flat
+// loads: those count on both memory counters, so the first wait for an LDS operation would also wait for every
+// weight load still in flight.
+template <typename T> __device__ __forceinline__ T gload(const void *p)
+{
+    return *(const T __attribute__((address_space(1))) *)(p);
+}
+
 template <int KIND>
 __device__ __forceinline__ void load16(Raw16<KIND> &r, const uint8_t *tab, const f16 *ms, const f16 *mz, uint32_t c,
                                        uint32_t cm)
 {
     if constexpr (KIND == TK_F16) {
         const u32x4 *p = reinterpret_cast<const u32x4 *>(reinterpret_cast<const f16 *>(tab) + c);
-        r.q = p[0];
-        r.q_hi = p[1];
+        r.q = gload<u32x4>(p);
+        r.q_hi = gload<u32x4>(p + 1);
     } else {
-        r.q = *reinterpret_cast<const u32x4 *>(tab + c);
+        r.q = gload<u32x4>(tab + c);
         if constexpr (KIND == TK_U8_COLS) {
             const u32x4 *a = reinterpret_cast<const u32x4 *>(ms + cm);
             const u32x4 *b = reinterpret_cast<const u32x4 *>(mz + cm);
-            r.ms[0] = a[0], r.ms[1] = a[1];
-            r.mz[0] = b[0], r.mz[1] = b[1];
+            r.ms[0] = gload<u32x4>(a), r.ms[1] = gload<u32x4>(a + 1);
+            r.mz[0] = gload<u32x4>(b), r.mz[1] = gload<u32x4>(b + 1);
         }
     }
 }

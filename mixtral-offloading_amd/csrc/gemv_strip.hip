@@ -102,7 +102,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     __shared__ int ticket_lds;
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    // the wave index as a scalar: what depends on it (the layer, its record, the K range) then lives in scalar
+    // registers, and the record is picked from the kernel arguments without a memory access of its own
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kb = blockIdx.x, rb = blockIdx.y;
     int g = 0;
     if constexpr (GROUPED) // absent groups begin at INT_MAX
@@ -185,31 +187,31 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
             for (int j = 0; j < (MT + 1) / 2; ++j) {
                 int m = 2 * j + (lane >> 5);
                 m = m < M ? m : 0;
-                r.xw[j] = *reinterpret_cast<const u32x4 *>(xl + (k0 + (uint32_t)(8 * (lane & 31)) + (uint32_t)(m * K)));
+                r.xw[j] = gload<u32x4>(xl + (k0 + (uint32_t)(8 * (lane & 31)) + (uint32_t)(m * K)));
             }
         } else {
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 const u32x4 *xp = reinterpret_cast<const u32x4 *>(xl + (k0 + (uint32_t)(16 * kq) + (uint32_t)((m < M ? m : 0) * K)));
-                r.xw[2 * m] = xp[0];
-                r.xw[2 * m + 1] = xp[1];
+                r.xw[2 * m] = gload<u32x4>(xp);
+                r.xw[2 * m + 1] = gload<u32x4>(xp + 1);
             }
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            r.cw[i] = *reinterpret_cast<const u32x4 *>(L.codes + (crow + k0 + (uint32_t)i * crow_step));
+            r.cw[i] = gload<u32x4>(L.codes + (crow + k0 + (uint32_t)i * crow_step));
         // Whole-tensor meta values ride with the slab, after its weight loads.  Their address is the same in every
         // lane, but it is written so that the compiler does not see that (lane >> 6 is zero): a load it knows to be
         // uniform is moved to scalar registers at once, and that move waits for it before any weight load is issued.
         const int zero_off = lane >> 6;
         r.sms = r.smz = r.zms = r.zmz = 0;
         if constexpr (SKIND == TK_U8_SCALAR) {
-            r.sms = reinterpret_cast<const uint16_t *>(L.s_ms)[zero_off];
-            r.smz = reinterpret_cast<const uint16_t *>(L.s_mz)[zero_off];
+            r.sms = gload<uint16_t>(reinterpret_cast<const uint16_t *>(L.s_ms) + zero_off);
+            r.smz = gload<uint16_t>(reinterpret_cast<const uint16_t *>(L.s_mz) + zero_off);
         }
         if constexpr (ZKIND == TK_U8_SCALAR) {
-            r.zms = reinterpret_cast<const uint16_t *>(L.z_ms)[zero_off];
-            r.zmz = reinterpret_cast<const uint16_t *>(L.z_mz)[zero_off];
+            r.zms = gload<uint16_t>(reinterpret_cast<const uint16_t *>(L.z_ms) + zero_off);
+            r.zmz = gload<uint16_t>(reinterpret_cast<const uint16_t *>(L.z_mz) + zero_off);
         }
     };
 
@@ -567,27 +569,48 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl, int64_t ti
     pl.MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
     if (pl.GP > 65535 || pl.RB > 65535 || (int64_t)pl.GP * pl.RB * sizeof(int) > kCounterBytes)
         return false;
-    // Shape of the split: S slabs per wave, KS waves per layer, BK blocks along K.  One slab per wave (the most
-    // waves in flight) unless a block that holds all of K would then need more than 16 waves; K is split over
-    // several blocks only when a single block cannot hold it or there would be too few blocks to cover the chip.
+    // Shape of the split: S slabs per wave, KS waves per layer, BK blocks along K.
     const int64_t tiles = tiles_all > 0 ? tiles_all : (int64_t)pl.GP * pl.RB;
     if (tiles * sizeof(int) > kCounterBytes)
         return false;
     const int max_waves = pl.MT == 1 ? 16 : 8; // wider batches need more registers and LDS staging per wave
     int S = 1, BK = 1;
     int KS = pl.NS;
-    if (KS * NL > max_waves && (pl.NS + 1) / 2 * NL <= max_waves) {
-        S = 2;
-        KS = (pl.NS + 1) / 2;
+    if (pl.MT == 1) {
+        // Single rows (measured on the Mixtral projections): as many waves as the slabs of a compute unit's share
+        // fill, one slab each, while that share is at most 16 slabs; beyond that two or four slabs per wave, the
+        // later ones loaded while the earlier are worked on.  Two-layer blocks run best as eight waves of four
+        // slabs, two blocks to a compute unit.  K is split over blocks when a block cannot hold it, or when there
+        // would be fewer than about a hundred blocks.
+        const int64_t share = tiles * pl.NS * NL / 256;
+        S = NL == 2 ? 4 : (share <= 16 ? 1 : (share <= 32 ? 2 : 4));
+        while (S > 1 && S > pl.NS)
+            S /= 2;
+        const int cap = NL == 2 && S == 4 ? 4 : max_waves / NL;
+        const int groups = (pl.NS + S - 1) / S;
+        KS = groups;
+        while (KS > cap || (tiles * BK < 100 && KS > 4 && BK < 16)) {
+            ++BK;
+            KS = (groups + BK - 1) / BK;
+        }
+    } else {
+        // One slab per wave unless a block that holds all of K would then need more than eight waves; K is split over
+        // several blocks only when a single block cannot hold it or there would be too few blocks to cover the chip.
+        if (KS * NL > max_waves && (pl.NS + 1) / 2 * NL <= max_waves) {
+            S = 2;
+            KS = (pl.NS + 1) / 2;
+        }
+        while (KS * NL > max_waves || (tiles * BK < 200 && KS > 4 && BK < 16)) {
+            ++BK;
+            KS = ((pl.NS + S - 1) / S + BK - 1) / BK;
+        }
     }
-    while (KS * NL > max_waves || (tiles * BK < 200 && KS > 4 && BK < 16)) {
-        ++BK;
-        KS = ((pl.NS + S - 1) / S + BK - 1) / BK;
+    if (env_int("HQQ_STRIP_K", (int)l->K) == (int)l->K && env_int("HQQ_STRIP_NL", NL) == NL) {
+        S = env_int("HQQ_STRIP_S", S);
+        KS = env_int("HQQ_STRIP_KS", KS);
+        BK = env_int("HQQ_STRIP_BK", BK);
     }
-    S = env_int("HQQ_STRIP_S", S);
-    KS = env_int("HQQ_STRIP_KS", KS);
-    BK = env_int("HQQ_STRIP_BK", BK);
-    if (S != 1 && S != 2)
+    if (S != 1 && S != 2 && !(S == 4 && pl.MT == 1))
         return false;
     if (KS < 1 || KS * NL > max_waves || BK < 1 || BK > 65535)
         return false;
@@ -595,7 +618,7 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl, int64_t ti
         return false;
     pl.S = S, pl.KS = KS, pl.BK = BK;
     pl.WAVES = KS * NL > 8 ? 16 : (KS * NL > 4 ? 8 : 4);
-    pl.D = S; // every slab of the wave in flight at once
+    pl.D = S < 2 ? S : 2; // slabs of a wave in flight at once
     return true;
 }
 
@@ -643,8 +666,10 @@ void launch_depth(const StripParams &p, const StripPlan &pl, dim3 grid, hipStrea
 {
     if (pl.S == 1)
         launch_waves<NBITS, MT, 1, 1, EPI, GROUPED>(p, pl, grid, s);
-    else
+    else if (pl.S == 2)
         launch_waves<NBITS, MT, 2, 2, EPI, GROUPED>(p, pl, grid, s);
+    else if constexpr (MT == 1)
+        launch_waves<NBITS, MT, 4, 2, EPI, GROUPED>(p, pl, grid, s);
 }
 
 // several groups in one launch and the two-expert sum exist for single-row batches only (the decode step)
