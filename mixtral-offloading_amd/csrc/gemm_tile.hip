@@ -232,6 +232,47 @@ __global__ __launch_bounds__(256) void tile_finish_kernel(const float *__restric
     }
 }
 
+// 3-bit codes (ten per 32-bit word, rows 10p .. 10p+9) rewritten as 4-bit codes (rows 2q, 2q+1 per byte, the even
+// row in the high nibble): a 3-bit code is a 4-bit code with the same value, so the tile kernel then runs unchanged
+// on the same tables.  Rows 2q and 2q+1 always share a word.  One thread: one word row, four columns.
+__global__ __launch_bounds__(256) void repack3_as4_kernel(const uint32_t *__restrict__ in, int64_t N, int64_t K,
+                                                          uint8_t *__restrict__ out)
+{
+    const int64_t words = (N + 9) / 10, chunks = K / 4;
+    for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < words * chunks; idx += (int64_t)gridDim.x * 256) {
+        const int64_t p = idx / chunks, c = (idx - p * chunks) * 4;
+        const u32x4 w = *reinterpret_cast<const u32x4 *>(in + p * K + c);
+#pragma unroll
+        for (int i = 0; i < 5; ++i) {
+            const int64_t q = 5 * p + i;
+            if (2 * q >= N)
+                break;
+            const int sh = 3 * (8 - 2 * i); // fields 2i (upper three bits of the six) and 2i+1
+            uint32_t b = 0;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint32_t v = (w[t] >> sh) & 0x3Fu;
+                b |= (((v >> 3) << 4) | (v & 7u)) << (8 * t);
+            }
+            *reinterpret_cast<uint32_t *>(out + q * K + c) = b;
+        }
+    }
+}
+
+// the layer as the tile kernel sees it: 3-bit layers are run through their 4-bit rewrite
+hqq_linear tile_view(const hqq_linear *l)
+{
+    hqq_linear v = *l;
+    if (l->nbits == 3)
+        v.nbits = 4;
+    return v;
+}
+
+size_t rewrite_bytes(const hqq_linear *l)
+{
+    return l->nbits == 3 ? (((size_t)(l->N / 2) * (size_t)l->K + 255) & ~(size_t)255) : 0;
+}
+
 struct TilePlan {
     int F, GP, RB, KT, BM, KSP, KTS;
 };
@@ -288,25 +329,46 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl)
 bool tile_supported(const hqq_linear *l, int64_t M)
 {
     TilePlan pl;
+    if (l->nbits == 3) { // below seven rows the 3-bit row kernel, run in passes of two rows, is faster than the rewrite
+        const hqq_linear v = tile_view(l);
+        return M > 6 && l->N % 2 == 0 && l->K % 4 == 0 && aligned16(l->codes) && make_plan(&v, M, pl);
+    }
     return M > 4 && make_plan(l, M, pl);
+}
+
+// [arrival counters of the decode kernels][fp32 partial sums when K is split][4-bit rewrite of 3-bit codes]
+static size_t partial_bytes(const hqq_linear *l, int64_t M, const TilePlan &pl)
+{
+    return pl.KSP == 1 ? 0 : (((size_t)pl.KSP * (size_t)M * (size_t)l->N * sizeof(float) + 255) & ~(size_t)255);
 }
 
 size_t tile_workspace_bytes(const hqq_linear *l, int64_t M)
 {
     TilePlan pl;
-    if (!make_plan(l, M, pl) || pl.KSP == 1)
+    const hqq_linear v = tile_view(l);
+    if (!make_plan(&v, M, pl))
         return 0;
-    // the head of a workspace holds the arrival counters of the decode kernels: partial sums go behind it
-    return workspace_head_bytes() + (size_t)pl.KSP * (size_t)M * (size_t)l->N * sizeof(float);
+    const size_t body = partial_bytes(l, M, pl) + rewrite_bytes(l);
+    return body ? workspace_head_bytes() + body : 0;
 }
 
-int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s)
+int launch_tile_matmul(const hqq_linear *l3, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s)
 {
     TilePlan pl;
+    hqq_linear view = tile_view(l3);
+    const hqq_linear *l = &view;
     if (!make_plan(l, M, pl) || (reinterpret_cast<uintptr_t>(x) & 15u))
         return HQQ_E_UNSUPPORTED;
-    if (pl.KSP > 1 && (!ws || ws_bytes < tile_workspace_bytes(l, M)))
+    const size_t need = tile_workspace_bytes(l3, M);
+    if (need > 0 && (!ws || ws_bytes < need))
         return HQQ_E_WORKSPACE;
+    if (l3->nbits == 3) {
+        uint8_t *codes4 = reinterpret_cast<uint8_t *>(ws) + workspace_head_bytes() + partial_bytes(l, M, pl);
+        const int64_t work = ((l3->N + 9) / 10) * (l3->K / 4);
+        const int grid = (int)(work / 256 < 1 ? 1 : (work / 256 > 8192 ? 8192 : work / 256));
+        repack3_as4_kernel<<<grid, 256, 0, s>>>(static_cast<const uint32_t *>(l3->codes), l3->N, l3->K, codes4);
+        view.codes = codes4;
+    }
     TileParams p = {};
     p.codes = static_cast<const uint8_t *>(l->codes);
     p.sc = make_table(l->scale), p.zr = make_table(l->zero);
