@@ -13,10 +13,17 @@
 //     step, eight exact fp16 weights (mask-and-insert into 2^e, subtract, subtract z, multiply s);
 //   * 2 * F * BM/16 MFMAs per wave.
 // Weight bytes come from HBM once; the x tile is re-read by N / (64*F) blocks, from L2.
+#include "gemv_parts.hpp"
 #include "hqq_common.hpp"
 #include "table_reader.hpp"
 
+#include <cstdlib>
+
 namespace hqq {
+using gemv::gload;
+using gemv::TK_F16;
+using gemv::TK_U8_COLS;
+using gemv::TK_U8_SCALAR;
 namespace {
 
 constexpr int kStepK = 64;
@@ -29,7 +36,8 @@ struct TileParams {
     const f16 *x;
     const f16 *bias;
     f16 *y;
-    float *part; // [KSP][M][N] fp32 partial sums when K is split over several blocks, else null
+    float *part; // [KSP][N/F][M][F] fp32 partial sums when K is split over several blocks, else null: the sixteen
+                 // batch rows a lane group holds for one row group are then 256 consecutive bytes
     int M, N, K, GP, KT;
     int KSP; // blocks along K
     int KTS; // steps per block
@@ -153,21 +161,20 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile_kernel(TileParams p)
                 B[b] = *reinterpret_cast<const f16x8 *>(&x_lds[(((h * 4 + kg) * BM) + b * 16 + (lane & 15)) * 8]);
 #pragma unroll
             for (int i = 0; i < F; ++i) {
-                const f16x8 S = *reinterpret_cast<const f16x8 *>(&s_lds[wave][((i * 2 + h) * 4 + kg) * 8]);
-                const f16x8 Z = *reinterpret_cast<const f16x8 *>(&z_lds[wave][((i * 2 + h) * 4 + kg) * 8]);
+                const u32x4 S = *reinterpret_cast<const u32x4 *>(&s_lds[wave][((i * 2 + h) * 4 + kg) * 8]);
+                const u32x4 Z = *reinterpret_cast<const u32x4 *>(&z_lds[wave][((i * 2 + h) * 4 + kg) * 8]);
                 const uint32_t mk = WField<NBITS>::mask(i), ex = WField<NBITS>::expo(i);
                 const f16 offv = (f16)WField<NBITS>::offset(i);
                 const f16x2 off = {offv, offv};
                 const uint32_t src[4] = {d0, d0s, d1, d1s};
-                f16x8 A;
+                u32x4 Au; // whole 32-bit words throughout: a pair of weights per register, no element inserts
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     const f16x2 q = as_f16x2((src[t] & mk) | ex) - off;          // exact code
-                    const f16x2 zz = {Z[2 * t], Z[2 * t + 1]}, ss = {S[2 * t], S[2 * t + 1]};
-                    const f16x2 w = (q - zz) * ss;                                // two fp16 roundings, as the reference
-                    A[2 * t] = w.x;
-                    A[2 * t + 1] = w.y;
+                    const f16x2 w = (q - as_f16x2(Z[t])) * as_f16x2(S[t]);        // two fp16 roundings, as the reference
+                    Au[t] = __builtin_bit_cast(uint32_t, w);
                 }
+                const f16x8 A = __builtin_bit_cast(f16x8, Au);
 #pragma unroll
                 for (int b = 0; b < MB; ++b)
                     acc[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B[b], acc[i][b], 0, 0, 0);
@@ -186,7 +193,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile_kernel(TileParams p)
             const int r = 16 * rb + 4 * kg + v;
             const int64_t n = (int64_t)F * (jp + (int64_t)r * p.GP);
             if (p.part) { // K is split over blocks: fp32 partial sums, added by the finishing kernel
-                float *dst = p.part + ((int64_t)ks * p.M + m) * p.N + n;
+                float *dst = p.part + (((int64_t)ks * (p.N / F) + n / F) * p.M + m) * F; // [K block][row group][batch row][F]
                 if constexpr (F == 4)
                     *reinterpret_cast<f32x4 *>(dst) = (f32x4){acc[0][b][v], acc[1][b][v], acc[2][b][v], acc[3][b][v]};
                 else
@@ -209,26 +216,288 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile_kernel(TileParams p)
     }
 }
 
-// y = cast(sum over the K blocks) (+ bias)
+
+// ---------------------------------------------------------------------------------------------------------------
+// The kernel for the two table layouts HQQ produces (8-bit tables with per-column meta for the scale and whole-tensor
+// meta for the zero; or fp16 tables).  Same tiling as above, organised around memory latency: codes and tables, which
+// come from HBM, are requested four steps ahead into one of four register sets; the x tile, which every block
+// re-reads from L2, two steps ahead into one of two; the x tile and the de-quantised tables of the next step are
+// written to the other half of a double-buffered LDS while this step is worked on, and there is one barrier per
+// step.  Every load is unconditional (a step past the end re-reads the last one; batch rows past M re-read row
+// M - 1, whose results are never stored), so the compiler's wait counts are exact; within a step the x loads are
+// issued before the weight loads, because loads retire in issue order and the x tile is needed first.  The x tile
+// is padded by two entries per k block: the sixteen lanes of an LDS write then fall into sixteen different groups
+// of banks.
+struct TileWeightRegs {
+    u32x4 cw;             // 16 code bytes: four columns per word, rows by field
+    uint32_t sq, zq;      // four table bytes (8-bit kinds)
+    u32x2 sm_s, sm_z;     // per-column meta of the scale: four halves each
+    u32x2 sf, zf;         // four table halves (fp16 kind)
+};
+
+template <int NBITS, int BM, int SKIND, int ZKIND>
+__global__ __launch_bounds__(kWaves * 64) void gemm_tile2_kernel(TileParams p)
+{
+    constexpr int F = 8 / NBITS;
+    constexpr int MB = BM / 16;
+    constexpr int XP = BM + 2;
+    constexpr int XCH = (BM * 8 + kWaves * 64 - 1) / (kWaves * 64);
+    constexpr int TAB = F * 2 * 4 * 8; // halves per wave and table: entry ((i*2 + h)*4 + kg) of 8 halves
+    __shared__ __attribute__((aligned(16))) f16 x_lds[2][8 * XP * 8];
+    __shared__ __attribute__((aligned(16))) f16 s_lds[2][kWaves][TAB];
+    __shared__ __attribute__((aligned(16))) f16 z_lds[2][kWaves][TAB];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int jblk = blockIdx.x / p.KSP, ks = blockIdx.x - jblk * p.KSP;
+    const int jp = jblk * kWaves + wave;
+    const int s_begin = ks * p.KTS;
+    const int s_end = s_begin + p.KTS < p.KT ? s_begin + p.KTS : p.KT;
+    const int s_last = s_end - 1;
+    const int rb = blockIdx.y;
+    const int m0 = blockIdx.z * BM;
+    const int K = p.K;
+    const int rr = lane & 15, kg = lane >> 4;
+    const int ti = lane >> 4, kq = lane & 15;
+    const bool tlane = ti < F;
+    const int ti_l = ti & (F - 1); // lanes past the table rows repeat a table lane's loads: issuing loads never diverges
+
+    const uint8_t *codes = p.codes + ((size_t)((uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)p.GP) * K + 16 * kg);
+    const uint32_t c_row = (uint32_t)(F * jp + ti_l) * (uint32_t)K + (uint32_t)(4 * kq);
+    const uint8_t *s_tab = static_cast<const uint8_t *>(p.sc.data), *z_tab = static_cast<const uint8_t *>(p.zr.data);
+    const uint32_t s_cols = (uint32_t)p.sc.meta_cols;
+    // whole-tensor meta of the zero table, splat
+    f16x2 zms = {(f16)0, (f16)0}, zmz = zms;
+    if constexpr (ZKIND == TK_U8_SCALAR) {
+        const f16 a = gload<f16>(p.zr.ms), b = gload<f16>(p.zr.mz);
+        zms = (f16x2){a, a}, zmz = (f16x2){b, b};
+    }
+    // x tile: thread t moves chunks (column m, k block kb) = (ch / 8, ch % 8), ch = t, t + 256, ...; k block kb = h*4 + kg
+    // holds the columns half h of lane group kg works on: 16*kg + 8*h .. +7
+    const f16 *xsrc[XCH];
+    int xdst[XCH];
+#pragma unroll
+    for (int c = 0; c < XCH; ++c) {
+        const int ch = (int)threadIdx.x + c * kWaves * 64;
+        const int chc = ch < BM * 8 ? ch : BM * 8 - 1;
+        int m = m0 + chc / 8;
+        m = m < p.M ? m : p.M - 1;
+        const int kb = chc % 8;
+        xsrc[c] = p.x + (size_t)m * K + 16 * (kb & 3) + 8 * (kb >> 2);
+        xdst[c] = (kb * XP + chc / 8) * 8;
+    }
+
+    typedef TileWeightRegs Regs;
+    struct XRegs {
+        u32x4 xr[XCH];
+    };
+    auto issue = [&](Regs &r, int s) __attribute__((always_inline)) {
+        s = s < s_last ? s : s_last;
+        const uint32_t k0 = (uint32_t)s * kStepK;
+        r.cw = gload<u32x4>(codes + k0);
+        const uint32_t c = c_row + k0;
+        if constexpr (SKIND == TK_F16) {
+            r.sf = gload<u32x2>(reinterpret_cast<const f16 *>(s_tab) + c);
+            r.zf = gload<u32x2>(reinterpret_cast<const f16 *>(z_tab) + c);
+        } else {
+            r.sq = gload<uint32_t>(s_tab + c);
+            r.zq = gload<uint32_t>(z_tab + c);
+            uint32_t cm = c - __umulhi(c, p.sc_inv) * s_cols; // c mod cols; the quotient estimate is at most 2 short
+            cm -= cm >= s_cols ? s_cols : 0;
+            cm -= cm >= s_cols ? s_cols : 0;
+            r.sm_s = gload<u32x2>(p.sc.ms + cm);
+            r.sm_z = gload<u32x2>(p.sc.mz + cm);
+        }
+    };
+    auto issue_x = [&](XRegs &r, int s) __attribute__((always_inline)) {
+        s = s < s_last ? s : s_last;
+        const uint32_t k0 = (uint32_t)s * kStepK;
+#pragma unroll
+        for (int c2 = 0; c2 < XCH; ++c2)
+            r.xr[c2] = gload<u32x4>(xsrc[c2] + k0);
+    };
+
+    // x tile and de-quantised tables of one step into LDS half `buf`
+    const int tab_w = (((ti_l * 2 + ((kq >> 1) & 1)) * 4 + (kq >> 2)) * 8) + 4 * (kq & 1);
+    auto stage = [&](const Regs &r, const XRegs &xr, int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int c = 0; c < XCH; ++c) {
+            // eight columns (0..7) stored in B-operand order (0,2,1,3,4,6,5,7)
+            const u32x4 v = xr.xr[c];
+            u32x4 o;
+            o.x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);
+            o.y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
+            o.z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
+            o.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
+            if (XCH * kWaves * 64 == BM * 8 || (int)threadIdx.x + c * kWaves * 64 < BM * 8)
+                *reinterpret_cast<u32x4 *>(&x_lds[buf][xdst[c]]) = o;
+        }
+        if (tlane) {
+            f16x2 s01, s23, z01, z23;
+            if constexpr (SKIND == TK_F16) {
+                s01 = as_f16x2(r.sf.x), s23 = as_f16x2(r.sf.y);
+                z01 = as_f16x2(r.zf.x), z23 = as_f16x2(r.zf.y);
+            } else {
+                // bytes -> fp16 exactly: 0x6400 | b is 1024 + b, then subtract 1024
+                const f16x2 k1024 = {(f16)1024.0f, (f16)1024.0f};
+                const f16x2 a01 = as_f16x2(__builtin_amdgcn_perm(0x64646464u, r.sq, 0x04010400u)) - k1024;
+                const f16x2 a23 = as_f16x2(__builtin_amdgcn_perm(0x64646464u, r.sq, 0x04030402u)) - k1024;
+                const f16x2 b01 = as_f16x2(__builtin_amdgcn_perm(0x64646464u, r.zq, 0x04010400u)) - k1024;
+                const f16x2 b23 = as_f16x2(__builtin_amdgcn_perm(0x64646464u, r.zq, 0x04030402u)) - k1024;
+                s01 = (a01 - as_f16x2(r.sm_z.x)) * as_f16x2(r.sm_s.x);
+                s23 = (a23 - as_f16x2(r.sm_z.y)) * as_f16x2(r.sm_s.y);
+                z01 = (b01 - zmz) * zms;
+                z23 = (b23 - zmz) * zms;
+            }
+            *reinterpret_cast<f16x4 *>(&s_lds[buf][wave][tab_w]) = (f16x4){s01.x, s23.x, s01.y, s23.y};
+            *reinterpret_cast<f16x4 *>(&z_lds[buf][wave][tab_w]) = (f16x4){z01.x, z23.x, z01.y, z23.y};
+        }
+    };
+
+    f32x4 acc[F][MB];
+#pragma unroll
+    for (int i = 0; i < F; ++i)
+#pragma unroll
+        for (int b = 0; b < MB; ++b)
+            acc[i][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    auto compute = [&](const u32x4 cw, int buf) __attribute__((always_inline)) {
+        const uint32_t d[4] = {cw.x, cw.y, cw.z, cw.w};
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t d0 = d[2 * h], d1 = d[2 * h + 1];
+            const uint32_t src[4] = {d0, d0 >> 8, d1, d1 >> 8};
+            f16x8 B[MB];
+#pragma unroll
+            for (int b = 0; b < MB; ++b)
+                B[b] = *reinterpret_cast<const f16x8 *>(&x_lds[buf][(((h * 4 + kg) * XP) + b * 16 + rr) * 8]);
+#pragma unroll
+            for (int i = 0; i < F; ++i) {
+                const u32x4 S = *reinterpret_cast<const u32x4 *>(&s_lds[buf][wave][((i * 2 + h) * 4 + kg) * 8]);
+                const u32x4 Z = *reinterpret_cast<const u32x4 *>(&z_lds[buf][wave][((i * 2 + h) * 4 + kg) * 8]);
+                const uint32_t mk = WField<NBITS>::mask(i), ex = WField<NBITS>::expo(i);
+                const f16 offv = (f16)WField<NBITS>::offset(i);
+                const f16x2 off = {offv, offv};
+                u32x4 Au;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const f16x2 q = as_f16x2((mk & src[t]) | (~mk & ex)) - off; // exact code (one v_bfi_b32)
+                    const f16x2 w = (q - as_f16x2(Z[t])) * as_f16x2(S[t]); // two fp16 roundings, as the reference
+                    Au[t] = __builtin_bit_cast(uint32_t, w);
+                }
+                const f16x8 A = __builtin_bit_cast(f16x8, Au);
+#pragma unroll
+                for (int b = 0; b < MB; ++b)
+                    acc[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B[b], acc[i][b], 0, 0, 0);
+            }
+        }
+    };
+
+    // Step s is worked on from LDS half (s - s_begin) & 1 while step s + 1 is staged into the other half; the
+    // register sets that step s + 1 leaves are refilled with the x tile of step s + 3 and the weights of step s + 5.
+    Regs T0, T1, T2, T3;
+    XRegs X0, X1;
+    issue_x(X0, s_begin);
+    issue(T0, s_begin);
+    issue_x(X1, s_begin + 1);
+    issue(T1, s_begin + 1);
+    issue(T2, s_begin + 2);
+    issue(T3, s_begin + 3);
+    stage(T0, X0, 0);
+    u32x4 cw = T0.cw;
+    issue_x(X0, s_begin + 2);
+    issue(T0, s_begin + 4);
+    __syncthreads();
+    auto step = [&](Regs &Tn, XRegs &Xn, int buf, int s) __attribute__((always_inline)) {
+        if (s < s_end)
+            compute(cw, buf);
+        stage(Tn, Xn, buf ^ 1);
+        cw = Tn.cw;
+        issue_x(Xn, s + 3);
+        issue(Tn, s + 5);
+        __syncthreads();
+    };
+    for (int s = s_begin; s < s_end; s += 4) {
+        step(T1, X1, 0, s);
+        step(T2, X0, 1, s + 1);
+        step(T3, X1, 0, s + 2);
+        step(T0, X0, 1, s + 3);
+    }
+
+    // D layout: column = batch column (lane & 15) of block b, rows r = 4*(lane>>4) + v
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+        const int m = m0 + b * 16 + (lane & 15);
+        if (m >= p.M)
+            continue;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int r = 16 * rb + 4 * kg + v;
+            const int64_t n = (int64_t)F * (jp + (int64_t)r * p.GP);
+            if (p.part) { // K is split over blocks: fp32 partial sums, added by the finishing kernel
+                float *dst = p.part + (((int64_t)ks * (p.N / F) + n / F) * p.M + m) * F; // [K block][row group][batch row][F]
+                if constexpr (F == 4)
+                    *reinterpret_cast<f32x4 *>(dst) = (f32x4){acc[0][b][v], acc[1][b][v], acc[2][b][v], acc[3][b][v]};
+                else
+                    *reinterpret_cast<float2 *>(dst) = make_float2(acc[0][b][v], acc[1][b][v]);
+                continue;
+            }
+            f16 o[F];
+#pragma unroll
+            for (int i = 0; i < F; ++i) {
+                o[i] = (f16)acc[i][b][v];
+                if (p.bias)
+                    o[i] = o[i] + p.bias[n + i];
+            }
+            f16 *dst = p.y + (int64_t)m * p.N + n;
+            if constexpr (F == 4)
+                *reinterpret_cast<f16x4 *>(dst) = (f16x4){o[0], o[1], o[2], o[3]};
+            else
+                *reinterpret_cast<f16x2 *>(dst) = (f16x2){o[0], o[1]};
+        }
+    }
+}
+
+// y = cast(sum over the K blocks) (+ bias).  A block adds a tile of 16 row groups x 16 batch rows: read along the
+// batch rows (the order the partial sums are stored in), written along the output row (the order y is stored in).
+template <int F>
 __global__ __launch_bounds__(256) void tile_finish_kernel(const float *__restrict__ part, int KSP, int M, int N,
                                                            const f16 *__restrict__ bias, f16 *__restrict__ y)
 {
-    const int64_t total = (int64_t)M * N / 4;
-    const int64_t stride = (int64_t)M * N;
-    for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
-        const int64_t e = idx * 4;
-        f32x4 a = {0, 0, 0, 0};
-        for (int s = 0; s < KSP; ++s)
-            a += *reinterpret_cast<const f32x4 *>(part + s * stride + e);
-        f16x4 out;
+    __shared__ f16 t_lds[16][16][F];
+    const int NG = N / F;
+    const int g0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
+    {
+        const int m = m0 + (threadIdx.x & 15), gl = threadIdx.x >> 4, g = g0 + gl;
+        if (m < M && g < NG) {
+            float a[F];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            f16 v = (f16)a[t];
-            if (bias)
-                v = v + bias[(e + t) % N];
-            out[t] = v;
+            for (int i = 0; i < F; ++i)
+                a[i] = 0.f;
+            for (int s = 0; s < KSP; ++s) {
+                const float *src = part + (((int64_t)s * NG + g) * M + m) * F;
+#pragma unroll
+                for (int i = 0; i < F; ++i)
+                    a[i] += src[i];
+            }
+#pragma unroll
+            for (int i = 0; i < F; ++i) {
+                f16 v = (f16)a[i];
+                if (bias)
+                    v = v + bias[F * g + i];
+                t_lds[threadIdx.x & 15][gl][i] = v;
+            }
         }
-        *reinterpret_cast<f16x4 *>(y + e) = out;
+    }
+    __syncthreads();
+    {
+        const int gl = threadIdx.x & 15, m = m0 + (threadIdx.x >> 4), g = g0 + gl;
+        if (m < M && g < NG) {
+            f16 *dst = y + (int64_t)m * N + F * g;
+#pragma unroll
+            for (int i = 0; i < F; ++i)
+                dst[i] = t_lds[threadIdx.x >> 4][gl][i];
+        }
     }
 }
 
@@ -275,6 +544,7 @@ size_t rewrite_bytes(const hqq_linear *l)
 
 struct TilePlan {
     int F, GP, RB, KT, BM, KSP, KTS;
+    int kinds; // 1: 8-bit tables as HQQ writes them, 3: fp16 tables (both run the pipelined kernel), 0: anything else
 };
 
 bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl)
@@ -305,23 +575,64 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl)
     pl.GP = (int)(G / F);
     pl.RB = l->group_size / 16;
     pl.KT = (int)(l->K / kStepK);
-    // batch tile: as wide as the batch up to 64 columns, so that every weight is rebuilt as few times as possible
+    const int sk = gemv::table_kind(l->scale), zk = gemv::table_kind(l->zero);
+    pl.kinds = sk == TK_U8_COLS && zk == TK_U8_SCALAR ? 1 : (sk == TK_F16 && zk == TK_F16 ? 3 : 0);
+    // batch tile: as wide as the batch, so that every weight is rebuilt as few times as possible; past 64 columns
+    // the width (64 or 128, the latter in the pipelined kernel only) that costs less over all tiles, a tile costing
+    // about 760 cycles of rebuilding and 8 cycles of MFMA per column and step
     pl.BM = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
+    if (M > 128 && pl.kinds != 0 && ((M + 127) / 128) * (760 + 8 * 128) <= ((M + 63) / 64) * (760 + 8 * 64))
+        pl.BM = 128;
+    if (const char *e = std::getenv("HQQ_TILE_BM"))
+        pl.BM = std::atoi(e);
     const int64_t mtiles = (M + pl.BM - 1) / pl.BM;
     if (mtiles > 65535)
         return false;
-    // K is split over blocks until about two blocks per compute unit exist (partial sums go through the workspace)
+    // K is split over blocks so that every SIMD gets one wave (two when there are more than 256 waves to begin
+    // with) and all waves do the same number of steps: measured at Mixtral shapes, one split more than that (waves
+    // left over for a second, partly filled round) costs 20-40 %, and partial sums cost HBM traffic of their own.
     const int64_t blocks = (int64_t)(pl.GP / kWaves) * pl.RB * mtiles;
-    int64_t ksp = (512 + blocks - 1) / blocks;
+    const int64_t waves = blocks * kWaves;
+    int64_t ksp = waves <= 256 ? 1024 / waves : (waves < 512 ? 2048 / waves : 1);
     if (ksp > pl.KT / 4)
         ksp = pl.KT / 4; // at least four steps per block
     if (ksp < 1)
         ksp = 1;
+    if (const char *e = std::getenv("HQQ_TILE_KSP"))
+        ksp = std::atoi(e);
     pl.KTS = (int)((pl.KT + ksp - 1) / ksp);
     pl.KSP = (pl.KT + pl.KTS - 1) / pl.KTS;
     if ((int64_t)(pl.GP / kWaves) * pl.KSP > 0x7fffffff)
         return false;
     return true;
+}
+
+template <int NBITS, int BM> void launch_tile2_kinds(const TileParams &p, const TilePlan &pl, dim3 grid, hipStream_t s)
+{
+    if (pl.kinds == 1)
+        gemm_tile2_kernel<NBITS, BM, TK_U8_COLS, TK_U8_SCALAR><<<grid, kWaves * 64, 0, s>>>(p);
+    else
+        gemm_tile2_kernel<NBITS, BM, TK_F16, TK_F16><<<grid, kWaves * 64, 0, s>>>(p);
+}
+
+template <int NBITS> void launch_tile2_bm(const TileParams &p, const TilePlan &pl, dim3 grid, hipStream_t s)
+{
+    if (pl.BM == 16)
+        launch_tile2_kinds<NBITS, 16>(p, pl, grid, s);
+    else if (pl.BM == 32)
+        launch_tile2_kinds<NBITS, 32>(p, pl, grid, s);
+    else if (pl.BM == 64)
+        launch_tile2_kinds<NBITS, 64>(p, pl, grid, s);
+    else
+        launch_tile2_kinds<NBITS, 128>(p, pl, grid, s);
+}
+
+void launch_tile2(const TileParams &p, const TilePlan &pl, int nbits, dim3 grid, hipStream_t s)
+{
+    if (nbits == 2)
+        launch_tile2_bm<2>(p, pl, grid, s);
+    else
+        launch_tile2_bm<4>(p, pl, grid, s);
 }
 
 } // namespace
@@ -379,7 +690,9 @@ int launch_tile_matmul(const hqq_linear *l3, const f16 *x, int64_t M, f16 *y, vo
     p.KSP = pl.KSP, p.KTS = pl.KTS;
     p.part = pl.KSP > 1 ? reinterpret_cast<float *>(static_cast<char *>(ws) + workspace_head_bytes()) : nullptr;
     const dim3 grid((unsigned)(pl.GP / kWaves * pl.KSP), (unsigned)pl.RB, (unsigned)((M + pl.BM - 1) / pl.BM));
-    if (l->nbits == 2) {
+    if (pl.kinds != 0) {
+        launch_tile2(p, pl, l->nbits, grid, s);
+    } else if (l->nbits == 2) {
         if (pl.BM == 16)
             gemm_tile_kernel<2, 16><<<grid, kWaves * 64, 0, s>>>(p);
         else if (pl.BM == 32)
@@ -397,9 +710,11 @@ int launch_tile_matmul(const hqq_linear *l3, const f16 *x, int64_t M, f16 *y, vo
     int rc = launch_status();
     if (rc != HQQ_OK || pl.KSP == 1)
         return rc;
-    const int64_t quads = M * l->N / 4;
-    const int fgrid = (int)(quads / 256 < 1 ? 1 : (quads / 256 > 4096 ? 4096 : quads / 256));
-    tile_finish_kernel<<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, p.bias, y);
+    const dim3 fgrid((unsigned)((l->N / pl.F + 15) / 16), (unsigned)((M + 15) / 16));
+    if (pl.F == 4)
+        tile_finish_kernel<4><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, p.bias, y);
+    else
+        tile_finish_kernel<2><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, p.bias, y);
     return launch_status();
 }
 

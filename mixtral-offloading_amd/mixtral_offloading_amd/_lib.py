@@ -9,7 +9,8 @@ import os
 from ctypes import c_char_p, c_int, c_int32, c_int64, c_size_t, c_void_p
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_PKG), "lib", "libhqq_mi355x.so")
+# HQQ_MI355X_LIB names another build of the library (a profiling or debug build); the default is the in-tree one
+LIB_PATH = os.environ.get("HQQ_MI355X_LIB") or os.path.join(os.path.dirname(_PKG), "lib", "libhqq_mi355x.so")
 
 if not os.path.exists(LIB_PATH):
     raise ImportError(
