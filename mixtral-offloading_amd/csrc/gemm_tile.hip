@@ -588,14 +588,16 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl)
     const int64_t mtiles = (M + pl.BM - 1) / pl.BM;
     if (mtiles > 65535)
         return false;
-    // K is split over blocks so that every SIMD gets one wave (two when there are more than 256 waves to begin
-    // with) and all waves do the same number of steps: measured at Mixtral shapes, one split more than that (waves
-    // left over for a second, partly filled round) costs 20-40 %, and partial sums cost HBM traffic of their own.
+    // K is split over blocks until every SIMD has a wave (two for batches up to 128 rows, whose partial sums are
+    // small), with at least eight steps per block.  Measured at Mixtral shapes: a split beyond that, which leaves
+    // waves over for a partly filled round, costs 20-40 %.
     const int64_t blocks = (int64_t)(pl.GP / kWaves) * pl.RB * mtiles;
     const int64_t waves = blocks * kWaves;
-    int64_t ksp = waves <= 256 ? 1024 / waves : (waves < 512 ? 2048 / waves : 1);
-    if (ksp > pl.KT / 4)
-        ksp = pl.KT / 4; // at least four steps per block
+    int64_t ksp = (M <= 128 ? 2048 : 1024) / waves;
+    if (ksp > 16)
+        ksp = 16;
+    if (ksp > pl.KT / 8)
+        ksp = pl.KT / 8;
     if (ksp < 1)
         ksp = 1;
     if (const char *e = std::getenv("HQQ_TILE_KSP"))
