@@ -145,11 +145,12 @@ def survey_section(dev):
         r = {"kernel": name, "us": round(us, 2), "GB_s": round(nbytes / us / 1e3, 0), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)}
         if flops:
             r["TFLOP_s"] = round(flops / us / 1e6, 1)
+            r["frac_mfma_f16"] = round(flops / us / 1e6 / 2500.0, 3)
         rows.append(r)
         print(f"{name:58s} {us:9.2f} us {r['GB_s']:8.0f} GB/s" + (f" {r['TFLOP_s']:8.1f} TFLOP/s" if flops else ""), file=sys.stderr, flush=True)
 
-    shapes = [(4, 4096, 4096, 64, (1, 4, 16, 128)), (4, 1024, 4096, 64, (1,)), (2, 14336, 4096, 16, (1, 4, 16, 128)),
-              (2, 4096, 14336, 16, (1, 4, 16, 128)), (3, 14336, 4096, 64, (1, 8)), (3, 4096, 14336, 64, (1, 8))]
+    shapes = [(4, 4096, 4096, 64, (1, 4, 16, 128, 512)), (4, 1024, 4096, 64, (1,)), (2, 14336, 4096, 16, (1, 4, 16, 128, 512)),
+              (2, 4096, 14336, 16, (1, 4, 16, 128, 512)), (3, 14336, 4096, 64, (1, 8, 128)), (3, 4096, 14336, 64, (1, 8, 128))]
     for nbits, n, k, gs, batches in shapes:
         wbytes = (n * k * nbits // 8 if nbits != 3 else ((n + 9) // 10) * k * 4) + 2 * (n * k // gs) + 4 * (n * k // gs // META_GROUP) + 4
         nl = max(2, min(16, (320 << 20) // wbytes + 1))

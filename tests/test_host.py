@@ -40,6 +40,23 @@ def test_argument_errors_without_touching_the_gpu():
     assert _lib.lib.hqq_pack_4bit_u8(1 << 20, 3, 4, 1 << 21, None) == -3  # odd height (reference src/packing.py:12)
     assert _lib.lib.hqq_pack_4bit_u8(None, 2, 4, 1 << 21, None) == -1
     assert _lib.lib.hqq_pack_4bit_u8(None, 0, 4, None, None) == 0  # empty input, even without addresses
+    # the decode-step entry points refuse bad arguments before any launch
+    lib = _lib.lib
+    assert lib.hqq_matmul_group(None, 3, 1 << 20, None, None, 0, None) == -1
+    ok = _lib.HqqLinear()
+    ok.nbits, ok.group_size, ok.N, ok.K, ok.codes = 4, 64, 256, 512, 1 << 20
+    ok.scale.data = ok.zero.data = 1 << 21
+    ptrs = (ctypes.POINTER(_lib.HqqLinear) * 1)(ctypes.pointer(ok))
+    ys = (ctypes.c_void_p * 1)(1 << 22)
+    assert lib.hqq_matmul_group(ptrs, 0, 1 << 20, ys, None, 0, None) == -3  # count out of 1..4
+    assert lib.hqq_matmul_group(ptrs, 5, 1 << 20, ys, None, 0, None) == -3
+    assert lib.hqq_matmul_group_workspace_bytes(ptrs, 5) == 0
+    assert lib.hqq_matmul_group(ptrs, 1, 1 << 20, ys, None, 0, None) == -5  # no workspace
+    assert lib.hqq_expert_pair_ffn_indexed(ctypes.byref(ok), ctypes.byref(ok), ctypes.byref(ok), None, None, None, None,
+                                           None, 0, None, 0, None) == -3  # w2 must map ffn -> hidden
+    assert lib.hqq_add_rmsnorm_router(None, None, None, 1e-5, None, 4096, None, 8, None, None, None, None) == -1
+    assert lib.hqq_add_rmsnorm_router(1 << 20, None, 1 << 21, 1e-5, 1 << 22, 4096, 1 << 23, 17, 1 << 24, 1 << 25, None,
+                                      None) == -3  # more than 16 experts
 
 
 def _plan(lib, c, experts):
