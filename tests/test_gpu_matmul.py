@@ -74,6 +74,29 @@ def test_matmul_forced_family(shape, family):
         assert ran >= (2 if family == 1 else 1)
 
 
+# the tile family at its edges: one to eleven 64-column steps (fewer than the pipeline is deep, odd counts, K splits
+# that do not divide evenly) and batches around every tile width, the 128-column tile included
+TILE_SHAPES = [
+    (2, 1024, 64, 16, 64, True, True),
+    (2, 1024, 128, 16, 128, True, True),
+    (2, 1024, 192, 16, 128, True, True),
+    (4, 512, 320, 64, 128, False, False),
+    (2, 512, 704, 16, 128, True, True),
+    (4, 1024, 576, 64, 128, True, True),
+]
+
+
+@pytest.mark.parametrize("shape", TILE_SHAPES, ids=lambda s: "w%d_%dx%d_g%d" % s[:4])
+@pytest.mark.parametrize("m", [5, 16, 40, 64, 65, 129, 200, 257])
+def test_tile_family_edges(shape, m):
+    nbits, n, k, gs, mgs, qs, qz = shape
+    rng = np.random.default_rng(n + k + m)
+    layer, _ = o.random_layer(rng, n, k, nbits, gs, qs, qz, meta_group_size=mgs)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    bias = rng.standard_normal(n).astype(np.float16) if m % 2 else None
+    _check(layer, x, family=2, bias=bias)  # a refusal (HqqError) fails the test: these shapes are the family's own
+
+
 def test_bias_leading_dims_and_empty():
     from mixtral_offloading_amd import hip_kernels
     rng = np.random.default_rng(5)
