@@ -576,8 +576,8 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl, int64_t ti
     const int max_waves = pl.MT == 1 ? 16 : 8; // wider batches need more registers and LDS staging per wave
     int S = 1, BK = 1;
     int KS = pl.NS;
-    if (pl.MT == 1) {
-        // Single rows (measured on the Mixtral projections): as many waves as the slabs of a compute unit's share
+    if (pl.MT <= 2) {
+        // One and two rows (measured on the Mixtral projections): as many waves as the slabs of a compute unit's share
         // fill, one slab each, while that share is at most 16 slabs; beyond that two or four slabs per wave, the
         // later ones loaded while the earlier are worked on.  Two-layer blocks run best as eight waves of four
         // slabs, two blocks to a compute unit.  K is split over blocks when a block cannot hold it, or when there
@@ -610,7 +610,7 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl, int64_t ti
         KS = env_int("HQQ_STRIP_KS", KS);
         BK = env_int("HQQ_STRIP_BK", BK);
     }
-    if (S != 1 && S != 2 && !(S == 4 && pl.MT == 1))
+    if (S != 1 && S != 2 && !(S == 4 && pl.MT <= 2))
         return false;
     if (KS < 1 || KS * NL > max_waves || BK < 1 || BK > 65535)
         return false;
@@ -668,7 +668,7 @@ void launch_depth(const StripParams &p, const StripPlan &pl, dim3 grid, hipStrea
         launch_waves<NBITS, MT, 1, 1, EPI, GROUPED>(p, pl, grid, s);
     else if (pl.S == 2)
         launch_waves<NBITS, MT, 2, 2, EPI, GROUPED>(p, pl, grid, s);
-    else if constexpr (MT == 1)
+    else if constexpr (MT <= 2)
         launch_waves<NBITS, MT, 4, 2, EPI, GROUPED>(p, pl, grid, s);
 }
 
