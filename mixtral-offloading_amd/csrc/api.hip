@@ -200,6 +200,9 @@ static size_t ffn_matmul_scratch(const hqq_linear *w1, const hqq_linear *w2, con
         mm = m2;
     if (m3 > mm)
         mm = m3;
+    const size_t g = tile_gate_workspace_bytes(w1, w3, M);
+    if (g > mm)
+        mm = g;
     return align256(mm);
 }
 
@@ -267,6 +270,10 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
     if (fast13) {
         rc = launch_smallbatch_gate_up(w1, w3, x, M, h, mm, mm_bytes, s);
         if (rc != HQQ_OK)
+            return rc;
+    } else if (prefer_tile && tile_gate_supported(w1, w3, M)) {
+        // both projections in one launch of the tile kernel, silu(a) * b in its finishing pass
+        if ((rc = launch_tile_gate_up(w1, w3, x, M, h, mm, mm_bytes, s)) != HQQ_OK)
             return rc;
     } else {
         if ((rc = run_matmul(w1, x, M, a, mm, mm_bytes, pick_family(w1, M), s)) != HQQ_OK)

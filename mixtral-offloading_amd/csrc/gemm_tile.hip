@@ -41,6 +41,13 @@ struct TileParams {
     int M, N, K, GP, KT;
     int KSP; // blocks along K
     int KTS; // steps per block
+    // second layer of a fused gate launch (pipelined kernel only): blocks JB * KSP and up work on it and write
+    // their partial sums part_lstride floats further; JB = row blocks per layer
+    const uint8_t *codes_b;
+    Table sc_b, zr_b;
+    uint32_t sc_b_inv;
+    int JB;
+    int64_t part_lstride;
 };
 
 template <int NBITS> struct WField {
@@ -249,8 +256,12 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile2_kernel(TileParams p)
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int jblk = blockIdx.x / p.KSP, ks = blockIdx.x - jblk * p.KSP;
+    const int jall = blockIdx.x / p.KSP, ks = blockIdx.x - jall * p.KSP;
+    const bool second = jall >= p.JB; // block-uniform: the selections below are scalar
+    const int jblk = jall - (second ? p.JB : 0);
     const int jp = jblk * kWaves + wave;
+    const Table &sc_t = second ? p.sc_b : p.sc, &zr_t = second ? p.zr_b : p.zr;
+    const uint32_t sc_inv = second ? p.sc_b_inv : p.sc_inv;
     const int s_begin = ks * p.KTS;
     const int s_end = s_begin + p.KTS < p.KT ? s_begin + p.KTS : p.KT;
     const int s_last = s_end - 1;
@@ -262,14 +273,15 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile2_kernel(TileParams p)
     const bool tlane = ti < F;
     const int ti_l = ti & (F - 1); // lanes past the table rows repeat a table lane's loads: issuing loads never diverges
 
-    const uint8_t *codes = p.codes + ((size_t)((uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)p.GP) * K + 16 * kg);
+    const uint8_t *codes = (second ? p.codes_b : p.codes) + ((size_t)((uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)p.GP) * K + 16 * kg);
     const uint32_t c_row = (uint32_t)(F * jp + ti_l) * (uint32_t)K + (uint32_t)(4 * kq);
-    const uint8_t *s_tab = static_cast<const uint8_t *>(p.sc.data), *z_tab = static_cast<const uint8_t *>(p.zr.data);
-    const uint32_t s_cols = (uint32_t)p.sc.meta_cols;
+    const uint8_t *s_tab = static_cast<const uint8_t *>(sc_t.data), *z_tab = static_cast<const uint8_t *>(zr_t.data);
+    const f16 *s_ms = sc_t.ms, *s_mz = sc_t.mz;
+    const uint32_t s_cols = (uint32_t)sc_t.meta_cols;
     // whole-tensor meta of the zero table, splat
     f16x2 zms = {(f16)0, (f16)0}, zmz = zms;
     if constexpr (ZKIND == TK_U8_SCALAR) {
-        const f16 a = gload<f16>(p.zr.ms), b = gload<f16>(p.zr.mz);
+        const f16 a = gload<f16>(zr_t.ms), b = gload<f16>(zr_t.mz);
         zms = (f16x2){a, a}, zmz = (f16x2){b, b};
     }
     // x tile: thread t moves chunks (column m, k block kb) = (ch / 8, ch % 8), ch = t, t + 256, ...; k block kb = h*4 + kg
@@ -302,11 +314,11 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile2_kernel(TileParams p)
         } else {
             r.sq = gload<uint32_t>(s_tab + c);
             r.zq = gload<uint32_t>(z_tab + c);
-            uint32_t cm = c - __umulhi(c, p.sc_inv) * s_cols; // c mod cols; the quotient estimate is at most 2 short
+            uint32_t cm = c - __umulhi(c, sc_inv) * s_cols; // c mod cols; the quotient estimate is at most 2 short
             cm -= cm >= s_cols ? s_cols : 0;
             cm -= cm >= s_cols ? s_cols : 0;
-            r.sm_s = gload<u32x2>(p.sc.ms + cm);
-            r.sm_z = gload<u32x2>(p.sc.mz + cm);
+            r.sm_s = gload<u32x2>(s_ms + cm);
+            r.sm_z = gload<u32x2>(s_mz + cm);
         }
     };
     auto issue_x = [&](XRegs &r, int s) __attribute__((always_inline)) {
@@ -435,7 +447,8 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile2_kernel(TileParams p)
             const int r = 16 * rb + 4 * kg + v;
             const int64_t n = (int64_t)F * (jp + (int64_t)r * p.GP);
             if (p.part) { // K is split over blocks: fp32 partial sums, added by the finishing kernel
-                float *dst = p.part + (((int64_t)ks * (p.N / F) + n / F) * p.M + m) * F; // [K block][row group][batch row][F]
+                float *dst = p.part + (second ? p.part_lstride : 0) +
+                             (((int64_t)ks * (p.N / F) + n / F) * p.M + m) * F; // [K block][row group][batch row][F]
                 if constexpr (F == 4)
                     *reinterpret_cast<f32x4 *>(dst) = (f32x4){acc[0][b][v], acc[1][b][v], acc[2][b][v], acc[3][b][v]};
                 else
@@ -460,9 +473,12 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile2_kernel(TileParams p)
 
 // y = cast(sum over the K blocks) (+ bias).  A block adds a tile of 16 row groups x 16 batch rows: read along the
 // batch rows (the order the partial sums are stored in), written along the output row (the order y is stored in).
-template <int F>
+// GATE: two sets of partial sums, lstride floats apart; y = silu(a) * b with both projections rounded to fp16, SiLU
+// in fp32 rounded once, product in fp16 (the reference's three ops, src/custom_layers.py:253-256).
+template <int F, bool GATE>
 __global__ __launch_bounds__(256) void tile_finish_kernel(const float *__restrict__ part, int KSP, int M, int N,
-                                                           const f16 *__restrict__ bias, f16 *__restrict__ y)
+                                                           const f16 *__restrict__ bias, f16 *__restrict__ y,
+                                                           int64_t lstride)
 {
     __shared__ f16 t_lds[16][16][F];
     const int NG = N / F;
@@ -470,21 +486,28 @@ __global__ __launch_bounds__(256) void tile_finish_kernel(const float *__restric
     {
         const int m = m0 + (threadIdx.x & 15), gl = threadIdx.x >> 4, g = g0 + gl;
         if (m < M && g < NG) {
-            float a[F];
+            float a[F], b[F];
 #pragma unroll
             for (int i = 0; i < F; ++i)
-                a[i] = 0.f;
+                a[i] = b[i] = 0.f;
             for (int s = 0; s < KSP; ++s) {
                 const float *src = part + (((int64_t)s * NG + g) * M + m) * F;
 #pragma unroll
-                for (int i = 0; i < F; ++i)
+                for (int i = 0; i < F; ++i) {
                     a[i] += src[i];
+                    if constexpr (GATE)
+                        b[i] += src[lstride + i];
+                }
             }
 #pragma unroll
             for (int i = 0; i < F; ++i) {
                 f16 v = (f16)a[i];
-                if (bias)
+                if constexpr (GATE) {
+                    const float u = (float)v;
+                    v = (f16)(u / (1.0f + __expf(-u))) * (f16)b[i];
+                } else if (bias) {
                     v = v + bias[F * g + i];
+                }
                 t_lds[threadIdx.x & 15][gl][i] = v;
             }
         }
@@ -547,7 +570,8 @@ struct TilePlan {
     int kinds; // 1: 8-bit tables as HQQ writes them, 3: fp16 tables (both run the pipelined kernel), 0: anything else
 };
 
-bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl)
+// nl: layers of the launch (2 for the fused gate, whose blocks count twice towards filling the chip)
+bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl, int nl = 1)
 {
     if ((l->nbits != 2 && l->nbits != 4) || M < 1)
         return false;
@@ -591,7 +615,7 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl)
     // K is split over blocks until every SIMD has a wave (two for batches up to 128 rows, whose partial sums are
     // small), with at least eight steps per block.  Measured at Mixtral shapes: a split beyond that, which leaves
     // waves over for a partly filled round, costs 20-40 %.
-    const int64_t blocks = (int64_t)(pl.GP / kWaves) * pl.RB * mtiles;
+    const int64_t blocks = (int64_t)(pl.GP / kWaves) * pl.RB * mtiles * nl;
     const int64_t waves = blocks * kWaves;
     int64_t ksp = (M <= 128 ? 2048 : 1024) / waves;
     if (ksp > 16)
@@ -604,7 +628,7 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl)
         ksp = std::atoi(e);
     pl.KTS = (int)((pl.KT + ksp - 1) / ksp);
     pl.KSP = (pl.KT + pl.KTS - 1) / pl.KTS;
-    if ((int64_t)(pl.GP / kWaves) * pl.KSP > 0x7fffffff)
+    if ((int64_t)(pl.GP / kWaves) * pl.KSP * nl > 0x7fffffff)
         return false;
     return true;
 }
@@ -649,49 +673,62 @@ bool tile_supported(const hqq_linear *l, int64_t M)
     return M > 4 && make_plan(l, M, pl);
 }
 
-// [arrival counters of the decode kernels][fp32 partial sums when K is split][4-bit rewrite of 3-bit codes]
-static size_t partial_bytes(const hqq_linear *l, int64_t M, const TilePlan &pl)
-{
-    return pl.KSP == 1 ? 0 : (((size_t)pl.KSP * (size_t)M * (size_t)l->N * sizeof(float) + 255) & ~(size_t)255);
-}
-
-size_t tile_workspace_bytes(const hqq_linear *l, int64_t M)
+// [arrival counters of the decode kernels][fp32 partial sums per layer][4-bit rewrite of 3-bit codes per layer]
+static size_t tile_job_bytes(const hqq_linear *l, int64_t M, int nl)
 {
     TilePlan pl;
     const hqq_linear v = tile_view(l);
-    if (!make_plan(&v, M, pl))
+    if (!make_plan(&v, M, pl, nl))
         return 0;
-    const size_t body = partial_bytes(l, M, pl) + rewrite_bytes(l);
+    const bool partial = pl.KSP > 1 || nl == 2;
+    const size_t one = partial ? (((size_t)pl.KSP * (size_t)M * (size_t)l->N * sizeof(float) + 255) & ~(size_t)255) : 0;
+    const size_t body = nl * (one + rewrite_bytes(l));
     return body ? workspace_head_bytes() + body : 0;
 }
 
-int launch_tile_matmul(const hqq_linear *l3, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s)
+// one layer (lb == nullptr) or the two projections of a gate: y = x W^T (+ bias), or y = silu(x Wa^T) * (x Wb^T)
+static int tile_job(const hqq_linear *la, const hqq_linear *lb, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
+                    hipStream_t s)
 {
+    const int nl = lb ? 2 : 1;
     TilePlan pl;
-    hqq_linear view = tile_view(l3);
-    const hqq_linear *l = &view;
-    if (!make_plan(l, M, pl) || (reinterpret_cast<uintptr_t>(x) & 15u))
+    hqq_linear view[2] = {tile_view(la), tile_view(lb ? lb : la)};
+    if (!make_plan(&view[0], M, pl, nl) || (reinterpret_cast<uintptr_t>(x) & 15u))
         return HQQ_E_UNSUPPORTED;
-    const size_t need = tile_workspace_bytes(l3, M);
+    if (nl == 2 && pl.kinds == 0)
+        return HQQ_E_UNSUPPORTED;
+    const size_t need = tile_job_bytes(la, M, nl);
     if (need > 0 && (!ws || ws_bytes < need))
         return HQQ_E_WORKSPACE;
-    if (l3->nbits == 3) {
-        uint8_t *codes4 = reinterpret_cast<uint8_t *>(ws) + workspace_head_bytes() + partial_bytes(l, M, pl);
-        const int64_t work = ((l3->N + 9) / 10) * (l3->K / 4);
-        const int grid = (int)(work / 256 < 1 ? 1 : (work / 256 > 8192 ? 8192 : work / 256));
-        repack3_as4_kernel<<<grid, 256, 0, s>>>(static_cast<const uint32_t *>(l3->codes), l3->N, l3->K, codes4);
-        view.codes = codes4;
+    const bool partial = pl.KSP > 1 || nl == 2;
+    const size_t one = partial ? (((size_t)pl.KSP * (size_t)M * (size_t)la->N * sizeof(float) + 255) & ~(size_t)255) : 0;
+    char *body = static_cast<char *>(ws) + workspace_head_bytes();
+    if (la->nbits == 3) {
+        const hqq_linear *src[2] = {la, lb};
+        for (int i = 0; i < nl; ++i) {
+            uint8_t *codes4 = reinterpret_cast<uint8_t *>(body + nl * one + i * rewrite_bytes(la));
+            const int64_t work = ((la->N + 9) / 10) * (la->K / 4);
+            const int grid = (int)(work / 256 < 1 ? 1 : (work / 256 > 8192 ? 8192 : work / 256));
+            repack3_as4_kernel<<<grid, 256, 0, s>>>(static_cast<const uint32_t *>(src[i]->codes), la->N, la->K, codes4);
+            view[i].codes = codes4;
+        }
     }
+    const hqq_linear *l = &view[0];
     TileParams p = {};
     p.codes = static_cast<const uint8_t *>(l->codes);
     p.sc = make_table(l->scale), p.zr = make_table(l->zero);
     p.sc_inv = l->scale.meta_cols > 0 ? (uint32_t)(0xFFFFFFFFull / (uint64_t)l->scale.meta_cols) : 0;
     p.zr_inv = l->zero.meta_cols > 0 ? (uint32_t)(0xFFFFFFFFull / (uint64_t)l->zero.meta_cols) : 0;
-    p.x = x, p.bias = static_cast<const f16 *>(l->bias), p.y = y;
+    p.codes_b = static_cast<const uint8_t *>(view[1].codes);
+    p.sc_b = make_table(view[1].scale), p.zr_b = make_table(view[1].zero);
+    p.sc_b_inv = view[1].scale.meta_cols > 0 ? (uint32_t)(0xFFFFFFFFull / (uint64_t)view[1].scale.meta_cols) : 0;
+    p.JB = pl.GP / kWaves;
+    p.part_lstride = (int64_t)(one / sizeof(float));
+    p.x = x, p.bias = nl == 1 ? static_cast<const f16 *>(l->bias) : nullptr, p.y = y;
     p.M = (int)M, p.N = (int)l->N, p.K = (int)l->K, p.GP = pl.GP, p.KT = pl.KT;
     p.KSP = pl.KSP, p.KTS = pl.KTS;
-    p.part = pl.KSP > 1 ? reinterpret_cast<float *>(static_cast<char *>(ws) + workspace_head_bytes()) : nullptr;
-    const dim3 grid((unsigned)(pl.GP / kWaves * pl.KSP), (unsigned)pl.RB, (unsigned)((M + pl.BM - 1) / pl.BM));
+    p.part = partial ? reinterpret_cast<float *>(body) : nullptr;
+    const dim3 grid((unsigned)(pl.GP / kWaves * pl.KSP * nl), (unsigned)pl.RB, (unsigned)((M + pl.BM - 1) / pl.BM));
     if (pl.kinds != 0) {
         launch_tile2(p, pl, l->nbits, grid, s);
     } else if (l->nbits == 2) {
@@ -710,14 +747,50 @@ int launch_tile_matmul(const hqq_linear *l3, const f16 *x, int64_t M, f16 *y, vo
             gemm_tile_kernel<4, 64><<<grid, kWaves * 64, 0, s>>>(p);
     }
     int rc = launch_status();
-    if (rc != HQQ_OK || pl.KSP == 1)
+    if (rc != HQQ_OK || !partial)
         return rc;
     const dim3 fgrid((unsigned)((l->N / pl.F + 15) / 16), (unsigned)((M + 15) / 16));
-    if (pl.F == 4)
-        tile_finish_kernel<4><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, p.bias, y);
-    else
-        tile_finish_kernel<2><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, p.bias, y);
+    if (nl == 2) {
+        if (pl.F == 4)
+            tile_finish_kernel<4, true><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, nullptr, y, p.part_lstride);
+        else
+            tile_finish_kernel<2, true><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, nullptr, y, p.part_lstride);
+    } else if (pl.F == 4) {
+        tile_finish_kernel<4, false><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, p.bias, y, 0);
+    } else {
+        tile_finish_kernel<2, false><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, p.bias, y, 0);
+    }
     return launch_status();
+}
+
+size_t tile_workspace_bytes(const hqq_linear *l, int64_t M) { return tile_job_bytes(l, M, 1); }
+
+int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s)
+{
+    return tile_job(l, nullptr, x, M, y, ws, ws_bytes, s);
+}
+
+// the two projections of an expert's gate in one launch, silu(a) * b applied by the finishing kernel
+bool tile_gate_supported(const hqq_linear *w1, const hqq_linear *w3, int64_t M)
+{
+    TilePlan a, b;
+    const hqq_linear va = tile_view(w1), vb = tile_view(w3);
+    return tile_supported(w1, M) && tile_supported(w3, M) && w1->N == w3->N && w1->K == w3->K && w1->nbits == w3->nbits &&
+           w1->group_size == w3->group_size && !w1->bias && !w3->bias && make_plan(&va, M, a, 2) && make_plan(&vb, M, b, 2) &&
+           a.kinds != 0 && a.kinds == b.kinds && w1->scale.meta_cols == w3->scale.meta_cols;
+}
+
+size_t tile_gate_workspace_bytes(const hqq_linear *w1, const hqq_linear *w3, int64_t M)
+{
+    return tile_gate_supported(w1, w3, M) ? tile_job_bytes(w1, M, 2) : 0;
+}
+
+int launch_tile_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
+                        size_t ws_bytes, hipStream_t s)
+{
+    if (!tile_gate_supported(w1, w3, M))
+        return HQQ_E_UNSUPPORTED;
+    return tile_job(w1, w3, x, M, h, ws, ws_bytes, s);
 }
 
 } // namespace hqq

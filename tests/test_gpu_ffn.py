@@ -37,7 +37,7 @@ def _tolerance(x, w1, w2, w3):
 
 
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "w%d_h%d_f%d_g%d_%s" % (s[0], s[1], s[2], s[3], "q" if s[4] else "f16"))
-@pytest.mark.parametrize("m", [1, 2, 3, 4, 16])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 16, 40])
 def test_expert_ffn_against_oracle(shape, m):
     from mixtral_offloading_amd import hip_kernels
     nbits, hidden, ffn, gs, qt = shape
@@ -87,7 +87,7 @@ def test_ffn_entry_point_equals_its_three_steps(m):
     assert err <= 2e-3 * steps.float().abs().max().item() + 1e-3, err
 
 
-@pytest.mark.parametrize("m", [1, 2, 4, 16])
+@pytest.mark.parametrize("m", [1, 2, 4, 8, 16, 128])
 def test_full_size_ffn_against_dequantize_then_matmul(m):
     """Mixtral shapes (2-bit g16, 4096 -> 14336 -> 4096): the library's bit-exact de-quantiser followed by torch
     matmuls with the reference's fp16 roundings."""
