@@ -234,6 +234,17 @@ def decode_section(dev, tokens_resident=256, tokens_offload=48):
             out["all_experts_resident_graph_tokens"] = tokens_resident
             del dec
             out["all_experts_resident_eager_tok_s"] = round(timed_eager(model, 48), 1)
+            # prompt processing (the multi-token kernels): a 128-token prompt through all 32 layers
+            long_prompt = torch.randint(0, cfg.vocab_size, (128,), device=dev, generator=gen)
+            cache = model.new_cache(130)
+            model.forward(long_prompt, cache, 0)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                model.forward(long_prompt, cache, 0)
+            torch.cuda.synchronize()
+            out["prefill_128_tokens_ms"] = round((time.perf_counter() - t0) / 3 * 1e3, 2)
+            del cache
         else:
             before = model.expert_cache.stats()
             out[f"expert_cache_{per_layer}_per_layer_tok_s"] = round(timed_eager(model, tokens_offload), 2)

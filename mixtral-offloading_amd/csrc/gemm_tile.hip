@@ -607,8 +607,9 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl, int nl = 1)
     pl.BM = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
     if (M > 128 && pl.kinds != 0 && ((M + 127) / 128) * (760 + 8 * 128) <= ((M + 63) / 64) * (760 + 8 * 64))
         pl.BM = 128;
-    if (const char *e = std::getenv("HQQ_TILE_BM"))
-        pl.BM = std::atoi(e);
+    if (tuning_overrides())
+        if (const char *e = std::getenv("HQQ_TILE_BM"))
+            pl.BM = std::atoi(e);
     const int64_t mtiles = (M + pl.BM - 1) / pl.BM;
     if (mtiles > 65535)
         return false;
@@ -624,8 +625,9 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl, int nl = 1)
         ksp = pl.KT / 8;
     if (ksp < 1)
         ksp = 1;
-    if (const char *e = std::getenv("HQQ_TILE_KSP"))
-        ksp = std::atoi(e);
+    if (tuning_overrides())
+        if (const char *e = std::getenv("HQQ_TILE_KSP"))
+            ksp = std::atoi(e);
     pl.KTS = (int)((pl.KT + ksp - 1) / ksp);
     pl.KSP = (pl.KT + pl.KTS - 1) / pl.KTS;
     if ((int64_t)(pl.GP / kWaves) * pl.KSP * nl > 0x7fffffff)

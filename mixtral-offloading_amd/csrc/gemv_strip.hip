@@ -605,7 +605,7 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl, int64_t ti
             KS = ((pl.NS + S - 1) / S + BK - 1) / BK;
         }
     }
-    if (env_int("HQQ_STRIP_K", (int)l->K) == (int)l->K && env_int("HQQ_STRIP_NL", NL) == NL) {
+    if (tuning_overrides() && env_int("HQQ_STRIP_K", (int)l->K) == (int)l->K && env_int("HQQ_STRIP_NL", NL) == NL) {
         S = env_int("HQQ_STRIP_S", S);
         KS = env_int("HQQ_STRIP_KS", KS);
         BK = env_int("HQQ_STRIP_BK", BK);

@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <cstdlib>
+
 #include "hqq_mi355x.h"
 
 namespace hqq {
@@ -75,6 +77,14 @@ __device__ __forceinline__ float wave_sum(float v)
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Launch shapes can be overridden through HQQ_* environment variables for experiments, but only in a process that
+// has HQQ_TUNING set when the library is first used: a normal call never reads the environment.
+inline bool tuning_overrides()
+{
+    static const bool on = std::getenv("HQQ_TUNING") != nullptr;
+    return on;
+}
 
 // launch-status helper: kernels are launched with <<<>>> and checked once
 inline int launch_status()
