@@ -14,6 +14,7 @@ from __future__ import annotations
 import copy
 from typing import Any, Dict
 
+import numpy as np
 import torch
 from torch import nn
 from torch.nn import functional as F
@@ -245,20 +246,33 @@ class SparseMoeWrapper(nn.Module):
 
         tokens = hidden_states.shape[0]
         final_hidden_states = torch.zeros((tokens, hidden_dim), dtype=hidden_states.dtype, device=hidden_states.device)
-        selected = selected_experts.tolist()  # one host sync per layer: the cache is driven from the host
-        active_experts = sorted({e for row in selected for e in row})
-
-        for (_layer_index, expert_idx), expert_layer in self.experts.load_experts(
-                *((self.layer_id, expert_idx) for expert_idx in active_experts), unordered=True):
-            if tokens == 1:
-                k = selected[0].index(expert_idx)
+        sel_host = selected_experts.cpu()  # one host sync per layer: the cache is driven from the host
+        if tokens == 1:
+            selected = sel_host[0].tolist()
+            for (_layer_index, expert_idx), expert_layer in self.experts.load_experts(
+                    *((self.layer_id, expert_idx) for expert_idx in sorted(set(selected))), unordered=True):
+                k = selected.index(expert_idx)
                 expert_layer(hidden_states, out=final_hidden_states, row_scale=routing_weights[0, k:k + 1],
                              accumulate=True)
-                continue
-            rows = [(t, row.index(expert_idx)) for t, row in enumerate(selected) if expert_idx in row]
-            top_x = torch.tensor([t for t, _ in rows], device=hidden_states.device)
-            idx = torch.tensor([k for _, k in rows], device=hidden_states.device)
-            current_state = hidden_states.index_select(0, top_x)
-            current_hidden_states = expert_layer(current_state, row_scale=routing_weights[top_x, idx])
-            final_hidden_states.index_add_(0, top_x, current_hidden_states.to(hidden_states.dtype))
+            return final_hidden_states.reshape(batch_size, sequence_length, hidden_dim), router_logits
+
+        # Several tokens: the (token, slot) pairs are grouped by expert on the host from that one copy, a single index
+        # tensor goes back to the device, the rows of every expert are gathered at once and their weighted outputs
+        # are added back with one index_add_ (reference :298-312 does a where / gather / index_add_ per expert; each
+        # token receives the same two fp16 terms, and their sum does not depend on the order).
+        flat = sel_host.reshape(-1).numpy()                     # pair p = token * top_k + slot
+        order = np.argsort(flat, kind="stable")
+        counts = np.bincount(flat, minlength=self.num_experts)
+        starts = np.concatenate(([0], np.cumsum(counts)))
+        order_dev = torch.from_numpy(order).to(hidden_states.device)
+        top_x = torch.div(order_dev, self.top_k, rounding_mode="floor")
+        scales = routing_weights.reshape(-1).index_select(0, order_dev)
+        gathered = hidden_states.index_select(0, top_x)
+        weighted = torch.empty_like(gathered)
+        active_experts = [e for e in range(self.num_experts) if counts[e] > 0]
+        for (_layer_index, expert_idx), expert_layer in self.experts.load_experts(
+                *((self.layer_id, expert_idx) for expert_idx in active_experts), unordered=True):
+            lo, hi = int(starts[expert_idx]), int(starts[expert_idx + 1])
+            expert_layer(gathered[lo:hi], out=weighted[lo:hi], row_scale=scales[lo:hi])
+        final_hidden_states.index_add_(0, top_x, weighted)
         return final_hidden_states.reshape(batch_size, sequence_length, hidden_dim), router_logits
