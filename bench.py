@@ -218,7 +218,7 @@ def decode_section(dev, tokens_resident=256, tokens_offload=48):
     for per_layer in (8, 4, 2):
         off = bm.OffloadConfig(main_size=32 * per_layer, offload_size=32 * (8 - per_layer), buffer_size=4,
                                offload_per_layer=8 - per_layer)
-        model = bm.build_model(dev, bm.default_quant_config(), off, model_config=cfg, seed=0, max_positions=512)
+        model = bm.build_model(dev, bm.default_quant_config(), off, model_config=cfg, seed=0, max_positions=1024)
         model.generate(prompt, 2)  # workspaces, allocator pools
         if per_layer == 8:
             dec = DecodeGraph(model, 64 + tokens_resident + 4)
@@ -233,6 +233,19 @@ def decode_section(dev, tokens_resident=256, tokens_offload=48):
             out["all_experts_resident_graph_tok_s"] = round(tokens_resident / (time.perf_counter() - t0), 1)
             out["all_experts_resident_graph_tokens"] = tokens_resident
             del dec
+            # the same step with a 512-token KV cache (BASELINE configs[3]): 64 tokens after a 512-token prompt
+            ctx = torch.randint(0, cfg.vocab_size, (512,), device=dev, generator=gen)
+            dec = DecodeGraph(model, 512 + 64 + 4)
+            dec.prefill(ctx)
+            dec.capture()
+            dec.prefill(ctx)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(64):
+                dec.step()
+            torch.cuda.synchronize()
+            out["all_experts_resident_graph_tok_s_kv512"] = round(64 / (time.perf_counter() - t0), 1)
+            del dec, ctx
             out["all_experts_resident_eager_tok_s"] = round(timed_eager(model, 48), 1)
             # prompt processing (the multi-token kernels): a 128-token prompt through all 32 layers
             long_prompt = torch.randint(0, cfg.vocab_size, (128,), device=dev, generator=gen)

@@ -263,8 +263,10 @@ __global__ __launch_bounds__(256) void add_rmsnorm_router_once_kernel(f16 *__res
 // output accumulated in fp32.  The current position is read from device memory, so the launch can be replayed
 // from a graph; positions 0 .. pos are attended (the new key and value are taken from registers, and also
 // written to the cache by the first head of each KV group).
-template <int HD>
-__global__ __launch_bounds__(256) void attention_decode_kernel(const f16 *__restrict__ q_in, const f16 *__restrict__ k_in,
+// One block of NT threads per head: 256 for caches of up to 512 positions, 1024 beyond (the block walks the head's
+// cache rows, so a long cache wants more threads and a short one fewer reduction steps).
+template <int HD, int NT>
+__global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restrict__ q_in, const f16 *__restrict__ k_in,
                                                                const f16 *__restrict__ v_in, const f16 *__restrict__ cos_t,
                                                                const f16 *__restrict__ sin_t, const int64_t *__restrict__ pos_p,
                                                                f16 *__restrict__ cache_k, f16 *__restrict__ cache_v,
@@ -273,8 +275,9 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const f16 *__rest
     extern __shared__ float score_lds[]; // [pos + 1]
     __shared__ __attribute__((aligned(16))) f16 q_lds[HD];
     __shared__ __attribute__((aligned(16))) f16 k_lds[HD];
-    __shared__ float red_lds[8];
-    __shared__ float acc_lds[256 / (HD / 8)][HD];
+    constexpr int NW = NT / 64;
+    __shared__ float red_lds[2 * NW];
+    __shared__ float acc_lds[NT / (HD / 8)][HD];
     const int h = blockIdx.x, kv = h / group;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t pos = pos_p[0];
@@ -298,7 +301,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const f16 *__rest
     // scores: one position per thread, the key row read as 16-byte pieces, q broadcast from LDS
     const float inv = 1.0f / __builtin_sqrtf((float)HD);
     float mx = -3.0e38f;
-    for (int64_t l = tid; l <= pos; l += 256) {
+    for (int64_t l = tid; l <= pos; l += NT) {
         const f16 *krow = l == pos ? k_lds : cache_k + ((int64_t)kv * max_len + l) * HD;
         float acc = 0.f;
 #pragma unroll
@@ -320,23 +323,29 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const f16 *__rest
     if (lane == 0)
         red_lds[wave] = mx;
     __syncthreads();
-    mx = fmaxf(fmaxf(red_lds[0], red_lds[1]), fmaxf(red_lds[2], red_lds[3]));
+    mx = red_lds[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w)
+        mx = fmaxf(mx, red_lds[w]);
     float sum = 0.f;
-    for (int64_t l = tid; l <= pos; l += 256) {
+    for (int64_t l = tid; l <= pos; l += NT) {
         const float e = __expf(score_lds[l] - mx);
         score_lds[l] = e;
         sum += e;
     }
     sum = wave_sum(sum);
     if (lane == 0)
-        red_lds[4 + wave] = sum;
+        red_lds[NW + wave] = sum;
     __syncthreads();
-    sum = red_lds[4] + red_lds[5] + red_lds[6] + red_lds[7];
+    sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w)
+        sum += red_lds[NW + w];
     const float rs = 1.0f / sum;
 
     // output: LPR threads share a value row (16 bytes each), the block covers ROWS rows per pass and four passes
     // are in flight; the ROWS partial outputs meet in LDS
-    constexpr int LPR = HD / 8, ROWS = 256 / LPR;
+    constexpr int LPR = HD / 8, ROWS = NT / LPR;
     const int rsub = tid / LPR, c8 = tid % LPR;
     float o[8];
 #pragma unroll
@@ -386,10 +395,14 @@ int launch_attention_decode(const f16 *q, const f16 *k, const f16 *v, const f16 
         return HQQ_E_ALIGN;
     const size_t lds = (size_t)max_len * sizeof(float);
     const int group = n_heads / n_kv_heads;
-    if (head_dim == 128)
-        attention_decode_kernel<128><<<n_heads, 256, lds, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len, group, out);
+    if (head_dim == 128 && max_len <= 512)
+        attention_decode_kernel<128, 256><<<n_heads, 256, lds, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len, group, out);
+    else if (head_dim == 128)
+        attention_decode_kernel<128, 1024><<<n_heads, 1024, lds, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len, group, out);
+    else if (max_len <= 512)
+        attention_decode_kernel<64, 256><<<n_heads, 256, lds, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len, group, out);
     else
-        attention_decode_kernel<64><<<n_heads, 256, lds, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len, group, out);
+        attention_decode_kernel<64, 1024><<<n_heads, 1024, lds, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len, group, out);
     return launch_status();
 }
 

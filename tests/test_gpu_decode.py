@@ -219,14 +219,16 @@ def test_graph_decode_refuses_offloaded_experts():
         DecodeGraph(model, 32)
 
 
-@pytest.mark.parametrize("heads,kv,hd,pos", [(32, 8, 128, 0), (32, 8, 128, 37), (32, 8, 128, 511), (4, 2, 64, 5), (8, 8, 64, 300)])
-def test_attention_decode_against_torch_ops(heads, kv, hd, pos):
+@pytest.mark.parametrize("heads,kv,hd,pos,L", [(32, 8, 128, 0, 512), (32, 8, 128, 37, 512), (32, 8, 128, 511, 512),
+                                               (4, 2, 64, 5, 512), (8, 8, 64, 300, 512),
+                                               # caches past 512 positions run the 1024-thread form of the kernel
+                                               (32, 8, 128, 3, 2048), (32, 8, 128, 1500, 2048), (8, 8, 64, 1100, 1200)])
+def test_attention_decode_against_torch_ops(heads, kv, hd, pos, L):
     """Same roundings as the harness's torch attention (rope terms, fp16 scores, fp32 softmax, fp16 probabilities)."""
     import math
     from mixtral_offloading_amd import hip_kernels
     from mixtral_offloading_amd.mixtral_model import Rotary
     g = torch.Generator(device="cuda").manual_seed(heads + pos)
-    L = 512
     rot = Rotary(hd, L, 1e6, torch.device("cuda"))
     q = torch.randn((1, heads * hd), device="cuda", generator=g).half()
     k = torch.randn((1, kv * hd), device="cuda", generator=g).half()
