@@ -161,6 +161,14 @@ size_t hqq_matmul_group_workspace_bytes(const hqq_linear *const *layers, int32_t
 int hqq_matmul_group(const hqq_linear *const *layers, int32_t count, const void *x_f16, void *const *ys_f16,
                      void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- hqq_add_rmsnorm folded into hqq_matmul_group: ys[i] = (norm_weight * rmsnorm(x + delta)) @ dequant(layers[i]).T,
+ *      and x + delta is written to x_sum (a buffer other than x: every block reads x while one writes x_sum).  The
+ *      input norm of a decoder layer and its q / k / v projections in one launch; delta may be NULL.  Results are
+ *      those of hqq_add_rmsnorm followed by hqq_matmul_group, bit for bit.  All pointers 16-byte aligned.          */
+int hqq_matmul_group_norm(const hqq_linear *const *layers, int32_t count, const void *x_f16, const void *delta_f16,
+                          const void *norm_weight_f16, float eps, void *x_sum_f16, void *const *ys_f16, void *workspace,
+                          size_t workspace_bytes, void *stream);
+
 /* ---- router of one token: logits = fp16(x W^T), fp32 softmax, the two largest probabilities renormalised and cast
  *      to fp16 (src/custom_layers.py:276-282), written to device memory: sel_out[2] expert indices (largest
  *      first), weights_f16_out[2]; logits_f16_out[n_experts] when not NULL.  n_experts <= 16.                       */

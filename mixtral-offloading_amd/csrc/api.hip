@@ -426,6 +426,36 @@ int hqq_matmul_group(const hqq_linear *const *layers, int32_t count, const void 
                               workspace_bytes, (hipStream_t)stream);
 }
 
+int hqq_matmul_group_norm(const hqq_linear *const *layers, int32_t count, const void *x_f16, const void *delta_f16,
+                          const void *norm_weight_f16, float eps, void *x_sum_f16, void *const *ys_f16, void *workspace,
+                          size_t workspace_bytes, void *stream)
+{
+    if (!layers || !ys_f16 || !x_f16 || !norm_weight_f16 || !x_sum_f16)
+        return HQQ_E_NULL;
+    if (count < 1 || count > 4)
+        return HQQ_E_SHAPE;
+    int rc;
+    for (int i = 0; i < count; ++i) {
+        if ((rc = validate_linear(layers[i])) != HQQ_OK)
+            return rc;
+        if (!ys_f16[i])
+            return HQQ_E_NULL;
+        if (layers[i]->K != layers[0]->K)
+            return HQQ_E_SHAPE;
+    }
+    const size_t need = strip_job_workspace_bytes(layers, count, 1, 1);
+    if (need == 0)
+        return HQQ_E_UNSUPPORTED;
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return HQQ_E_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(x_f16) | reinterpret_cast<uintptr_t>(delta_f16) |
+         reinterpret_cast<uintptr_t>(norm_weight_f16) | reinterpret_cast<uintptr_t>(x_sum_f16)) & 15u)
+        return HQQ_E_ALIGN;
+    const StripNorm norm = {(const f16 *)delta_f16, (const f16 *)norm_weight_f16, (f16 *)x_sum_f16, eps};
+    return launch_strip_group(layers, count, (const f16 *)x_f16, reinterpret_cast<f16 *const *>(ys_f16), workspace,
+                              workspace_bytes, (hipStream_t)stream, &norm);
+}
+
 int hqq_router_top2(const void *x_f16, const void *gate_w_f16, int32_t n_experts, int64_t hidden, int32_t *sel_out,
                     void *weights_f16_out, void *logits_f16_out, void *stream)
 {

@@ -69,6 +69,11 @@ struct StripParams {
     const f16 *row_scale;
     int rs_lstride; // EPI 2: layer l scales by row_scale[l * rs_lstride + m]
     int accumulate;
+    // NORM launches: the activations are weight * rmsnorm(x + delta) of the single row x (delta may be null), computed
+    // by every block for itself; block (0, 0, 0) also writes x + delta to x_sum.
+    const f16 *norm_delta, *norm_weight;
+    f16 *x_sum;
+    float norm_eps;
 };
 
 template <int MT, int SKIND, int ZKIND> struct SlabRegs {
@@ -79,12 +84,14 @@ template <int MT, int SKIND, int ZKIND> struct SlabRegs {
     u32x4 xw[MT <= 2 ? (MT + 1) / 2 : 2 * MT];
     u32x4 cw[4];             // codes: load i holds rows 4i .. 4i+3 of the tile, 16 lanes x 16 bytes per row
     uint32_t sms, smz, zms, zmz; // whole-tensor meta values, raw fp16 bits
+    u32x4 xd, xg;            // NORM launches: the slab's pieces of delta and of the norm weight
 };
 
 // EPI: 0 y = o (+ bias) (* row_scale) (+ y);  1 y = silu(o0) * o1;  2 y = (y +) o0 * row_scale[0] + o1 * row_scale[1]
-template <int NBITS, int MT, int S, int D, int WAVES, int SKIND, int ZKIND, int EPI, bool GROUPED = false>
+template <int NBITS, int MT, int S, int D, int WAVES, int SKIND, int ZKIND, int EPI, bool GROUPED = false, bool NORM = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
 {
+    static_assert(!NORM || (MT == 1 && WAVES >= 4), "the fused norm is for single rows and blocks of four waves and more");
     constexpr int F = 8 / NBITS;
     constexpr int ENTRY = 8; // halves per B-operand entry (16 bytes)
     constexpr int STEP_HALVES = F * 2 * 4 * MT * ENTRY;
@@ -100,6 +107,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     __shared__ __attribute__((aligned(16))) float red_lds[WAVES][16][MT][F];
     __shared__ __attribute__((aligned(16))) float fin_lds[2][16][MT][F];
     __shared__ int ticket_lds;
+    __shared__ float norm_lds[4];
 
     const int lane = threadIdx.x & 63;
     // the wave index as a scalar: what depends on it (the layer, its record, the K range) then lives in scalar
@@ -189,6 +197,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
                 m = m < M ? m : 0;
                 r.xw[j] = gload<u32x4>(xl + (k0 + (uint32_t)(8 * (lane & 31)) + (uint32_t)(m * K)));
             }
+            if constexpr (NORM) {
+                r.xg = gload<u32x4>(p.norm_weight + (k0 + (uint32_t)(8 * (lane & 31))));
+                r.xd = p.norm_delta ? gload<u32x4>(p.norm_delta + (k0 + (uint32_t)(8 * (lane & 31)))) : (u32x4){0, 0, 0, 0};
+            }
         } else {
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
@@ -230,14 +242,28 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
 #pragma unroll
     for (int m = 0; m < MT; ++m)
         bias_acc[m] = 0.f;
+    float rnorm = 1.0f; // NORM launches: 1 / sqrt(mean(x^2) + eps), known once the block has added the row up
 
     uint8_t *code_w = &code_lds[wave][0];
     auto compute = [&](const SlabRegs<MT, SKIND, ZKIND> &r) __attribute__((always_inline)) {
         // ------------------------------------------------------------ staging: x and the codes change lanes through LDS
         if constexpr (STAGE) {
 #pragma unroll
-            for (int j = 0; j < (MT + 1) / 2; ++j)
-                *reinterpret_cast<u32x4 *>(&xw_lds[wave][2 * j + (lane >> 5)][8 * (lane & 31)]) = r.xw[j];
+            for (int j = 0; j < (MT + 1) / 2; ++j) {
+                u32x4 xv = r.xw[j];
+                if constexpr (NORM) { // weight * fp16(fp32(x + delta) * r): the roundings of the stand-alone norm kernel
+                    f16x8 v = __builtin_bit_cast(f16x8, xv);
+                    if (p.norm_delta)
+                        v = v + __builtin_bit_cast(f16x8, r.xd);
+                    const f16x8 g = __builtin_bit_cast(f16x8, r.xg);
+                    f16x8 o;
+#pragma unroll
+                    for (int t = 0; t < 8; ++t)
+                        o[t] = g[t] * (f16)((float)v[t] * rnorm);
+                    xv = __builtin_bit_cast(u32x4, o);
+                }
+                *reinterpret_cast<u32x4 *>(&xw_lds[wave][2 * j + (lane >> 5)][8 * (lane & 31)]) = xv;
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i)
                 *reinterpret_cast<u32x4 *>(code_w + (4 * i + lrow) * CODE_PITCH + 16 * lchunk) = r.cw[i];
@@ -322,12 +348,64 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     // ---------------------------------------------------------------- S slabs, D of them in flight
     // A slab past the end of K is issued all the same (it re-reads the last slab and is never used): with a fixed
     // number of loads the compiler waits for exactly the loads a slab needs and leaves the later ones in flight.
+    SlabRegs<MT, SKIND, ZKIND> regs[D];
+    const int last = p.NS - 1;
+    // NORM launches: the row (x + delta) for the mean of squares is requested first, by the first four waves, two
+    // pieces of eight elements per thread and pass (rows of up to 4096 elements take one pass); loads retire in issue
+    // order, so these must go out before the weights for the sum to be ready while the weights still travel.
+    constexpr int NPIECE = 2;
+    f16x8 nv[NPIECE];
+    if constexpr (NORM) {
+#pragma unroll
+        for (int c = 0; c < NPIECE; ++c) {
+            const int k = ((int)threadIdx.x + c * 256) * 8;
+            const int kc = threadIdx.x < 256 && k < K ? k : 0;
+            nv[c] = gload<f16x8>(p.x + kc);
+            if (p.norm_delta)
+                nv[c] = nv[c] + gload<f16x8>(p.norm_delta + kc);
+        }
+    }
     if (wave_on) {
-        SlabRegs<MT, SKIND, ZKIND> regs[D];
-        const int last = p.NS - 1;
 #pragma unroll
         for (int i = 0; i < D; ++i)
             issue(regs[i], slab0 + i < p.NS ? slab0 + i : last);
+    }
+    if constexpr (NORM) {
+        // the sum in the order the stand-alone norm kernel adds it (256 threads, 8 elements each per pass), so that both
+        // give the same bits
+        float ss = 0.f;
+        if (threadIdx.x < 256) {
+            const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0;
+#pragma unroll
+            for (int c = 0; c < NPIECE; ++c) {
+                const int k = ((int)threadIdx.x + c * 256) * 8;
+                if (k < K) {
+                    if (writer)
+                        *reinterpret_cast<f16x8 *>(p.x_sum + k) = nv[c];
+#pragma unroll
+                    for (int t = 0; t < 8; ++t)
+                        ss += (float)nv[c][t] * (float)nv[c][t];
+                }
+            }
+            for (int k = ((int)threadIdx.x + NPIECE * 256) * 8; k < K; k += 256 * 8) { // longer rows: the rest, late
+                f16x8 v = gload<f16x8>(p.x + k);
+                if (p.norm_delta)
+                    v = v + gload<f16x8>(p.norm_delta + k);
+                if (writer)
+                    *reinterpret_cast<f16x8 *>(p.x_sum + k) = v;
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    ss += (float)v[t] * (float)v[t];
+            }
+            ss = wave_sum(ss);
+            if (lane == 0)
+                norm_lds[wave] = ss;
+        }
+        __syncthreads();
+        const float mean = (norm_lds[0] + norm_lds[1] + norm_lds[2] + norm_lds[3]) / (float)K;
+        rnorm = 1.0f / __builtin_sqrtf(mean + p.norm_eps);
+    }
+    if (wave_on) {
 #pragma unroll
         for (int i = 0; i < S; ++i) {
             if (slab0 + i < p.NS)
@@ -640,6 +718,15 @@ void fill_layer(StripLayer &L, const hqq_linear *l)
 template <int NBITS, int MT, int S, int D, int WAVES, int EPI, bool GROUPED>
 void launch_kinds(const StripParams &p, const StripPlan &pl, dim3 grid, hipStream_t s)
 {
+    if constexpr (GROUPED && EPI == 0 && MT == 1 && WAVES >= 4) {
+        if (p.norm_weight) { // the fused norm exists for the grouped single-row projections only
+            if (pl.SKIND == TK_F16)
+                gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_F16, TK_F16, EPI, true, true><<<grid, dim3(WAVES * 64), 0, s>>>(p);
+            else
+                gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_U8_COLS, TK_U8_SCALAR, EPI, true, true><<<grid, dim3(WAVES * 64), 0, s>>>(p);
+            return;
+        }
+    }
     if (pl.SKIND == TK_F16)
         gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_F16, TK_F16, EPI, GROUPED><<<grid, dim3(WAVES * 64), 0, s>>>(p);
     else
@@ -700,6 +787,9 @@ struct StripJob {
     f16 *y[kMaxGroups];
     const f16 *row_scale;
     int rs_lstride, accumulate;
+    const f16 *norm_delta, *norm_weight; // norm_weight != null: activations = norm_weight * rmsnorm(x + norm_delta)
+    f16 *x_sum;
+    float norm_eps;
 };
 
 bool same_family(const hqq_linear *a, const hqq_linear *b)
@@ -786,9 +876,15 @@ int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t
     p.RB = pl.RB, p.NS = pl.NS, p.KS = pl.KS, p.BK = pl.BK, p.NL = j.NL;
     p.counter = reinterpret_cast<int *>(base);
     p.row_scale = j.row_scale, p.rs_lstride = j.rs_lstride, p.accumulate = j.accumulate;
+    if (j.norm_weight) {
+        // every launch shape the planner can pick for this job has the fused-norm form except blocks under four waves
+        if (j.EPI != 0 || j.NL != 1 || M != 1 || pl.WAVES < 4 || !j.x_sum)
+            return HQQ_E_UNSUPPORTED;
+        p.norm_delta = j.norm_delta, p.norm_weight = j.norm_weight, p.x_sum = j.x_sum, p.norm_eps = j.norm_eps;
+    }
     const dim3 grid((unsigned)pl.BK, (unsigned)pl.RB, (unsigned)z);
     const bool two = j.shape[0]->nbits == 2;
-    if (j.NG > 1) {
+    if (j.NG > 1 || j.norm_weight) {
         if (j.EPI == 0 && j.NL == 1)
             two ? launch_batch<2, 0, true>(p, pl, grid, s) : launch_batch<4, 0, true>(p, pl, grid, s);
         else if (j.EPI == 1 && j.NL == 2)
@@ -869,8 +965,9 @@ int launch_strip_down_pair(const hqq_linear *w2, const f16 *h0, int64_t h_stride
 }
 
 // Up to four projections of the same K, code width and group size applied to the same single row in one launch.
+// With norm: the row is norm->weight * rmsnorm(x + norm->delta), and x + delta is written to norm->x_sum.
 int launch_strip_group(const hqq_linear *const *layers, int count, const f16 *x, f16 *const *ys, void *ws,
-                       size_t ws_bytes, hipStream_t s)
+                       size_t ws_bytes, hipStream_t s, const StripNorm *norm)
 {
     if (count < 1 || count > kMaxGroups)
         return HQQ_E_UNSUPPORTED;
@@ -878,6 +975,11 @@ int launch_strip_group(const hqq_linear *const *layers, int count, const f16 *x,
     for (int g = 0; g < count; ++g)
         j.shape[g] = layers[g], j.y[g] = ys[g];
     j.NG = count, j.NL = 1, j.EPI = 0, j.x = x;
+    if (norm) {
+        if (!norm->weight || !norm->x_sum || layers[0]->K % 8 != 0)
+            return HQQ_E_UNSUPPORTED;
+        j.norm_delta = norm->delta, j.norm_weight = norm->weight, j.x_sum = norm->x_sum, j.norm_eps = norm->eps;
+    }
     return run_job(j, 1, ws, ws_bytes, s);
 }
 

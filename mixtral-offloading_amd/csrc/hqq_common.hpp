@@ -130,8 +130,15 @@ int launch_strip_gate_up_pair(const hqq_linear *w1, const hqq_linear *w3, const 
                               size_t ws_bytes, hipStream_t s, const StripIndex &ix);
 int launch_strip_down_pair(const hqq_linear *w2, const f16 *h0, int64_t h_stride, f16 *y, const f16 *row_scale,
                            int accumulate, void *ws, size_t ws_bytes, hipStream_t s, const StripIndex &ix);
+// residual add and RMSNorm folded into a grouped launch: the row is weight * rmsnorm(x + delta) (delta may be null)
+// and x + delta goes to x_sum
+struct StripNorm {
+    const f16 *delta, *weight;
+    f16 *x_sum;
+    float eps;
+};
 int launch_strip_group(const hqq_linear *const *layers, int count, const f16 *x, f16 *const *ys, void *ws,
-                       size_t ws_bytes, hipStream_t s);
+                       size_t ws_bytes, hipStream_t s, const StripNorm *norm = nullptr);
 size_t strip_job_workspace_bytes(const hqq_linear *const *layers, int count, int NL, int64_t M);
 int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s);
 size_t workspace_head_bytes();

@@ -63,6 +63,8 @@ _SIGNATURES = {
                                             c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
     "hqq_matmul_group_workspace_bytes": (c_size_t, [_P(_P(HqqLinear)), c_int32]),
     "hqq_matmul_group": (c_int, [_P(_P(HqqLinear)), c_int32, c_void_p, _P(c_void_p), c_void_p, c_size_t, c_void_p]),
+    "hqq_matmul_group_norm": (c_int, [_P(_P(HqqLinear)), c_int32, c_void_p, c_void_p, c_void_p, ctypes.c_float, c_void_p,
+                                      _P(c_void_p), c_void_p, c_size_t, c_void_p]),
     "hqq_router_top2": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "hqq_add_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, ctypes.c_float, c_void_p, c_int64, c_void_p]),
     "hqq_add_rmsnorm_router": (c_int, [c_void_p, c_void_p, c_void_p, ctypes.c_float, c_void_p, c_int64, c_void_p, c_int32,

@@ -282,6 +282,25 @@ class LinearGroup:
         return outs
 
 
+def matmul_group_norm(group: LinearGroup, x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
+                      eps: float, x_sum: torch.Tensor):
+    """``add_rmsnorm`` folded into the grouped launch: returns the group's outputs for the row
+    ``weight * rmsnorm(x + delta)`` and writes ``x + delta`` to ``x_sum`` (which must not be ``x``)."""
+    d0 = group.descs[0]
+    assert x.dtype == torch.float16 and x.is_contiguous() and x.numel() == d0.K and x.device == d0.device
+    assert x_sum.dtype == torch.float16 and x_sum.numel() == d0.K and x_sum.data_ptr() != x.data_ptr()
+    assert weight.dtype == torch.float16 and weight.numel() == d0.K
+    outs = [torch.empty((1, d.N), device=x.device, dtype=torch.float16) for d in group.descs]
+    ys = (ctypes.c_void_p * len(outs))(*[o.data_ptr() for o in outs])
+    with torch.cuda.device(x.device):
+        ws = workspace(x.device, group.need)
+        _lib.check(_lib.lib.hqq_matmul_group_norm(group._ptrs, len(outs), x.data_ptr(),
+                                                  delta.data_ptr() if delta is not None else None, weight.data_ptr(),
+                                                  float(eps), x_sum.data_ptr(), ys, ws.data_ptr(), ws.numel(),
+                                                  _lib.current_stream_ptr(x.device)), "hqq_matmul_group_norm")
+    return outs
+
+
 def router_top2(x: torch.Tensor, gate_weight: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
                 logits: Optional[torch.Tensor] = None) -> None:
     """Router of one token into device tensors ``sel`` (int32[2]) and ``weights`` (fp16[2])

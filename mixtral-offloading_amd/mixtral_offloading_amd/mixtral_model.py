@@ -148,6 +148,7 @@ class DecodeGraph:
         self.pos = torch.zeros(1, dtype=torch.int64, **mk)
         self.arange = torch.arange(max_len, **mk)
         self.x = torch.zeros((1, cfg.hidden_size), dtype=torch.float16, **mk)
+        self.x2 = torch.zeros_like(self.x)
         self.xn = torch.zeros_like(self.x)
         self.moe = torch.zeros_like(self.x)
         self.att = torch.zeros((1, cfg.num_attention_heads * (cfg.hidden_size // cfg.num_attention_heads)), dtype=torch.float16, **mk)
@@ -165,15 +166,17 @@ class DecodeGraph:
         hd = cfg.hidden_size // H
         g = H // KV
         eps = cfg.rms_norm_eps
-        x = self.x
+        x, spare = self.x, self.x2  # the residual stream alternates between two buffers where the norm is fused
         x.copy_(m.model.embed_tokens(self.tok))
         delta = None
         for layer, (ck, cv), table, qkv in zip(m.model.layers, self.cache, self.tables, self.qkv):
             attn = layer.self_attn
-            hip_kernels.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps, self.xn)
             if qkv.supported:
-                q, k, v = qkv(self.xn)
+                # residual add, input norm and the three projections in one launch
+                q, k, v = hip_kernels.matmul_group_norm(qkv, x, delta, layer.input_layernorm.weight, eps, spare)
+                x, spare = spare, x
             else:
+                hip_kernels.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps, self.xn)
                 q, k, v = attn.q_proj(self.xn), attn.k_proj(self.xn), attn.v_proj(self.xn)
             out = hip_kernels.attention_decode(q, k, v, m.rotary.cos, m.rotary.sin, self.pos, ck, cv, self.att)
             attn_out = attn.o_proj(out)

@@ -170,6 +170,31 @@ def test_matmul_group_equals_single_calls(nbits, gs, k, ns, bias):
             assert float((err > 0).float().mean()) < 0.2
 
 
+@pytest.mark.parametrize("nbits,gs,k,ns", [(4, 64, 4096, (4096, 1024, 1024)), (4, 64, 1024, (512, 128, 128)),
+                                           (2, 16, 512, (256, 64))])
+@pytest.mark.parametrize("with_delta", [False, True])
+def test_matmul_group_norm_equals_norm_then_group(nbits, gs, k, ns, with_delta):
+    """Residual add and RMSNorm folded into the grouped launch: the bits of hqq_add_rmsnorm followed by
+    hqq_matmul_group, and x + delta in the second buffer."""
+    from mixtral_offloading_amd import hip_kernels
+    rng = np.random.default_rng(k + len(ns) + with_delta)
+    descs = [desc_of(o.random_layer(rng, n, k, nbits, gs)[0]) for n in ns]
+    group = hip_kernels.LinearGroup(descs)
+    assert group.supported
+    for rep in range(3):
+        x = to_dev(rng.standard_normal((1, k)).astype(np.float16))
+        d = to_dev(rng.standard_normal((1, k)).astype(np.float16)) if with_delta else None
+        w = to_dev((1 + 0.1 * rng.standard_normal(k)).astype(np.float16))
+        x_ref, xn = x.clone(), torch.empty_like(x)
+        hip_kernels.add_rmsnorm(x_ref, d, w, 1e-5, xn)
+        want = group(xn)
+        x_sum = torch.full_like(x, float("nan"))
+        got = hip_kernels.matmul_group_norm(group, x, d, w, 1e-5, x_sum)
+        assert torch.equal(x_sum, x_ref)
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+
+
 def test_matmul_group_refuses_mixed_layers():
     from mixtral_offloading_amd import hip_kernels
     rng = np.random.default_rng(3)
