@@ -152,6 +152,17 @@ int hqq_expert_pair_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, cons
                                 const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
                                 void *stream);
 
+/* ---- the whole MoE block of one token in two launches: hqq_add_rmsnorm_router followed by
+ *      hqq_expert_pair_ffn_indexed, with the norm and the router run by every block of the first launch in front of
+ *      the gates (src/custom_layers.py:276-312 after the decoder layer's post-attention norm).  x + delta is written to
+ *      x_sum (a buffer other than x), the router's choice to sel_out[2] and weights_f16_out[2] (device memory),
+ *      y (+)= the weighted sum of the two experts' outputs.  hidden <= 4096, n_experts <= 8; workspace as
+ *      hqq_expert_pair_ffn_workspace_bytes.  Results are those of the two calls it replaces, bit for bit.           */
+int hqq_moe_pair_routed(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *device_table,
+                        const void *x_f16, const void *delta_f16, const void *norm_weight_f16, float eps, void *x_sum_f16,
+                        const void *gate_w_f16, int32_t n_experts, int32_t *sel_out, void *weights_f16_out, void *y_f16,
+                        int accumulate, void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- up to four HQQLinearTritonSavable.forward_triton calls (src/custom_layers.py:100-118) on the same single row
  *      in one launch: ys[i] = x @ dequant(layers[i]).T (+ bias).  The layers share K, code width, group size and
  *      table kinds but not N -- the q, k and v projections of an attention block.  Results are those of

@@ -391,6 +391,44 @@ int hqq_expert_pair_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, cons
                                   mm_bytes, s, down);
 }
 
+int hqq_moe_pair_routed(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *device_table,
+                        const void *x_f16, const void *delta_f16, const void *norm_weight_f16, float eps, void *x_sum_f16,
+                        const void *gate_w_f16, int32_t n_experts, int32_t *sel_out, void *weights_f16_out, void *y_f16,
+                        int accumulate, void *workspace, size_t workspace_bytes, void *stream)
+{
+    int rc;
+    if ((rc = validate_linear(w1)) != HQQ_OK || (rc = validate_linear(w2)) != HQQ_OK ||
+        (rc = validate_linear(w3)) != HQQ_OK)
+        return rc;
+    if (w1->N != w3->N || w1->K != w3->K || w2->K != w1->N || w2->N != w1->K)
+        return HQQ_E_SHAPE;
+    if (!x_f16 || !y_f16 || !device_table || !norm_weight_f16 || !x_sum_f16 || !gate_w_f16 || !sel_out || !weights_f16_out)
+        return HQQ_E_NULL;
+    if (n_experts < 2 || n_experts > 8 || w1->K > 4096 || w1->K % 8 != 0)
+        return HQQ_E_UNSUPPORTED;
+    if ((reinterpret_cast<uintptr_t>(x_f16) | reinterpret_cast<uintptr_t>(delta_f16) | reinterpret_cast<uintptr_t>(gate_w_f16) |
+         reinterpret_cast<uintptr_t>(norm_weight_f16) | reinterpret_cast<uintptr_t>(x_sum_f16)) & 15u)
+        return HQQ_E_ALIGN;
+    const size_t mm_bytes = pair_scratch(w1, w2, w3);
+    if (mm_bytes == 0)
+        return HQQ_E_UNSUPPORTED;
+    if (!workspace || workspace_bytes < hqq_expert_pair_ffn_workspace_bytes(w1, w2, w3) ||
+        (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return HQQ_E_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    char *p = static_cast<char *>(workspace);
+    const size_t mid = align256((size_t)w1->N * 2);
+    f16 *h0 = (f16 *)(p + mm_bytes), *h1 = (f16 *)(p + mm_bytes + mid);
+    // the first launch chooses the experts and leaves its choice in sel_out, which the second one reads
+    const StripIndex gate = {device_table, nullptr, 3, 0}, down = {device_table, sel_out, 3, 2};
+    const StripNorm norm = {(const f16 *)delta_f16, (const f16 *)norm_weight_f16, (f16 *)x_sum_f16, eps};
+    if ((rc = launch_strip_gate_up_pair_routed(w1, w3, (const f16 *)x_f16, norm, (const f16 *)gate_w_f16, n_experts, sel_out,
+                                               (f16 *)weights_f16_out, h0, h1, p, mm_bytes, s, gate)) != HQQ_OK)
+        return rc;
+    return launch_strip_down_pair(w2, h0, (int64_t)(mid / 2), (f16 *)y_f16, (const f16 *)weights_f16_out, accumulate, p,
+                                  mm_bytes, s, down);
+}
+
 size_t hqq_matmul_group_workspace_bytes(const hqq_linear *const *layers, int32_t count)
 {
     if (!layers || count < 1 || count > 4)

@@ -1,42 +1,10 @@
 // Small decode-step kernels around the quantized linears: the router (reference src/custom_layers.py:276-282)
 // and the residual add + RMSNorm of the decoder layer.  One block each: at batch 1 they are latency, not bandwidth.
 #include "hqq_common.hpp"
+#include "norm_route.hpp"
 
 namespace hqq {
 namespace {
-
-constexpr int kMaxExperts = 16;
-
-// softmax over the fp16-rounded logits in fp32, the two largest probabilities renormalised by their sum and cast to
-// fp16 (reference src/custom_layers.py:277-282); one thread.
-__device__ void route_top2(const float *logit_lds, int n_experts, int *__restrict__ sel, f16 *__restrict__ weights,
-                           f16 *__restrict__ logits_out)
-{
-    float mx = logit_lds[0];
-    for (int i = 1; i < n_experts; ++i)
-        mx = fmaxf(mx, logit_lds[i]);
-    float prob[kMaxExperts], sum = 0.f;
-    for (int i = 0; i < n_experts; ++i) {
-        prob[i] = __expf(logit_lds[i] - mx);
-        sum += prob[i];
-    }
-    int b0 = 0, b1 = -1;
-    for (int i = 0; i < n_experts; ++i) {
-        prob[i] /= sum;
-        if (logits_out)
-            logits_out[i] = (f16)logit_lds[i];
-    }
-    for (int i = 1; i < n_experts; ++i)
-        if (prob[i] > prob[b0])
-            b0 = i;
-    for (int i = 0; i < n_experts; ++i)
-        if (i != b0 && (b1 < 0 || prob[i] > prob[b1]))
-            b1 = i;
-    const float tot = prob[b0] + prob[b1];
-    sel[0] = b0, sel[1] = b1;
-    weights[0] = (f16)(prob[b0] / tot);
-    weights[1] = (f16)(prob[b1] / tot);
-}
 
 // logits = fp16(x W^T) (fp32 accumulation, one rounding, as a half linear does); softmax in fp32; the two largest
 // probabilities, renormalised by their sum, cast to fp16 (reference src/custom_layers.py:277-282).
@@ -45,6 +13,7 @@ __global__ __launch_bounds__(64 * kMaxExperts) void router_top2_kernel(const f16
                                                                        f16 *__restrict__ weights, f16 *__restrict__ logits_out)
 {
     __shared__ float logit_lds[kMaxExperts];
+    __shared__ float prob_lds[kMaxExperts];
     const int lane = threadIdx.x & 63, e = threadIdx.x >> 6;
     if (e < n_experts) {
         const f16 *row = w + (int64_t)e * hidden;
@@ -61,8 +30,8 @@ __global__ __launch_bounds__(64 * kMaxExperts) void router_top2_kernel(const f16
             logit_lds[e] = (float)(f16)acc;
     }
     __syncthreads();
-    if (threadIdx.x == 0)
-        route_top2(logit_lds, n_experts, sel, weights, logits_out);
+    if (threadIdx.x < kMaxExperts)
+        route_top2(logit_lds, prob_lds, n_experts, sel, weights, logits_out);
 }
 
 // x += delta (fp16 add, when delta is given; x is written back), then y = weight * fp16(x * rsqrt(mean(x^2) + eps))
@@ -113,6 +82,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_router_kernel(f16 *__restrict
     __shared__ float part_lds[4];
     __shared__ float dot_lds[4][kMaxExperts];
     __shared__ float logit_lds[kMaxExperts];
+    __shared__ float prob_lds[kMaxExperts];
     const int tid = threadIdx.x;
     float ss = 0.f;
     for (int k = tid * 8; k < hidden; k += 256 * 8) {
@@ -165,8 +135,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_router_kernel(f16 *__restrict
     if (tid < n_experts)
         logit_lds[tid] = (float)(f16)(dot_lds[0][tid] + dot_lds[1][tid] + dot_lds[2][tid] + dot_lds[3][tid]);
     __syncthreads();
-    if (tid == 0)
-        route_top2(logit_lds, n_experts, sel, weights, logits_out);
+    if (tid < kMaxExperts)
+        route_top2(logit_lds, prob_lds, n_experts, sel, weights, logits_out);
 }
 
 // The same computation for hidden <= CH * 2048 and at most NE experts with every global load issued before the
@@ -180,81 +150,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_router_once_kernel(f16 *__res
                                                                       int *__restrict__ sel, f16 *__restrict__ weights,
                                                                       f16 *__restrict__ logits_out)
 {
-    __shared__ float part_lds[4];
-    __shared__ float dot_lds[NE][256 + 4];
-    __shared__ float logit_lds[kMaxExperts];
-    const int tid = threadIdx.x;
-    f16x8 xv[CH], wv[CH], gv[CH][NE];
-    bool on[CH];
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int k = (c * 256 + tid) * 8;
-        on[c] = k < hidden;
-        const int kc = on[c] ? k : 0;
-        xv[c] = *reinterpret_cast<const f16x8 *>(x + kc);
-        if (delta)
-            xv[c] = xv[c] + *reinterpret_cast<const f16x8 *>(delta + kc);
-        wv[c] = *reinterpret_cast<const f16x8 *>(weight + kc);
-#pragma unroll
-        for (int e = 0; e < NE; ++e)
-            gv[c][e] = *reinterpret_cast<const f16x8 *>(gate_w + (int64_t)(e < n_experts ? e : 0) * hidden + kc);
-    }
-    float ss = 0.f;
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        if (on[c]) {
-            if (delta)
-                *reinterpret_cast<f16x8 *>(x + (c * 256 + tid) * 8) = xv[c];
-#pragma unroll
-            for (int t = 0; t < 8; ++t)
-                ss += (float)xv[c][t] * (float)xv[c][t];
-        }
-    }
-    ss = wave_sum(ss);
-    if ((tid & 63) == 0)
-        part_lds[tid >> 6] = ss;
-    __syncthreads();
-    const float mean = (part_lds[0] + part_lds[1] + part_lds[2] + part_lds[3]) / (float)hidden;
-    const float r = 1.0f / __builtin_sqrtf(mean + eps);
-    float dot[NE];
-#pragma unroll
-    for (int e = 0; e < NE; ++e)
-        dot[e] = 0.f;
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        if (on[c]) {
-            f16x8 o;
-#pragma unroll
-            for (int t = 0; t < 8; ++t)
-                o[t] = wv[c][t] * (f16)((float)xv[c][t] * r);
-            *reinterpret_cast<f16x8 *>(y + (c * 256 + tid) * 8) = o;
-#pragma unroll
-            for (int e = 0; e < NE; ++e)
-#pragma unroll
-                for (int t = 0; t < 8; ++t)
-                    dot[e] += (float)o[t] * (float)gv[c][e][t];
-        }
-    }
-#pragma unroll
-    for (int e = 0; e < NE; ++e)
-        dot_lds[e][tid] = dot[e];
-    __syncthreads();
-    // sixteen threads per expert: each adds sixteen of the 256 partial sums, then the sixteen meet by lane shuffles
-    const int e = tid >> 4, i = tid & 15;
-    if (e < NE) {
-        float a = 0.f;
-#pragma unroll
-        for (int j = 0; j < 16; ++j)
-            a += dot_lds[e][16 * j + i];
-#pragma unroll
-        for (int off = 8; off > 0; off >>= 1)
-            a += __shfl_xor(a, off, 64);
-        if (i == 0 && e < n_experts)
-            logit_lds[e] = (float)(f16)a;
-    }
-    __syncthreads();
-    if (tid == 0)
-        route_top2(logit_lds, n_experts, sel, weights, logits_out);
+    __shared__ NormRouteLds<NE> lds;
+    norm_route_block<CH, NE>(x, delta, weight, eps, x, y, hidden, gate_w, n_experts, sel, weights, logits_out, lds);
 }
 
 // Rotary embedding, KV-cache append and attention of ONE new token (the reference takes them from HF transformers'

@@ -20,8 +20,10 @@
 // columns 16*kq .. 16*kq+15, i.e. step kq >> 2, MFMA lane group kq & 3.
 #include "gemv_parts.hpp"
 #include "hqq_common.hpp"
+#include "norm_route.hpp"
 
 #include <cstdlib>
+#include <type_traits>
 
 namespace hqq {
 using namespace gemv;
@@ -74,6 +76,12 @@ struct StripParams {
     const f16 *norm_delta, *norm_weight;
     f16 *x_sum;
     float norm_eps;
+    // ROUTED launches (the gates of both active experts): the router runs in the block's prologue on the normed row
+    // and its choice replaces sel; block (0, 0, 0) also writes the choice and the routing weights out.
+    const f16 *gate_w;
+    int n_experts;
+    int *sel_out;
+    f16 *rw_out;
 };
 
 template <int MT, int SKIND, int ZKIND> struct SlabRegs {
@@ -88,10 +96,13 @@ template <int MT, int SKIND, int ZKIND> struct SlabRegs {
 };
 
 // EPI: 0 y = o (+ bias) (* row_scale) (+ y);  1 y = silu(o0) * o1;  2 y = (y +) o0 * row_scale[0] + o1 * row_scale[1]
-template <int NBITS, int MT, int S, int D, int WAVES, int SKIND, int ZKIND, int EPI, bool GROUPED = false, bool NORM = false>
+// NORM: 0 the activations are x; 1 weight * rmsnorm(x + delta), the mean of squares added up while the weights travel;
+// 2 the same with the router of the normed row in the prologue, whose choice picks the experts of the launch
+template <int NBITS, int MT, int S, int D, int WAVES, int SKIND, int ZKIND, int EPI, bool GROUPED = false, int NORM = 0>
 __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
 {
     static_assert(!NORM || (MT == 1 && WAVES >= 4), "the fused norm is for single rows and blocks of four waves and more");
+    constexpr bool ROUTED = NORM == 2;
     constexpr int F = 8 / NBITS;
     constexpr int ENTRY = 8; // halves per B-operand entry (16 bytes)
     constexpr int STEP_HALVES = F * 2 * 4 * MT * ENTRY;
@@ -108,6 +119,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     __shared__ __attribute__((aligned(16))) float fin_lds[2][16][MT][F];
     __shared__ int ticket_lds;
     __shared__ float norm_lds[4];
+    __shared__ int sel_lds[2];
+    __shared__ f16 rw_lds[2];
+    // ROUTED launches: the normed row, written once by the prologue and read by every slab (hidden <= 4096)
+    __shared__ __attribute__((aligned(16))) f16 xn_lds[ROUTED ? 4096 : 8];
 
     const int lane = threadIdx.x & 63;
     // the wave index as a scalar: what depends on it (the layer, its record, the K range) then lives in scalar
@@ -123,11 +138,28 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     const int layer = wave >= p.KS ? 1 : 0;
     const int ks = wave - layer * p.KS;
     const bool wave_on = wave < p.KS * p.NL;
+    float rnorm = 1.0f; // NORM launches: 1 / sqrt(mean(x^2) + eps), known once the block has added the row up
+    if constexpr (ROUTED) {
+        // every block routes for itself (the router's rows come from L2): which records to read is known only then
+        const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0;
+        // the router's scratch shares the code staging buffer, which nothing touches before the first slab is worked
+        // on: with an LDS array of its own the block no longer fits twice into a compute unit
+        static_assert(!ROUTED || sizeof(code_lds) >= sizeof(NormRouteLds<8>), "router scratch does not fit the staging buffer");
+        NormRouteLds<8> &route_lds = *reinterpret_cast<NormRouteLds<8> *>(&code_lds[0][0]);
+        rnorm = norm_route_block<2, 8>(p.x, p.norm_delta, p.norm_weight, p.norm_eps, writer ? p.x_sum : nullptr, xn_lds, p.K,
+                                       p.gate_w, p.n_experts, sel_lds, rw_lds, nullptr, route_lds);
+        __syncthreads();
+        if (writer && threadIdx.x < 2) {
+            p.sel_out[threadIdx.x] = sel_lds[threadIdx.x];
+            p.rw_out[threadIdx.x] = rw_lds[threadIdx.x];
+        }
+    }
     // both layer records come from the kernel arguments and are selected in registers: no dependent loads
     StripLayer L;
     if (p.table) {
         // one word of the record per lane, then broadcast: the record's address is known only now
-        const int e = __builtin_amdgcn_readfirstlane(p.sel[g * p.sel_gstride + layer * p.sel_lstride]);
+        const int sel_at = g * p.sel_gstride + layer * p.sel_lstride;
+        const int e = __builtin_amdgcn_readfirstlane(ROUTED ? sel_lds[sel_at] : p.sel[sel_at]);
         const uint32_t *src =
             reinterpret_cast<const uint32_t *>(p.table + (e * p.table_stride + p.table_first + layer * p.first_lstride));
         const uint32_t word = src[lane < 18 ? lane : 0];
@@ -190,16 +222,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
         load16<SKIND>(r.s, L.sq, L.s_ms, L.s_mz, c, scm);
         load16<ZKIND>(r.z, L.zq, L.z_ms, L.z_mz, c, zcm);
         // x: one coalesced piece per pair of batch rows (16 bytes per lane, 32 lanes per row)
-        if constexpr (STAGE) {
+        if constexpr (ROUTED) {
+            // the row is in LDS already
+        } else if constexpr (STAGE) {
 #pragma unroll
             for (int j = 0; j < (MT + 1) / 2; ++j) {
                 int m = 2 * j + (lane >> 5);
                 m = m < M ? m : 0;
                 r.xw[j] = gload<u32x4>(xl + (k0 + (uint32_t)(8 * (lane & 31)) + (uint32_t)(m * K)));
             }
-            if constexpr (NORM) {
+            if constexpr (NORM == 1) {
                 r.xg = gload<u32x4>(p.norm_weight + (k0 + (uint32_t)(8 * (lane & 31))));
-                r.xd = p.norm_delta ? gload<u32x4>(p.norm_delta + (k0 + (uint32_t)(8 * (lane & 31)))) : (u32x4){0, 0, 0, 0};
+                // unconditional (a launch without delta re-reads x and ignores the value): a load under a branch
+                // would make every later wait a wait for all loads
+                r.xd = gload<u32x4>((p.norm_delta ? p.norm_delta : p.x) + (k0 + (uint32_t)(8 * (lane & 31))));
             }
         } else {
 #pragma unroll
@@ -242,19 +278,18 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
 #pragma unroll
     for (int m = 0; m < MT; ++m)
         bias_acc[m] = 0.f;
-    float rnorm = 1.0f; // NORM launches: 1 / sqrt(mean(x^2) + eps), known once the block has added the row up
 
     uint8_t *code_w = &code_lds[wave][0];
-    auto compute = [&](const SlabRegs<MT, SKIND, ZKIND> &r) __attribute__((always_inline)) {
+    auto compute = [&](const SlabRegs<MT, SKIND, ZKIND> &r, int slab) __attribute__((always_inline)) {
         // ------------------------------------------------------------ staging: x and the codes change lanes through LDS
         if constexpr (STAGE) {
 #pragma unroll
-            for (int j = 0; j < (MT + 1) / 2; ++j) {
+            for (int j = 0; j < (ROUTED ? 0 : (MT + 1) / 2); ++j) {
                 u32x4 xv = r.xw[j];
-                if constexpr (NORM) { // weight * fp16(fp32(x + delta) * r): the roundings of the stand-alone norm kernel
+                if constexpr (NORM == 1) { // weight * fp16(fp32(x + delta) * r): the roundings of the stand-alone norm kernel
                     f16x8 v = __builtin_bit_cast(f16x8, xv);
-                    if (p.norm_delta)
-                        v = v + __builtin_bit_cast(f16x8, r.xd);
+                    const f16x8 vd = v + __builtin_bit_cast(f16x8, r.xd);
+                    v = p.norm_delta ? vd : v;
                     const f16x8 g = __builtin_bit_cast(f16x8, r.xg);
                     f16x8 o;
 #pragma unroll
@@ -288,7 +323,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
             for (int m = 0; m < MT; ++m) {
                 if (m < M) {
                     u32x4 x0, x1;
-                    if constexpr (STAGE) {
+                    if constexpr (ROUTED) {
+                        const u32x4 *xp = reinterpret_cast<const u32x4 *>(&xn_lds[slab * kSlab + 16 * kq]);
+                        x0 = xp[0], x1 = xp[1];
+                    } else if constexpr (STAGE) {
                         const u32x4 *xp = reinterpret_cast<const u32x4 *>(&xw_lds[wave][m][16 * kq]);
                         x0 = xp[0], x1 = xp[1];
                     } else {
@@ -355,7 +393,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     // order, so these must go out before the weights for the sum to be ready while the weights still travel.
     constexpr int NPIECE = 2;
     f16x8 nv[NPIECE];
-    if constexpr (NORM) {
+    if constexpr (NORM == 1) {
 #pragma unroll
         for (int c = 0; c < NPIECE; ++c) {
             const int k = ((int)threadIdx.x + c * 256) * 8;
@@ -370,7 +408,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
         for (int i = 0; i < D; ++i)
             issue(regs[i], slab0 + i < p.NS ? slab0 + i : last);
     }
-    if constexpr (NORM) {
+    if constexpr (NORM == 1) {
         // the sum in the order the stand-alone norm kernel adds it (256 threads, 8 elements each per pass), so that both
         // give the same bits
         float ss = 0.f;
@@ -409,7 +447,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
 #pragma unroll
         for (int i = 0; i < S; ++i) {
             if (slab0 + i < p.NS)
-                compute(regs[i % D]);
+                compute(regs[i % D], slab0 + i);
             if (i + D < S)
                 issue(regs[i % D], slab0 + i + D < p.NS ? slab0 + i + D : last);
         }
@@ -721,9 +759,18 @@ void launch_kinds(const StripParams &p, const StripPlan &pl, dim3 grid, hipStrea
     if constexpr (GROUPED && EPI == 0 && MT == 1 && WAVES >= 4) {
         if (p.norm_weight) { // the fused norm exists for the grouped single-row projections only
             if (pl.SKIND == TK_F16)
-                gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_F16, TK_F16, EPI, true, true><<<grid, dim3(WAVES * 64), 0, s>>>(p);
+                gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_F16, TK_F16, EPI, true, 1><<<grid, dim3(WAVES * 64), 0, s>>>(p);
             else
-                gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_U8_COLS, TK_U8_SCALAR, EPI, true, true><<<grid, dim3(WAVES * 64), 0, s>>>(p);
+                gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_U8_COLS, TK_U8_SCALAR, EPI, true, 1><<<grid, dim3(WAVES * 64), 0, s>>>(p);
+            return;
+        }
+    }
+    if constexpr (GROUPED && EPI == 1 && MT == 1 && WAVES >= 4) {
+        if (p.gate_w) { // the routed gate of the decode step
+            if (pl.SKIND == TK_F16)
+                gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_F16, TK_F16, EPI, true, 2><<<grid, dim3(WAVES * 64), 0, s>>>(p);
+            else
+                gemv_strip_kernel<NBITS, MT, S, D, WAVES, TK_U8_COLS, TK_U8_SCALAR, EPI, true, 2><<<grid, dim3(WAVES * 64), 0, s>>>(p);
             return;
         }
     }
@@ -790,6 +837,10 @@ struct StripJob {
     const f16 *norm_delta, *norm_weight; // norm_weight != null: activations = norm_weight * rmsnorm(x + norm_delta)
     f16 *x_sum;
     float norm_eps;
+    const f16 *gate_w; // != null: routed gate launch (needs the norm fields and an index table)
+    int n_experts;
+    int *sel_out;
+    f16 *rw_out;
 };
 
 bool same_family(const hqq_linear *a, const hqq_linear *b)
@@ -877,10 +928,14 @@ int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t
     p.counter = reinterpret_cast<int *>(base);
     p.row_scale = j.row_scale, p.rs_lstride = j.rs_lstride, p.accumulate = j.accumulate;
     if (j.norm_weight) {
-        // every launch shape the planner can pick for this job has the fused-norm form except blocks under four waves
-        if (j.EPI != 0 || j.NL != 1 || M != 1 || pl.WAVES < 4 || !j.x_sum)
+        // every launch shape the planner can pick for these jobs has the fused-norm form except blocks under four waves
+        const bool plain = j.EPI == 0 && j.NL == 1 && !j.gate_w;
+        const bool routed = j.EPI == 1 && j.NL == 2 && j.NG == 2 && j.gate_w && j.ix && j.sel_out && j.rw_out &&
+                            j.n_experts >= 2 && j.n_experts <= 8 && j.shape[0]->K <= 4096 && j.shape[0]->K % 8 == 0;
+        if ((!plain && !routed) || M != 1 || pl.WAVES < 4 || !j.x_sum)
             return HQQ_E_UNSUPPORTED;
         p.norm_delta = j.norm_delta, p.norm_weight = j.norm_weight, p.x_sum = j.x_sum, p.norm_eps = j.norm_eps;
+        p.gate_w = j.gate_w, p.n_experts = j.n_experts, p.sel_out = j.sel_out, p.rw_out = j.rw_out;
     }
     const dim3 grid((unsigned)pl.BK, (unsigned)pl.RB, (unsigned)z);
     const bool two = j.shape[0]->nbits == 2;
@@ -950,6 +1005,24 @@ int launch_strip_gate_up_pair(const hqq_linear *w1, const hqq_linear *w3, const 
     j.shape[0] = j.shape[2] = w1, j.shape[1] = j.shape[3] = w3;
     j.NG = 2, j.NL = 2, j.EPI = 1, j.ix = &ix, j.sel_gstride = 1, j.first_lstride = 1;
     j.x = x, j.y[0] = h0, j.y[1] = h1;
+    return run_job(j, 1, ws, ws_bytes, s);
+}
+
+// The same launch with the post-attention norm and the router in front of it: every block forms
+// weight * rmsnorm(x + delta), routes it over gate_w (n_experts x K) and takes the gates of the two experts chosen;
+// x + delta goes to x_sum, the choice to sel_out[2] and the routing weights to rw_out[2].
+int launch_strip_gate_up_pair_routed(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, const StripNorm &norm,
+                                     const f16 *gate_w, int n_experts, int *sel_out, f16 *rw_out, f16 *h0, f16 *h1,
+                                     void *ws, size_t ws_bytes, hipStream_t s, const StripIndex &ix)
+{
+    StripJob j = {};
+    j.shape[0] = j.shape[2] = w1, j.shape[1] = j.shape[3] = w3;
+    j.NG = 2, j.NL = 2, j.EPI = 1, j.ix = &ix, j.sel_gstride = 1, j.first_lstride = 1;
+    j.x = x, j.y[0] = h0, j.y[1] = h1;
+    j.norm_delta = norm.delta, j.norm_weight = norm.weight, j.x_sum = norm.x_sum, j.norm_eps = norm.eps;
+    j.gate_w = gate_w, j.n_experts = n_experts, j.sel_out = sel_out, j.rw_out = rw_out;
+    if (!norm.weight || !gate_w)
+        return HQQ_E_NULL;
     return run_job(j, 1, ws, ws_bytes, s);
 }
 

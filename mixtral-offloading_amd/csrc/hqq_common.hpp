@@ -139,6 +139,9 @@ struct StripNorm {
 };
 int launch_strip_group(const hqq_linear *const *layers, int count, const f16 *x, f16 *const *ys, void *ws,
                        size_t ws_bytes, hipStream_t s, const StripNorm *norm = nullptr);
+int launch_strip_gate_up_pair_routed(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, const StripNorm &norm,
+                                     const f16 *gate_w, int n_experts, int *sel_out, f16 *rw_out, f16 *h0, f16 *h1,
+                                     void *ws, size_t ws_bytes, hipStream_t s, const StripIndex &ix);
 size_t strip_job_workspace_bytes(const hqq_linear *const *layers, int count, int NL, int64_t M);
 int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s);
 size_t workspace_head_bytes();

@@ -61,6 +61,9 @@ _SIGNATURES = {
     "hqq_expert_pair_ffn_workspace_bytes": (c_size_t, [_P(HqqLinear), _P(HqqLinear), _P(HqqLinear)]),
     "hqq_expert_pair_ffn_indexed": (c_int, [_P(HqqLinear), _P(HqqLinear), _P(HqqLinear), c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
+    "hqq_moe_pair_routed": (c_int, [_P(HqqLinear), _P(HqqLinear), _P(HqqLinear), c_void_p, c_void_p, c_void_p, c_void_p,
+                                    ctypes.c_float, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int,
+                                    c_void_p, c_size_t, c_void_p]),
     "hqq_matmul_group_workspace_bytes": (c_size_t, [_P(_P(HqqLinear)), c_int32]),
     "hqq_matmul_group": (c_int, [_P(_P(HqqLinear)), c_int32, c_void_p, _P(c_void_p), c_void_p, c_size_t, c_void_p]),
     "hqq_matmul_group_norm": (c_int, [_P(_P(HqqLinear)), c_int32, c_void_p, c_void_p, c_void_p, ctypes.c_float, c_void_p,

@@ -259,6 +259,31 @@ def expert_pair_ffn_indexed(table: ExpertTable, expert_index: torch.Tensor, x: t
     return out
 
 
+def moe_pair_routed(table: ExpertTable, x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                    x_sum: torch.Tensor, gate_weight: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
+                    out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
+    """``add_rmsnorm_router`` and ``expert_pair_ffn_indexed`` in two launches: the norm of ``x + delta`` and the router
+    run in front of the gates of the two experts they choose.  ``x + delta`` goes to ``x_sum`` (not ``x`` itself)."""
+    w1, w2, w3 = table.shape
+    n_experts, hidden = gate_weight.shape
+    assert x.dtype == torch.float16 and x.is_contiguous() and x.numel() == w1.K == hidden
+    assert x_sum.dtype == torch.float16 and x_sum.numel() == hidden and x_sum.data_ptr() != x.data_ptr()
+    assert weight.dtype == torch.float16 and weight.numel() == hidden and gate_weight.dtype == torch.float16
+    assert gate_weight.is_contiguous() and sel.dtype == torch.int32 and sel.numel() >= 2
+    assert weights.dtype == torch.float16 and weights.numel() >= 2
+    assert out.is_contiguous() and out.numel() == w2.N and out.dtype == torch.float16
+    with torch.cuda.device(x.device):
+        need = _lib.lib.hqq_expert_pair_ffn_workspace_bytes(w1.ref, w2.ref, w3.ref)
+        ws = workspace(x.device, need)
+        _lib.check(_lib.lib.hqq_moe_pair_routed(w1.ref, w2.ref, w3.ref, table.table.data_ptr(), x.data_ptr(),
+                                                delta.data_ptr() if delta is not None else None, weight.data_ptr(),
+                                                float(eps), x_sum.data_ptr(), gate_weight.data_ptr(), n_experts,
+                                                sel.data_ptr(), weights.data_ptr(), out.data_ptr(), int(accumulate),
+                                                ws.data_ptr(), ws.numel(), _lib.current_stream_ptr(x.device)),
+                   "hqq_moe_pair_routed")
+    return out
+
+
 class LinearGroup:
     """Up to four layers applied to the same single row in one launch (``hqq_matmul_group``): the q, k and v
     projections of an attention block.  ``supported`` is False when the layers do not fit one launch."""

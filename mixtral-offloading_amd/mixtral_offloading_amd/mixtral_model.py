@@ -140,6 +140,7 @@ class DecodeGraph:
                 [(m._expert[0].w1._desc(), m._expert[0].w2._desc(), m._expert[0].w3._desc()) for m in mods]))
         # the two active experts in two launches, q / k / v in one, where the shapes allow
         self.pair = all(hip_kernels.expert_pair_supported(t) for t in self.tables)
+        self.routed = self.pair and cfg.hidden_size <= 4096 and cfg.hidden_size % 8 == 0 and 2 <= cfg.num_local_experts <= 8
         self.qkv = [hip_kernels.LinearGroup([p._desc() for p in (l.self_attn.q_proj, l.self_attn.k_proj, l.self_attn.v_proj)])
                     for l in model.model.layers]
         self.cache = model.new_cache(max_len)
@@ -180,6 +181,13 @@ class DecodeGraph:
                 q, k, v = attn.q_proj(self.xn), attn.k_proj(self.xn), attn.v_proj(self.xn)
             out = hip_kernels.attention_decode(q, k, v, m.rotary.cos, m.rotary.sin, self.pos, ck, cv, self.att)
             attn_out = attn.o_proj(out)
+            if self.routed:
+                # post-attention norm, router and both experts in two launches
+                hip_kernels.moe_pair_routed(table, x, attn_out, layer.post_attention_layernorm.weight, eps, spare,
+                                            layer.block_sparse_moe.gate.weight, self.sel, self.rw, self.moe)
+                x, spare = spare, x
+                delta = self.moe
+                continue
             hip_kernels.add_rmsnorm_router(x, attn_out, layer.post_attention_layernorm.weight, eps, self.xn,
                                            layer.block_sparse_moe.gate.weight, self.sel, self.rw)
             if self.pair:

@@ -146,6 +146,47 @@ def test_expert_pair_equals_two_indexed_calls(shape):
             assert float((err > 0).float().mean()) < 0.5
 
 
+@pytest.mark.parametrize("shape", [(2, 512, 1024, 16, True), (2, 4096, 14336, 16, True), (4, 512, 2048, 64, True)],
+                         ids=lambda s: "w%d_h%d_f%d" % s[:3])
+def test_moe_pair_routed_equals_the_calls_it_replaces(shape):
+    """Norm, router and both experts in two launches: the bits of hqq_add_rmsnorm_router followed by
+    hqq_expert_pair_ffn_indexed."""
+    from mixtral_offloading_amd import hip_kernels
+    from test_gpu_matmul import _full_size_layer
+    nbits, hidden, ffn, gs, qt = shape
+    rng = np.random.default_rng(hidden + ffn + 1)
+    experts = []
+    for e in range(8):
+        if hidden >= 4096:
+            experts.append((_full_size_layer(nbits, ffn, hidden, gs, seed=3 * e), _full_size_layer(nbits, hidden, ffn, gs, seed=3 * e + 1),
+                            _full_size_layer(nbits, ffn, hidden, gs, seed=3 * e + 2)))
+            continue
+        w1, _ = o.random_layer(rng, ffn, hidden, nbits, gs, qt, qt)
+        w3, _ = o.random_layer(rng, ffn, hidden, nbits, gs, qt, qt)
+        w2, _ = o.random_layer(rng, hidden, ffn, nbits, gs, qt, qt)
+        experts.append((desc_of(w1), desc_of(w2), desc_of(w3)))
+    table = hip_kernels.ExpertTable(experts)
+    for trial in range(4):
+        x = to_dev(rng.standard_normal((1, hidden)).astype(np.float16))
+        d = to_dev(rng.standard_normal((1, hidden)).astype(np.float16)) if trial else None
+        w = to_dev((1 + 0.1 * rng.standard_normal(hidden)).astype(np.float16))
+        gw = to_dev((0.05 * rng.standard_normal((8, hidden))).astype(np.float16))
+        base = to_dev(rng.standard_normal((1, hidden)).astype(np.float16))
+        for accumulate in (False, True):
+            x1, xn = x.clone(), torch.empty_like(x)
+            sel1, rw1 = torch.zeros(2, dtype=torch.int32, device="cuda"), torch.zeros(2, dtype=torch.float16, device="cuda")
+            hip_kernels.add_rmsnorm_router(x1, d, w, 1e-5, xn, gw, sel1, rw1)
+            want = base.clone()
+            hip_kernels.expert_pair_ffn_indexed(table, sel1, xn, want, rw1, accumulate=accumulate)
+            x_sum = torch.full_like(x, float("nan"))
+            sel2, rw2 = torch.full_like(sel1, -1), torch.zeros_like(rw1)
+            got = base.clone()
+            hip_kernels.moe_pair_routed(table, x, d, w, 1e-5, x_sum, gw, sel2, rw2, got, accumulate=accumulate)
+            assert torch.equal(x_sum, x1)
+            assert sel1.tolist() == sel2.tolist() and torch.equal(rw1, rw2)
+            assert torch.equal(got, want), float((got.float() - want.float()).abs().max())
+
+
 @pytest.mark.parametrize("nbits,gs,k,ns,bias", [(4, 64, 4096, (4096, 1024, 1024), False), (4, 64, 1024, (512, 128, 128), True),
                                                 (2, 16, 512, (256, 64), False), (4, 32, 1024, (64, 64, 64, 128), True)])
 def test_matmul_group_equals_single_calls(nbits, gs, k, ns, bias):
