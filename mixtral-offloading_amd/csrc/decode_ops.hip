@@ -178,6 +178,8 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restr
     const int h = blockIdx.x, kv = h / group;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t pos = pos_p[0];
+    if (pos < 0 || pos >= max_len) // the position lives in device memory: a step past the cache must not write past it
+        return;
     const f16 *cs = cos_t + pos * HD, *sn = sin_t + pos * HD;
     if (tid < HD) {
         const int d = tid, o = d < HD / 2 ? d + HD / 2 : d - HD / 2;

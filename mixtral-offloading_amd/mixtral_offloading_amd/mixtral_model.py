@@ -157,6 +157,7 @@ class DecodeGraph:
         self.rw = torch.zeros(2, dtype=torch.float16, **mk)
         self.logits = torch.zeros((1, cfg.vocab_size), dtype=torch.float16, **mk)
         self.graph = None
+        self._host_pos = 0  # host mirror of ``pos``: the cache capacity is checked without reading the device
 
     @torch.inference_mode()
     def _step(self):
@@ -203,6 +204,9 @@ class DecodeGraph:
 
     def capture(self):
         """Warm up on a side stream (workspaces and allocator pools get their final size), then record the step."""
+        if self._host_pos + 3 > self.max_len:  # two warm-up steps and the recorded one each write one position further
+            raise ValueError(f"capture at position {self._host_pos} needs a cache of {self._host_pos + 3} positions, "
+                             f"this one holds {self.max_len}")
         keep = (self.tok.clone(), self.pos.clone())
         side = torch.cuda.Stream(device=self.model.device)
         side.wait_stream(torch.cuda.current_stream(self.model.device))
@@ -221,14 +225,20 @@ class DecodeGraph:
     @torch.inference_mode()
     def prefill(self, prompt_ids: torch.Tensor) -> torch.Tensor:
         """Runs the prompt through the eager path into this graph's cache; returns the first generated token."""
+        if prompt_ids.numel() >= self.max_len:
+            raise ValueError(f"a prompt of {prompt_ids.numel()} tokens does not fit a cache of {self.max_len} positions")
         logits = self.model.forward(prompt_ids, self.cache, 0)
         tok = logits[-1].argmax()
         self.tok.copy_(tok.view(1))
         self.pos.fill_(prompt_ids.numel())
+        self._host_pos = prompt_ids.numel()
         return tok
 
     def step(self):
         """One decode step; afterwards ``self.tok`` holds the next token and ``self.logits`` its logits."""
+        if self._host_pos >= self.max_len:
+            raise ValueError(f"the cache of {self.max_len} positions is full")
+        self._host_pos += 1
         if self.graph is None:
             self._step()
         else:

@@ -273,6 +273,39 @@ def test_graph_decode_matches_eager_logits():
     assert int(dec.pos) == pos
 
 
+def test_graph_decode_guards_its_cache_capacity():
+    """A prompt or a step past the cache raises on the host; the attention kernel itself leaves a position past the
+    cache alone."""
+    from mixtral_offloading_amd import build_model as bm, hip_kernels
+    from mixtral_offloading_amd.mixtral_model import DecodeGraph, Rotary
+    cfg = bm.mixtral_config(hidden_size=256, intermediate_size=512, num_hidden_layers=1, num_attention_heads=4,
+                            num_key_value_heads=2, vocab_size=128, num_local_experts=8)
+    off = bm.OffloadConfig(main_size=8, offload_size=0, buffer_size=1, offload_per_layer=0)
+    model = bm.build_model(torch.device("cuda:0"), bm.default_quant_config(), off, model_config=cfg, seed=5,
+                           max_positions=64)
+    dec = DecodeGraph(model, 12)
+    with pytest.raises(ValueError):
+        dec.prefill(torch.zeros(12, dtype=torch.int64, device="cuda"))
+    dec.prefill(torch.arange(10, device="cuda"))
+    with pytest.raises(ValueError):
+        dec.capture()  # needs positions 10, 11 and 12
+    dec.step()
+    dec.step()
+    with pytest.raises(ValueError):
+        dec.step()
+    hd, L = 64, 16
+    rot = Rotary(hd, 64, 1e6, torch.device("cuda"))
+    ck = torch.zeros((2, L, hd), dtype=torch.float16, device="cuda")
+    cv = torch.zeros_like(ck)
+    guard = torch.zeros((2, 4 * hd), dtype=torch.float16, device="cuda")  # would be hit by a write at position L
+    q = torch.randn((1, 4 * hd), device="cuda").half()
+    k = torch.randn((1, 2 * hd), device="cuda").half()
+    out = torch.zeros((1, 4 * hd), dtype=torch.float16, device="cuda")
+    hip_kernels.attention_decode(q, k, k, rot.cos, rot.sin, torch.tensor([L], device="cuda"), ck, cv, out)
+    torch.cuda.synchronize()
+    assert float(ck.abs().sum()) == 0 and float(cv.abs().sum()) == 0 and float(out.abs().sum()) == 0 and float(guard.abs().sum()) == 0
+
+
 def test_graph_decode_refuses_offloaded_experts():
     from mixtral_offloading_amd import build_model as bm
     from mixtral_offloading_amd.mixtral_model import DecodeGraph
