@@ -129,7 +129,8 @@ int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, i
  *      the layer is resident.  The table holds 3 records per expert in the order w1, w3, w2, each
  *      hqq_expert_record_bytes() long and written by hqq_expert_record_fill into HOST memory (the caller copies the
  *      table to the device once).  w1 / w2 / w3 describe the common shape of all experts (any one expert's
- *      descriptors).  Batches of at most 4 rows.  Workspace as for hqq_expert_ffn.                                  */
+ *      descriptors).  Batches of at most 4 rows.  Workspace as for hqq_expert_ffn.  expert_index[0] is read on the
+ *      device and not checked: it must name an expert of the table.                                                 */
 size_t hqq_expert_record_bytes(void);
 int hqq_expert_record_fill(const hqq_linear *l, void *host_record);
 int hqq_expert_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *device_table,
