@@ -242,24 +242,30 @@ struct TileWeightRegs {
     u32x2 sf, zf;         // four table halves (fp16 kind)
 };
 
-template <int NBITS, int BM, int SKIND, int ZKIND>
-__global__ __launch_bounds__(kWaves * 64) void gemm_tile2_kernel(TileParams p)
+// NFW: waves that share a packed table row, each taking F / NFW of its fields (1: a wave owns all fields; 2: the block
+// is eight waves, every weight is still rebuilt once, and a wave holds half the accumulators -- what lets two waves
+// share a SIMD at the 128-column batch tile).
+template <int NBITS, int BM, int SKIND, int ZKIND, int NFW>
+__global__ __launch_bounds__(kWaves * NFW * 64) void gemm_tile2_kernel(TileParams p)
 {
     constexpr int F = 8 / NBITS;
+    constexpr int FW = F / NFW;       // fields per wave
+    constexpr int NW = kWaves * NFW;  // waves per block
     constexpr int MB = BM / 16;
     constexpr int XP = BM + 2;
-    constexpr int XCH = (BM * 8 + kWaves * 64 - 1) / (kWaves * 64);
-    constexpr int TAB = F * 2 * 4 * 8; // halves per wave and table: entry ((i*2 + h)*4 + kg) of 8 halves
+    constexpr int XCH = (BM * 8 + NW * 64 - 1) / (NW * 64);
+    constexpr int TAB = FW * 2 * 4 * 8; // halves per wave and table: entry ((i*2 + h)*4 + kg) of 8 halves
     __shared__ __attribute__((aligned(16))) f16 x_lds[2][8 * XP * 8];
-    __shared__ __attribute__((aligned(16))) f16 s_lds[2][kWaves][TAB];
-    __shared__ __attribute__((aligned(16))) f16 z_lds[2][kWaves][TAB];
+    __shared__ __attribute__((aligned(16))) f16 s_lds[2][NW][TAB];
+    __shared__ __attribute__((aligned(16))) f16 z_lds[2][NW][TAB];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int jall = blockIdx.x / p.KSP, ks = blockIdx.x - jall * p.KSP;
     const bool second = jall >= p.JB; // block-uniform: the selections below are scalar
     const int jblk = jall - (second ? p.JB : 0);
-    const int jp = jblk * kWaves + wave;
+    const int jp = jblk * kWaves + wave / NFW;
+    const int f0 = (wave % NFW) * FW; // first field of this wave
     const Table &sc_t = second ? p.sc_b : p.sc, &zr_t = second ? p.zr_b : p.zr;
     const uint32_t sc_inv = second ? p.sc_b_inv : p.sc_inv;
     const int s_begin = ks * p.KTS;
@@ -270,11 +276,11 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile2_kernel(TileParams p)
     const int K = p.K;
     const int rr = lane & 15, kg = lane >> 4;
     const int ti = lane >> 4, kq = lane & 15;
-    const bool tlane = ti < F;
-    const int ti_l = ti & (F - 1); // lanes past the table rows repeat a table lane's loads: issuing loads never diverges
+    const bool tlane = ti < FW;
+    const int ti_l = ti & (FW - 1); // lanes past the table rows repeat a table lane's loads: issuing loads never diverges
 
     const uint8_t *codes = (second ? p.codes_b : p.codes) + ((size_t)((uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)p.GP) * K + 16 * kg);
-    const uint32_t c_row = (uint32_t)(F * jp + ti_l) * (uint32_t)K + (uint32_t)(4 * kq);
+    const uint32_t c_row = (uint32_t)(F * jp + f0 + ti_l) * (uint32_t)K + (uint32_t)(4 * kq);
     const uint8_t *s_tab = static_cast<const uint8_t *>(sc_t.data), *z_tab = static_cast<const uint8_t *>(zr_t.data);
     const f16 *s_ms = sc_t.ms, *s_mz = sc_t.mz;
     const uint32_t s_cols = (uint32_t)sc_t.meta_cols;
@@ -290,7 +296,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile2_kernel(TileParams p)
     int xdst[XCH];
 #pragma unroll
     for (int c = 0; c < XCH; ++c) {
-        const int ch = (int)threadIdx.x + c * kWaves * 64;
+        const int ch = (int)threadIdx.x + c * NW * 64;
         const int chc = ch < BM * 8 ? ch : BM * 8 - 1;
         int m = m0 + chc / 8;
         m = m < p.M ? m : p.M - 1;
@@ -341,7 +347,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile2_kernel(TileParams p)
             o.y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
             o.z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
             o.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
-            if (XCH * kWaves * 64 == BM * 8 || (int)threadIdx.x + c * kWaves * 64 < BM * 8)
+            if (XCH * NW * 64 == BM * 8 || (int)threadIdx.x + c * NW * 64 < BM * 8)
                 *reinterpret_cast<u32x4 *>(&x_lds[buf][xdst[c]]) = o;
         }
         if (tlane) {
@@ -366,9 +372,9 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile2_kernel(TileParams p)
         }
     };
 
-    f32x4 acc[F][MB];
+    f32x4 acc[FW][MB];
 #pragma unroll
-    for (int i = 0; i < F; ++i)
+    for (int i = 0; i < FW; ++i)
 #pragma unroll
         for (int b = 0; b < MB; ++b)
             acc[i][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -384,11 +390,13 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile2_kernel(TileParams p)
             for (int b = 0; b < MB; ++b)
                 B[b] = *reinterpret_cast<const f16x8 *>(&x_lds[buf][(((h * 4 + kg) * XP) + b * 16 + rr) * 8]);
 #pragma unroll
-            for (int i = 0; i < F; ++i) {
+            for (int i = 0; i < FW; ++i) {
                 const u32x4 S = *reinterpret_cast<const u32x4 *>(&s_lds[buf][wave][((i * 2 + h) * 4 + kg) * 8]);
                 const u32x4 Z = *reinterpret_cast<const u32x4 *>(&z_lds[buf][wave][((i * 2 + h) * 4 + kg) * 8]);
-                const uint32_t mk = WField<NBITS>::mask(i), ex = WField<NBITS>::expo(i);
-                const f16 offv = (f16)WField<NBITS>::offset(i);
+                // the field's constants: f0 is uniform over the wave, so these are scalar selects
+                const uint32_t mk = f0 ? WField<NBITS>::mask(i + (NFW - 1) * FW) : WField<NBITS>::mask(i);
+                const uint32_t ex = f0 ? WField<NBITS>::expo(i + (NFW - 1) * FW) : WField<NBITS>::expo(i);
+                const f16 offv = (f16)(f0 ? WField<NBITS>::offset(i + (NFW - 1) * FW) : WField<NBITS>::offset(i));
                 const f16x2 off = {offv, offv};
                 u32x4 Au;
 #pragma unroll
@@ -445,28 +453,33 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_tile2_kernel(TileParams p)
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int r = 16 * rb + 4 * kg + v;
-            const int64_t n = (int64_t)F * (jp + (int64_t)r * p.GP);
+            const int64_t ng = (int64_t)F * (jp + (int64_t)r * p.GP); // first output row of the group of F
+            const int64_t n = ng + f0;                                // first output row of this wave's fields
             if (p.part) { // K is split over blocks: fp32 partial sums, added by the finishing kernel
                 float *dst = p.part + (second ? p.part_lstride : 0) +
-                             (((int64_t)ks * (p.N / F) + n / F) * p.M + m) * F; // [K block][row group][batch row][F]
-                if constexpr (F == 4)
+                             (((int64_t)ks * (p.N / F) + ng / F) * p.M + m) * F + f0; // [K block][row group][batch row][F]
+                if constexpr (FW == 4)
                     *reinterpret_cast<f32x4 *>(dst) = (f32x4){acc[0][b][v], acc[1][b][v], acc[2][b][v], acc[3][b][v]};
-                else
+                else if constexpr (FW == 2)
                     *reinterpret_cast<float2 *>(dst) = make_float2(acc[0][b][v], acc[1][b][v]);
+                else
+                    *dst = acc[0][b][v];
                 continue;
             }
-            f16 o[F];
+            f16 o[FW];
 #pragma unroll
-            for (int i = 0; i < F; ++i) {
+            for (int i = 0; i < FW; ++i) {
                 o[i] = (f16)acc[i][b][v];
                 if (p.bias)
                     o[i] = o[i] + p.bias[n + i];
             }
             f16 *dst = p.y + (int64_t)m * p.N + n;
-            if constexpr (F == 4)
+            if constexpr (FW == 4)
                 *reinterpret_cast<f16x4 *>(dst) = (f16x4){o[0], o[1], o[2], o[3]};
-            else
+            else if constexpr (FW == 2)
                 *reinterpret_cast<f16x2 *>(dst) = (f16x2){o[0], o[1]};
+            else
+                *dst = o[0];
         }
     }
 }
@@ -637,10 +650,12 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl, int nl = 1)
 
 template <int NBITS, int BM> void launch_tile2_kinds(const TileParams &p, const TilePlan &pl, dim3 grid, hipStream_t s)
 {
+    // the widest batch tile runs with two waves per packed table row (half the accumulators each)
+    constexpr int NFW = BM == 128 ? 2 : 1;
     if (pl.kinds == 1)
-        gemm_tile2_kernel<NBITS, BM, TK_U8_COLS, TK_U8_SCALAR><<<grid, kWaves * 64, 0, s>>>(p);
+        gemm_tile2_kernel<NBITS, BM, TK_U8_COLS, TK_U8_SCALAR, NFW><<<grid, kWaves * NFW * 64, 0, s>>>(p);
     else
-        gemm_tile2_kernel<NBITS, BM, TK_F16, TK_F16><<<grid, kWaves * 64, 0, s>>>(p);
+        gemm_tile2_kernel<NBITS, BM, TK_F16, TK_F16, NFW><<<grid, kWaves * NFW * 64, 0, s>>>(p);
 }
 
 template <int NBITS> void launch_tile2_bm(const TileParams &p, const TilePlan &pl, dim3 grid, hipStream_t s)
