@@ -18,7 +18,8 @@ from torch import nn
 from .custom_layers import HQQLinearTritonSavable, MixtralBLockSparseTop2MLP_HQQ, SparseMoeWrapper
 from .expert_cache import ExpertCache
 from .expert_wrapper import MixtralExpertWrapper
-from .hqq_core import BaseQuantizeConfig
+from .hqq_core import BaseQuantizeConfig, BitPack
+from .packing import unpack_2bit_u8_common, unpack_3bit_i32_common, unpack_4bit_u8_common
 from .mixtral_model import MixtralForCausalLM
 from .utils import with_default_dtype
 
@@ -132,6 +133,71 @@ def make_and_load_expert_wrapper(config, quant_config: QuantConfig, states_dir: 
     expert = make_empty_expert(config, quant_config)
     expert.load_state_dict(state_dict, strict=True)
     return MixtralExpertWrapper(expert, device)
+
+
+_STEP_PACK = {"4bit_u8": (unpack_4bit_u8_common, BitPack.pack_4bit_u8), "2bit_u8": (unpack_2bit_u8_common, BitPack.pack_2bit_u8),
+              "3bit_32": (unpack_3bit_i32_common, BitPack.pack_3bit_32)}
+
+
+def codes_in_checkpoint_layout(lin: HQQLinearTritonSavable) -> torch.Tensor:
+    """The codes of a layer as hqq wrote them and as the reference's checkpoints hold them: the ``(N, K)`` codes viewed
+    as ``(group_size, N*K/group_size)`` and packed in hqq's step layout (code rows one ``step`` apart share a byte or
+    word).  It is the inverse of what ``repack`` does at load (reference src/custom_layers.py:41-47)."""
+    meta = lin.meta
+    unpack, pack = _STEP_PACK[meta["packing"]]
+    n = int(meta["shape"][0])
+    codes = unpack(lin.W_q)[:n]
+    return pack(codes.reshape(int(meta["group_size"]), -1)).contiguous()
+
+
+def iterate_experts(model) -> tp.Iterator[tp.Tuple[tp.Tuple[int, int], MixtralBLockSparseTop2MLP_HQQ]]:
+    """Every registered expert, in uid order, as a module on the device.  All of them are views of one scratch slab
+    that the next iteration overwrites (filled from the expert's pinned host copy)."""
+    cache_ = model.expert_cache
+    scratch = MixtralExpertWrapper(copy.deepcopy(cache_.slots[0]._expert[0]), cache_.device)
+    for uid, info in sorted(cache_.registered_experts.items()):
+        scratch.storage.copy_(info.host_slab.untyped_storage())
+        yield uid, scratch._expert[0]
+
+
+def save_quantized_checkpoint(model, state_path: str, layout: str = "hqq") -> None:
+    """Writes the directory that ``build_model(..., state_path)`` reads (reference src/build_model.py:137-205):
+    ``model.safetensors.index.json`` whose ``weight_map`` names, for every key, one of the safetensors files beside
+    it -- one file for the trunk (embedding, norms, attention, routers, head) and one per expert, keys in the flat
+    schema of ``HQQLinearTritonSavable`` (reference src/custom_layers.py:136-166).
+
+    ``layout="hqq"`` stores the codes as the reference's checkpoints do (quantise-time shape, step layout), so the
+    reference can read the directory as well; ``layout="kernel"`` stores them as they sit in memory, ``(N/f, K)``
+    interleaved, which only this package reads (it tells the two apart by the shape of ``W_q``)."""
+    from safetensors.torch import save_file
+
+    assert layout in ("hqq", "kernel")
+    os.makedirs(state_path, exist_ok=True)
+    weight_map: tp.Dict[str, str] = {}
+
+    def plain(state):
+        return {k: torch.Tensor.as_subclass(v, torch.Tensor).detach().cpu().contiguous().clone() for k, v in state.items()}
+
+    def linears_in_file_layout(module, state, prefix):
+        if layout == "hqq":
+            for name, sub in module.named_modules():
+                if isinstance(sub, HQQLinearTritonSavable):
+                    state[prefix + (name + "." if name else "") + "W_q"] = codes_in_checkpoint_layout(sub)
+        return state
+
+    def write(fname, state, index_prefix=""):
+        save_file(plain(state), os.path.join(state_path, fname))
+        weight_map.update({index_prefix + k: fname for k in state})
+
+    write("trunk.safetensors", linears_in_file_layout(model, dict(model.state_dict()), ""))
+    for (layer_idx, expert_idx), expert in iterate_experts(model):
+        prefix = f"model.layers.{layer_idx}.block_sparse_moe.experts.{expert_idx}."
+        # an expert's file holds the keys of the expert module itself (``w1.W_q`` ...): the reference hands the whole
+        # file to ``expert.load_state_dict`` (src/build_model.py:151-153); only the index carries the full names
+        write(f"expert-{layer_idx}-{expert_idx}.safetensors", linears_in_file_layout(expert, dict(expert.state_dict()), ""),
+              index_prefix=prefix)
+    with open(os.path.join(state_path, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {"layout": layout}, "weight_map": weight_map}, f)
 
 
 def build_model(device: torch.device, quant_config: QuantConfig, offload_config: OffloadConfig,

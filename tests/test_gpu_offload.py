@@ -161,3 +161,48 @@ def test_generate_offloaded_equals_resident():
     step_logits = [model_res.forward(prompt[i:i + 1], cache2, i)[0] for i in range(prompt.numel())]
     got = torch.stack(step_logits).float()
     assert torch.allclose(got, full.float(), atol=3e-2 * float(full.float().abs().max()), rtol=3e-2)
+
+
+@pytest.mark.parametrize("layout", ["hqq", "kernel"])
+@pytest.mark.parametrize("ffn_bits,ffn_group", [(2, 16), (3, 64), (4, 64)])
+def test_checkpoint_round_trip(tmp_path, layout, ffn_bits, ffn_group):
+    """A model written as a checkpoint directory and built again from it is the same model, bit for bit: the flat
+    state-dict keys, the safetensors index, and (``hqq`` layout) the step-layout codes of the reference's files,
+    which ``repack`` turns into the kernel layout at load."""
+    import json
+    from safetensors.torch import load_file
+    from mixtral_offloading_amd import build_model as bm
+    from mixtral_offloading_amd.hqq_core import BaseQuantizeConfig
+    cfg = bm.mixtral_config(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                            num_key_value_heads=2, vocab_size=128, num_local_experts=4)
+    qc = bm.QuantConfig(ffn_config=BaseQuantizeConfig(nbits=ffn_bits, group_size=ffn_group, quant_zero=True, quant_scale=True),
+                        attn_config=bm.default_quant_config().attn_config)
+    off = bm.OffloadConfig(main_size=4, offload_size=4, buffer_size=2, offload_per_layer=2)
+    dev = torch.device("cuda:0")
+    model = bm.build_model(dev, qc, off, model_config=cfg, seed=5, max_positions=64)
+    bm.save_quantized_checkpoint(model, str(tmp_path), layout=layout)
+
+    index = json.load(open(tmp_path / "model.safetensors.index.json"))["weight_map"]
+    w1_key = "model.layers.1.block_sparse_moe.experts.3.w1.W_q"
+    assert index["model.embed_tokens.weight"] != index[w1_key]
+    on_disk = load_file(str(tmp_path / index[w1_key]))["w1.W_q"]  # the file holds the expert module's own keys
+    n, k = 512, 256
+    if layout == "kernel":
+        assert tuple(on_disk.shape) == ((n + 9) // 10 if ffn_bits == 3 else n * ffn_bits // 8, k)
+    else:  # quantise-time shape: group_size code rows (70 for the padded 3-bit words) packed down the rows
+        rows = {2: ffn_group // 4, 4: ffn_group // 2, 3: (ffn_group + 9) // 10}[ffn_bits]
+        assert tuple(on_disk.shape) == (rows, n * k // ffn_group)
+
+    again = bm.build_model(dev, qc, off, state_path=str(tmp_path), model_config=cfg, max_positions=64)
+    a, b = model.state_dict(), again.state_dict()
+    assert list(a) == list(b)
+    for key in a:
+        assert torch.equal(torch.Tensor.as_subclass(a[key], torch.Tensor), torch.Tensor.as_subclass(b[key], torch.Tensor)), key
+    for (uid, ea), (uid_b, eb) in zip(bm.iterate_experts(model), bm.iterate_experts(again)):
+        sa, sb = ea.state_dict(), eb.state_dict()
+        assert uid == uid_b and list(sa) == list(sb) and len(sa) == 3 * 7
+        for key in sa:
+            assert torch.equal(torch.Tensor.as_subclass(sa[key], torch.Tensor), torch.Tensor.as_subclass(sb[key], torch.Tensor)), (uid, key)
+    prompt = torch.randint(0, cfg.vocab_size, (7,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(1))
+    assert torch.equal(model.generate(prompt, 6), again.generate(prompt, 6))
+    assert torch.equal(model.forward(prompt, model.new_cache(16), 0), again.forward(prompt, again.new_cache(16), 0))
