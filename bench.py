@@ -268,6 +268,26 @@ def decode_section(dev, tokens_resident=256, tokens_offload=48):
         del model
         gc.collect()
         torch.cuda.empty_cache()
+
+    # the other mixed-quant variant of the reference: 3-bit g64 experts under the same 4-bit attention
+    from mixtral_offloading_amd.hqq_core import BaseQuantizeConfig
+    qc3 = bm.QuantConfig(ffn_config=BaseQuantizeConfig(nbits=3, group_size=64, quant_zero=True, quant_scale=True),
+                         attn_config=bm.default_quant_config().attn_config)
+    off = bm.OffloadConfig(main_size=32 * 8, offload_size=0, buffer_size=4, offload_per_layer=0)
+    model = bm.build_model(dev, qc3, off, model_config=cfg, seed=0, max_positions=1024)
+    dec = DecodeGraph(model, 64 + 128 + 4)
+    dec.prefill(prompt)
+    dec.capture()
+    dec.prefill(prompt)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(128):
+        dec.step()
+    torch.cuda.synchronize()
+    out["experts_3bit_g64_all_resident_graph_tok_s"] = round(128 / (time.perf_counter() - t0), 1)
+    del dec, model
+    gc.collect()
+    torch.cuda.empty_cache()
     return out
 
 

@@ -129,7 +129,8 @@ int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, i
  *      the layer is resident.  The table holds 3 records per expert in the order w1, w3, w2, each
  *      hqq_expert_record_bytes() long and written by hqq_expert_record_fill into HOST memory (the caller copies the
  *      table to the device once).  w1 / w2 / w3 describe the common shape of all experts (any one expert's
- *      descriptors).  Batches of at most 4 rows.  Workspace as for hqq_expert_ffn.  expert_index[0] is read on the
+ *      descriptors).  Batches of at most 4 rows (2- and 4-bit experts) or 16 rows (3-bit experts, K a multiple of
+ *      256 and at least ten groups down N).  Workspace as for hqq_expert_ffn.  expert_index[0] is read on the
  *      device and not checked: it must name an expert of the table.                                                 */
 size_t hqq_expert_record_bytes(void);
 int hqq_expert_record_fill(const hqq_linear *l, void *host_record);
@@ -143,7 +144,9 @@ int hqq_expert_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq
  *      active experts of a single token, each product and the sum rounded to fp16 as index_add_ on fp16 tensors
  *      rounds them (what two hqq_expert_ffn_indexed calls give, the second accumulating, up to the order in which the
  *      fp32 partial sums over K are added).  One launch
- *      computes silu(w1 x) * w3 x of both experts, one both down projections and their weighted sum.  x is one row
+ *      computes silu(w1 x) * w3 x of both experts, one both down projections and their weighted sum (3-bit experts:
+ *      three launches -- the four gate projections, then one down projection per expert that applies silu(a) * b
+ *      as it reads them, the second adding into y).  x is one row
  *      (hidden fp16), expert_index two device int32, row_scale two device fp16.  Table as for
  *      hqq_expert_ffn_indexed.  HQQ_E_UNSUPPORTED when the shapes do not fit the decode kernel (the workspace query
  *      then returns 0): call hqq_expert_ffn_indexed twice instead.                                                 */
@@ -157,8 +160,9 @@ int hqq_expert_pair_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, cons
  *      hqq_expert_pair_ffn_indexed, with the norm and the router run by every block of the first launch in front of
  *      the gates (src/custom_layers.py:276-312 after the decoder layer's post-attention norm).  x + delta is written to
  *      x_sum (a buffer other than x), the router's choice to sel_out[2] and weights_f16_out[2] (device memory),
- *      y (+)= the weighted sum of the two experts' outputs.  hidden <= 4096, n_experts <= 8; workspace as
- *      hqq_expert_pair_ffn_workspace_bytes.  Results are those of the two calls it replaces, bit for bit.           */
+ *      y (+)= the weighted sum of the two experts' outputs.  hidden <= 4096, n_experts <= 8, 2- or 4-bit experts
+ *      (HQQ_E_UNSUPPORTED otherwise: make the two calls); workspace as hqq_expert_pair_ffn_workspace_bytes.  Results
+ *      are those of the two calls it replaces, bit for bit.                                                         */
 int hqq_moe_pair_routed(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *device_table,
                         const void *x_f16, const void *delta_f16, const void *norm_weight_f16, float eps, void *x_sum_f16,
                         const void *gate_w_f16, int32_t n_experts, int32_t *sel_out, void *weights_f16_out, void *y_f16,

@@ -203,6 +203,9 @@ static size_t ffn_matmul_scratch(const hqq_linear *w1, const hqq_linear *w2, con
     const size_t g = tile_gate_workspace_bytes(w1, w3, M);
     if (g > mm)
         mm = g;
+    const size_t v = vec3_ffn_workspace_bytes(w1, w2, M, 1);
+    if (v > mm)
+        mm = v;
     return align256(mm);
 }
 
@@ -263,6 +266,15 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
     const f16 *x = (const f16 *)x_f16;
     f16 *y = (f16 *)y_f16;
 
+    // 3-bit decode batches: both gate projections in one launch, silu(a) * b folded into the down projection's loads
+    if (pick_family(w1, M) == FAM_VEC3 && pick_family(w2, M) == FAM_VEC3 && vec3_ffn_supported(w1, w2, w3, M, 1)) {
+        if ((rc = launch_vec3_gate(w1, w3, x, M, a, (int64_t)(mid / 2), 1, mm, mm_bytes, s)) != HQQ_OK)
+            return rc;
+        SmallBatchEpilogue ep;
+        ep.row_scale = (const f16 *)row_scale_f16;
+        ep.accumulate = accumulate;
+        return launch_vec3_down(w2, a, b, M, y, mm, mm_bytes, ep, s);
+    }
     // fused gate: decode batches always; wider ones only where the tile kernel does not take the shape
     const bool prefer_tile = tile_supported(w1, M) && tile_supported(w3, M) && !strip_supported(w1, M);
     const bool fast13 = !prefer_tile && smallbatch_supported(w1, M) && smallbatch_supported(w3, M) && !w1->bias &&
@@ -305,7 +317,7 @@ int hqq_expert_record_fill(const hqq_linear *l, void *host_record)
         return rc;
     if (!host_record)
         return HQQ_E_NULL;
-    if (!strip_supported(l, 1))
+    if (!strip_supported(l, 1) && !vec3_supported(l, 1))
         return HQQ_E_UNSUPPORTED;
     strip_fill_record(host_record, l);
     return HQQ_OK;
@@ -325,7 +337,8 @@ int hqq_expert_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq
         return HQQ_OK;
     if (!x_f16 || !y_f16 || !device_table || !expert_index)
         return HQQ_E_NULL;
-    if (!strip_supported(w1, M) || !strip_supported(w3, M) || !strip_supported(w2, M))
+    const bool three = w1->nbits == 3 && vec3_ffn_supported(w1, w2, w3, M, 1);
+    if (!three && (!strip_supported(w1, M) || !strip_supported(w3, M) || !strip_supported(w2, M)))
         return HQQ_E_UNSUPPORTED;
     const size_t need = hqq_expert_ffn_workspace_bytes(w1, w2, w3, M);
     if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
@@ -334,6 +347,17 @@ int hqq_expert_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq
     char *p = static_cast<char *>(workspace);
     const size_t mm_bytes = ffn_matmul_scratch(w1, w2, w3, M);
     f16 *h = (f16 *)(p + mm_bytes);
+    if (three) {
+        const size_t mid = align256((size_t)M * w1->N * 2), outb = align256((size_t)M * w2->N * 2);
+        f16 *a = (f16 *)(p + mm_bytes + mid + outb), *b = (f16 *)(p + mm_bytes + 2 * mid + outb);
+        const StripIndex gate3 = {device_table, expert_index, 3, 0}, down3 = {device_table, expert_index, 3, 2};
+        if ((rc = launch_vec3_gate(w1, w3, (const f16 *)x_f16, M, a, (int64_t)(mid / 2), 1, p, mm_bytes, s, &gate3)) != HQQ_OK)
+            return rc;
+        SmallBatchEpilogue ep3;
+        ep3.row_scale = (const f16 *)row_scale_f16;
+        ep3.accumulate = accumulate;
+        return launch_vec3_down(w2, a, b, M, (f16 *)y_f16, p, mm_bytes, ep3, s, &down3);
+    }
     const StripIndex gate = {device_table, expert_index, 3, 0}, down = {device_table, expert_index, 3, 2};
     if ((rc = launch_strip_gate_up(w1, w3, (const f16 *)x_f16, M, h, p, mm_bytes, s, &gate)) != HQQ_OK)
         return rc;
@@ -346,6 +370,8 @@ int hqq_expert_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq
 // workspace of the two-expert step: [strip scratch, counters first][h of expert 0][h of expert 1]
 static size_t pair_scratch(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3)
 {
+    if (w1->nbits == 3)
+        return vec3_ffn_supported(w1, w2, w3, 1, 2) ? align256(vec3_ffn_workspace_bytes(w1, w2, 1, 2)) : 0;
     const hqq_linear *gate[4] = {w1, w3, w1, w3}, *down[2] = {w2, w2};
     const size_t a = strip_job_workspace_bytes(gate, 4, 2, 1), b = strip_job_workspace_bytes(down, 2, 2, 1);
     if (a == 0 || b == 0)
@@ -358,7 +384,8 @@ size_t hqq_expert_pair_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linea
     if (validate_linear(w1) != HQQ_OK || validate_linear(w2) != HQQ_OK || validate_linear(w3) != HQQ_OK)
         return 0;
     const size_t mm = pair_scratch(w1, w2, w3);
-    return mm ? mm + 2 * align256((size_t)w1->N * 2) : 0;
+    // h of both experts; 3-bit layers keep the two gate projections of each apart (silu(a) * b is applied on load)
+    return mm ? mm + (w1->nbits == 3 ? 4 : 2) * align256((size_t)w1->N * 2) : 0;
 }
 
 int hqq_expert_pair_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3,
@@ -385,6 +412,21 @@ int hqq_expert_pair_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, cons
     const size_t mid = align256((size_t)w1->N * 2);
     f16 *h0 = (f16 *)(p + mm_bytes), *h1 = (f16 *)(p + mm_bytes + mid);
     const StripIndex gate = {device_table, expert_index, 3, 0}, down = {device_table, expert_index, 3, 2};
+    if (w1->nbits == 3) {
+        // a0, b0, a1, b1 from one launch, then one down projection per expert, the second adding into y
+        const int64_t ls = (int64_t)(mid / 2);
+        if ((rc = launch_vec3_gate(w1, w3, (const f16 *)x_f16, 1, h0, ls, 2, p, mm_bytes, s, &gate)) != HQQ_OK)
+            return rc;
+        const StripIndex down1 = {device_table, expert_index + 1, 3, 2};
+        SmallBatchEpilogue ep;
+        ep.row_scale = (const f16 *)row_scale_f16;
+        ep.accumulate = accumulate;
+        if ((rc = launch_vec3_down(w2, h0, h0 + ls, 1, (f16 *)y_f16, p, mm_bytes, ep, s, &down)) != HQQ_OK)
+            return rc;
+        ep.row_scale = (const f16 *)row_scale_f16 + 1;
+        ep.accumulate = 1;
+        return launch_vec3_down(w2, h0 + 2 * ls, h0 + 3 * ls, 1, (f16 *)y_f16, p, mm_bytes, ep, s, &down1);
+    }
     if ((rc = launch_strip_gate_up_pair(w1, w3, (const f16 *)x_f16, h0, h1, p, mm_bytes, s, gate)) != HQQ_OK)
         return rc;
     return launch_strip_down_pair(w2, h0, (int64_t)(mid / 2), (f16 *)y_f16, (const f16 *)row_scale_f16, accumulate, p,
@@ -404,8 +446,8 @@ int hqq_moe_pair_routed(const hqq_linear *w1, const hqq_linear *w2, const hqq_li
         return HQQ_E_SHAPE;
     if (!x_f16 || !y_f16 || !device_table || !norm_weight_f16 || !x_sum_f16 || !gate_w_f16 || !sel_out || !weights_f16_out)
         return HQQ_E_NULL;
-    if (n_experts < 2 || n_experts > 8 || w1->K > 4096 || w1->K % 8 != 0)
-        return HQQ_E_UNSUPPORTED;
+    if (n_experts < 2 || n_experts > 8 || w1->K > 4096 || w1->K % 8 != 0 || w1->nbits == 3)
+        return HQQ_E_UNSUPPORTED; // 3-bit experts: hqq_add_rmsnorm_router, then hqq_expert_pair_ffn_indexed
     if ((reinterpret_cast<uintptr_t>(x_f16) | reinterpret_cast<uintptr_t>(delta_f16) | reinterpret_cast<uintptr_t>(gate_w_f16) |
          reinterpret_cast<uintptr_t>(norm_weight_f16) | reinterpret_cast<uintptr_t>(x_sum_f16)) & 15u)
         return HQQ_E_ALIGN;

@@ -29,14 +29,7 @@ namespace hqq {
 using namespace gemv;
 namespace {
 
-struct StripLayer {
-    const uint8_t *codes;
-    const uint8_t *sq, *zq; // 8-bit tables, or fp16 tables
-    const f16 *s_ms, *s_mz; // meta of the scale table
-    const f16 *z_ms, *z_mz; // meta of the zero table
-    uint32_t s_cols, z_cols, s_inv, z_inv;
-};
-static_assert(sizeof(StripLayer) == 72, "the record is read as 18 words");
+using StripLayer = LayerRecord;
 
 // A launch may hold several groups of layers: group g covers blockIdx.z = z_begin .. z_begin + GP - 1 and has its
 // own output.  Groups share K, the code width and the group size, not N (q, k and v projections in one launch;
@@ -738,20 +731,7 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl, int64_t ti
     return true;
 }
 
-void fill_layer(StripLayer &L, const hqq_linear *l)
-{
-    L.codes = static_cast<const uint8_t *>(l->codes);
-    L.sq = static_cast<const uint8_t *>(l->scale.data);
-    L.zq = static_cast<const uint8_t *>(l->zero.data);
-    L.s_ms = static_cast<const f16 *>(l->scale.meta_scale);
-    L.s_mz = static_cast<const f16 *>(l->scale.meta_zero);
-    L.z_ms = static_cast<const f16 *>(l->zero.meta_scale);
-    L.z_mz = static_cast<const f16 *>(l->zero.meta_zero);
-    L.s_cols = (uint32_t)l->scale.meta_cols;
-    L.z_cols = (uint32_t)l->zero.meta_cols;
-    L.s_inv = L.s_cols ? (uint32_t)(0xFFFFFFFFull / L.s_cols) : 0;
-    L.z_inv = L.z_cols ? (uint32_t)(0xFFFFFFFFull / L.z_cols) : 0;
-}
+void fill_layer(StripLayer &L, const hqq_linear *l) { fill_layer_record(L, l); }
 
 template <int NBITS, int MT, int S, int D, int WAVES, int EPI, bool GROUPED>
 void launch_kinds(const StripParams &p, const StripPlan &pl, dim3 grid, hipStream_t s)

@@ -17,6 +17,13 @@
 // The waves of a block split K (two slabs each); when K needs several blocks (or the window count alone would leave
 // most of the chip idle) the blocks of a tile store fp32 partial sums with device-scope stores and the block that
 // arrives last at the tile's counter adds them in a fixed order.  Batches above two rows run as passes of two.
+//
+// A launch may hold up to four layers of one shape (blockIdx.z = layer * P + window): the two projections of an
+// expert's gate, or those of two experts.  Their records come from the kernel arguments or from a device table
+// (record sel[layer / lper] * stride + first + layer % lper), so that the expert can be chosen on the device.
+// XMODE 1 builds the activations on the fly as silu(xa) * xb, which is how the down projection reads the two
+// gate outputs without an elementwise launch in between; the epilogue can multiply by a routing weight per row
+// and add into y.
 #include "gemv_parts.hpp"
 #include "hqq_common.hpp"
 
@@ -25,21 +32,29 @@ using namespace gemv;
 namespace {
 
 constexpr int kW3Waves = 8;
-constexpr int kW3S = 2; // slabs per wave
+constexpr int kW3S = 2; // most slabs per wave
+
+constexpr int kW3MaxLayers = 4;
 
 struct W3Params {
-    const uint8_t *codes; // int32 [NW][K]
-    const uint8_t *sq, *zq;
-    const f16 *s_ms, *s_mz, *z_ms, *z_mz;
-    uint32_t s_cols, s_inv;
-    const f16 *x;
-    f16 *y;
-    const f16 *bias;
-    float *part; // [BK][M][N]
+    LayerRecord layer[kW3MaxLayers];
+    const LayerRecord *table; // indexed launch (table != null)
+    const int *sel;
+    int stride, first, lper;
+    const f16 *x;       // XMODE 0: (M, K)
+    const f16 *xa, *xb; // XMODE 1: x = silu(xa) * xb, both (M, K)
+    f16 *y;             // layer l writes y + l * y_lstride
+    int64_t y_lstride;
+    const f16 *bias;      // single layer from the kernel arguments only
+    const f16 *row_scale; // optional multiplier per batch row
+    int accumulate;       // add into y
+    float *part; // layer l: part + l * part_lstride, [BK][M][N]
+    int64_t part_lstride;
     int *counter;
     int M, N, K, G, P, NW, RB;
     int NS; // K / 256
     int KS; // waves of a block that have slabs
+    int S;  // slabs per wave
     int SB; // slabs per block
     int BK; // blocks along K per tile
 };
@@ -62,7 +77,15 @@ __device__ __forceinline__ float quad_sum(float v)
     return v;
 }
 
-template <int MT, bool Q8> // Q8: scale u8 + per-column meta, zero u8 + whole-tensor meta; else fp16 tables
+// silu in fp32 with one rounding, then the fp16 product: the two roundings of the elementwise kernel
+__device__ __forceinline__ f16 silu_mul(f16 a, f16 b)
+{
+    const float v = (float)a;
+    return (f16)(v / (1.0f + __expf(-v))) * b;
+}
+
+// Q8: scale u8 + per-column meta, zero u8 + whole-tensor meta; else fp16 tables.  XMODE 1: x = silu(xa) * xb
+template <int MT, bool Q8, int XMODE>
 __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
 {
     constexpr int NT = kW3Waves * 64;
@@ -73,7 +96,26 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int kb = blockIdx.x, rb = blockIdx.y, w0 = blockIdx.z;
+    const int kb = blockIdx.x, rb = blockIdx.y;
+    const int layer = (int)(blockIdx.z >= (unsigned)p.P) + (int)(blockIdx.z >= 2u * p.P) + (int)(blockIdx.z >= 3u * p.P);
+    const int w0 = (int)blockIdx.z - layer * p.P;
+    // The layer's record.  From a table it is read one word per lane and broadcast; every load through it below is
+    // an explicit device-memory load (a pointer out of a record has lost its address space).
+    LayerRecord R;
+    if (p.table) {
+        const int e = __builtin_amdgcn_readfirstlane(p.sel[layer / p.lper]);
+        const uint32_t *src = reinterpret_cast<const uint32_t *>(p.table + (e * p.stride + p.first + layer % p.lper));
+        const uint32_t word = src[lane < 18 ? lane : 0];
+        uint32_t rec[18];
+#pragma unroll
+        for (int i = 0; i < 18; ++i)
+            rec[i] = __builtin_amdgcn_readlane(word, i);
+        __builtin_memcpy(&R, rec, sizeof(R));
+    } else {
+        R = p.layer[__builtin_amdgcn_readfirstlane(layer)];
+    }
+    f16 *const yl = p.y + (int64_t)layer * p.y_lstride;
+    float *const partl = p.part + (int64_t)layer * p.part_lstride;
     const int M = MT == 1 ? 1 : p.M;
     const int K = p.K;
     const int t = lane >> 2, c = lane & 3;
@@ -89,24 +131,26 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
         for (int m = 0; m < MT; ++m)
             acc[i][m] = zacc[i][m] = 0.f;
 
-    const int slab_lo = kb * p.SB + wave * kW3S;
+    const int slab_lo = kb * p.SB + wave * p.S;
     int slab_hi = (kb + 1) * p.SB;
     if (slab_hi > p.NS)
         slab_hi = p.NS;
-    // whole-tensor meta of the zero table; the address is the same in every lane but written so that the compiler
-    // does not see it (lane >> 6 is zero): a load it knows to be uniform is moved to scalar registers at once,
-    // which waits for it before any weight load has been issued
-    uint32_t zms_raw = 0, zmz_raw = 0;
-    if constexpr (Q8) {
-        zms_raw = reinterpret_cast<const uint16_t *>(p.z_ms)[lane >> 6];
-        zmz_raw = reinterpret_cast<const uint16_t *>(p.z_mz)[lane >> 6];
-    }
 
-    for (int sl = 0; sl < kW3S; ++sl) {
+    for (int sl = 0; sl < p.S; ++sl) {
         const int slab = slab_lo + sl;
         if (wave >= p.KS || slab >= slab_hi)
             break;
         const uint32_t k0 = (uint32_t)slab * kSlab;
+        // Every load of the slab is issued before any of its arithmetic, in the order the arithmetic needs them
+        // (loads retire in issue order): zero meta, tables, x, codes.
+        // Whole-tensor meta of the zero table: the address is the same in every lane but written so that the
+        // compiler does not see it (lane >> 6 is zero): a load it knows to be uniform is moved to scalar registers
+        // at once, which waits for it before any weight load has been issued.
+        uint32_t zms_raw = 0, zmz_raw = 0;
+        if constexpr (Q8) {
+            zms_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_ms) + (lane >> 6));
+            zmz_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_mz) + (lane >> 6));
+        }
         // ------------------------------------------------------------ loads: tables and x (lane l: columns 4l..4l+3), codes
         uint32_t sraw[10][2], zraw[10][2];
         u32x2 msr[10], mzr[10];
@@ -116,29 +160,47 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
             j -= j >= (uint32_t)p.G ? (uint32_t)p.G : 0u;
             const uint32_t ce = j * (uint32_t)K + k0 + (uint32_t)(4 * lane);
             if constexpr (Q8) {
-                sraw[i][0] = *reinterpret_cast<const uint32_t *>(p.sq + ce);
-                zraw[i][0] = *reinterpret_cast<const uint32_t *>(p.zq + ce);
-                uint32_t cm = ce - __umulhi(ce, p.s_inv) * p.s_cols; // ce mod cols; the quotient estimate is at most 2 short
-                cm -= cm >= p.s_cols ? p.s_cols : 0;
-                cm -= cm >= p.s_cols ? p.s_cols : 0;
-                msr[i] = *reinterpret_cast<const u32x2 *>(p.s_ms + cm);
-                mzr[i] = *reinterpret_cast<const u32x2 *>(p.s_mz + cm);
+                sraw[i][0] = gload<uint32_t>(R.sq + ce);
+                zraw[i][0] = gload<uint32_t>(R.zq + ce);
+                uint32_t cm = ce - __umulhi(ce, R.s_inv) * R.s_cols; // ce mod cols; the quotient estimate is at most 2 short
+                cm -= cm >= R.s_cols ? R.s_cols : 0;
+                cm -= cm >= R.s_cols ? R.s_cols : 0;
+                msr[i] = gload<u32x2>(R.s_ms + cm);
+                mzr[i] = gload<u32x2>(R.s_mz + cm);
             } else {
-                const u32x2 a = *reinterpret_cast<const u32x2 *>(reinterpret_cast<const f16 *>(p.sq) + ce);
-                const u32x2 b = *reinterpret_cast<const u32x2 *>(reinterpret_cast<const f16 *>(p.zq) + ce);
+                const u32x2 a = gload<u32x2>(reinterpret_cast<const f16 *>(R.sq) + ce);
+                const u32x2 b = gload<u32x2>(reinterpret_cast<const f16 *>(R.zq) + ce);
                 sraw[i][0] = a.x, sraw[i][1] = a.y, zraw[i][0] = b.x, zraw[i][1] = b.y;
             }
         }
-        u32x2 xr[MT];
+        u32x2 xr[MT], xg[XMODE ? MT : 1];
 #pragma unroll
-        for (int m = 0; m < MT; ++m)
-            xr[m] = *reinterpret_cast<const u32x2 *>(p.x + ((uint32_t)((m < M ? m : 0) * K) + k0 + (uint32_t)(4 * lane)));
+        for (int m = 0; m < MT; ++m) {
+            const uint32_t at = (uint32_t)((m < M ? m : 0) * K) + k0 + (uint32_t)(4 * lane);
+            if constexpr (XMODE) {
+                xg[m] = gload<u32x2>(p.xa + at);
+                xr[m] = gload<u32x2>(p.xb + at);
+            } else {
+                xr[m] = gload<u32x2>(p.x + at);
+            }
+        }
         u32x4 cw[16];
 #pragma unroll
         for (int m = 0; m < 16; ++m)
-            cw[m] = *reinterpret_cast<const u32x4 *>(p.codes + (code_base + 4u * k0 + (uint32_t)(64 * m)));
+            cw[m] = gload<u32x4>(R.codes + (code_base + 4u * k0 + (uint32_t)(64 * m)));
+        __builtin_amdgcn_sched_barrier(0); // nothing below moves above the loads, no load sinks into the arithmetic
+        if constexpr (Q8) // the meta values become opaque here, so no use of them is hoisted above the loads
+            asm volatile("" : "+v"(zms_raw), "+v"(zmz_raw));
 
         // ------------------------------------------------------------ table phase: xs into LDS, zero term accumulated
+        if constexpr (XMODE) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const f16x2 a01 = as_h2(xg[m].x), a23 = as_h2(xg[m].y), b01 = as_h2(xr[m].x), b23 = as_h2(xr[m].y);
+                xr[m].x = as_u32((f16x2){silu_mul(a01.x, b01.x), silu_mul(a01.y, b01.y)});
+                xr[m].y = as_u32((f16x2){silu_mul(a23.x, b23.x), silu_mul(a23.y, b23.y)});
+            }
+        }
         {
             const f16x2 k1024 = {(f16)1024.0f, (f16)1024.0f};
             const f16x2 k32 = {(f16)kXsScale, (f16)kXsScale};
@@ -220,7 +282,16 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
 
     // ---------------------------------------------------------------- block result
     const bool alone = p.BK == 1;
-    const int tile = w0 * p.RB + rb;
+    const int tile = (layer * p.P + w0) * p.RB + rb;
+    auto finish = [&](int m_t, int64_t n, float v) {
+        f16 val = (f16)v;
+        if (p.bias)
+            val = val + p.bias[n];
+        if (p.row_scale)
+            val = val * p.row_scale[m_t];
+        f16 *dst = yl + (int64_t)m_t * p.N + n;
+        *dst = p.accumulate ? (f16)(*dst + val) : val;
+    };
     for (int u = threadIdx.x; u < 16 * 10 * MT; u += NT) {
         const int m_t = u % MT, i_t = (u / MT) % 10, t_t = u / (10 * MT);
         float v = 0.f;
@@ -230,14 +301,10 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
         const int64_t n = 10 * wr_t + i_t;
         if (m_t >= M || wr_t >= p.NW || n >= p.N)
             continue;
-        if (alone) {
-            f16 val = (f16)v;
-            if (p.bias)
-                val = val + p.bias[n];
-            p.y[(int64_t)m_t * p.N + n] = val;
-        } else {
-            __hip_atomic_store(p.part + ((int64_t)kb * M + m_t) * p.N + n, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+        if (alone)
+            finish(m_t, n, v);
+        else
+            __hip_atomic_store(partl + ((int64_t)kb * M + m_t) * p.N + n, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (alone)
         return;
@@ -262,16 +329,13 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
             continue;
         float v = 0.f;
         for (int s = 0; s < p.BK; ++s)
-            v += __hip_atomic_load(p.part + ((int64_t)s * M + m_t) * p.N + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        f16 val = (f16)v;
-        if (p.bias)
-            val = val + p.bias[n];
-        p.y[(int64_t)m_t * p.N + n] = val;
+            v += __hip_atomic_load(partl + ((int64_t)s * M + m_t) * p.N + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        finish(m_t, n, v);
     }
 }
 
 struct W3Plan {
-    int G, P, NW, RB, NS, KS, SB, BK;
+    int G, P, NW, RB, NS, KS, S, SB, BK;
     bool q8;
 };
 
@@ -284,9 +348,10 @@ int gcd_int(int a, int b)
     return a;
 }
 
-bool make_plan(const hqq_linear *l, int64_t M, W3Plan &pl)
+// NL: layers of the launch (they share the plan)
+bool make_plan(const hqq_linear *l, int64_t M, int NL, W3Plan &pl)
 {
-    if (l->nbits != 3 || M < 1)
+    if (l->nbits != 3 || M < 1 || NL < 1 || NL > kW3MaxLayers)
         return false;
     const int64_t G = l->N / l->group_size;
     if (l->K % kSlab != 0 || G < 10 || G > (1 << 20))
@@ -311,14 +376,121 @@ bool make_plan(const hqq_linear *l, int64_t M, W3Plan &pl)
     pl.NS = (int)(l->K / kSlab);
     // blocks along K: enough that the windows cover the chip, and at most 16 slabs (8 waves x 2) per block
     int BK = (pl.NS + kW3Waves * kW3S - 1) / (kW3Waves * kW3S);
-    while ((int64_t)pl.P * pl.RB * BK < 200 && BK < pl.NS)
+    while ((int64_t)pl.P * pl.RB * NL * BK < 200 && BK < pl.NS)
         ++BK;
+    const bool tune = tuning_overrides() && (!std::getenv("HQQ_W3_K") || std::atoi(std::getenv("HQQ_W3_K")) == (int)l->K);
+    if (tune && std::getenv("HQQ_W3_BK"))
+        BK = std::atoi(std::getenv("HQQ_W3_BK"));
+    if (BK < 1 || BK > pl.NS || (pl.NS + BK - 1) / BK > kW3Waves * kW3S)
+        return false;
     pl.SB = (pl.NS + BK - 1) / BK;
     pl.BK = (pl.NS + pl.SB - 1) / pl.SB;
-    pl.KS = (pl.SB + kW3S - 1) / kW3S;
-    if (pl.P > 65535 || pl.RB > 65535 || (int64_t)pl.P * pl.RB * sizeof(int) > kCounterBytes)
+    pl.S = pl.SB > kW3Waves ? kW3S : 1;
+    if (tune && std::getenv("HQQ_W3_S"))
+        pl.S = std::atoi(std::getenv("HQQ_W3_S")) == 2 ? 2 : pl.S;
+    pl.KS = (pl.SB + pl.S - 1) / pl.S;
+    if ((int64_t)pl.P * NL > 65535 || pl.RB > 65535 || (int64_t)pl.P * pl.RB * NL * sizeof(int) > kCounterBytes)
         return false;
     return true;
+}
+
+// Layers that may share a launch: same shape, grouping and table layout (the records carry the pointers only).
+bool same_layout(const hqq_linear *a, const hqq_linear *b)
+{
+    return a->nbits == b->nbits && a->group_size == b->group_size && a->N == b->N && a->K == b->K &&
+           table_kind(a->scale) == table_kind(b->scale) && table_kind(a->zero) == table_kind(b->zero) &&
+           a->scale.meta_cols == b->scale.meta_cols;
+}
+
+struct W3Job {
+    const hqq_linear *layers[kW3MaxLayers]; // NL descriptors; with a table only layers[0] is read, for the shape
+    int NL;
+    const StripIndex *ix; // records from a device table: layer l is record sel[l / lper] * stride + first + l % lper
+    int lper;
+    const f16 *x, *xa, *xb; // x, or xa and xb (x = silu(xa) * xb)
+    f16 *y;
+    int64_t y_lstride;
+    SmallBatchEpilogue ep;
+};
+
+template <int MT, bool Q8> void launch_xmode(const W3Params &p, bool fused, dim3 grid, hipStream_t s)
+{
+    if (fused)
+        gemv_w3_kernel<MT, Q8, 1><<<grid, dim3(kW3Waves * 64), 0, s>>>(p);
+    else
+        gemv_w3_kernel<MT, Q8, 0><<<grid, dim3(kW3Waves * 64), 0, s>>>(p);
+}
+
+size_t job_workspace_bytes(const W3Plan &pl, const hqq_linear *l, int NL)
+{
+    return kCounterBytes + (pl.BK > 1 ? (size_t)NL * pl.BK * 2 * (size_t)l->N * sizeof(float) : 0);
+}
+
+int run_job(const W3Job &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
+{
+    const hqq_linear *l = j.layers[0];
+    W3Plan pl;
+    if (!make_plan(l, M, j.NL, pl))
+        return HQQ_E_UNSUPPORTED;
+    const bool fused = j.xa != nullptr;
+    if (!j.ix) {
+        for (int i = 1; i < j.NL; ++i) {
+            W3Plan other;
+            if (!same_layout(l, j.layers[i]) || !make_plan(j.layers[i], M, j.NL, other))
+                return HQQ_E_UNSUPPORTED;
+        }
+    }
+    for (int i = 0; i < (j.ix ? 1 : j.NL); ++i)
+        if (j.layers[i]->bias && (j.NL > 1 || j.ix))
+            return HQQ_E_UNSUPPORTED; // the bias is not part of a record
+    if (pl.BK > 1 && (!ws || ws_bytes < job_workspace_bytes(pl, l, j.NL)))
+        return HQQ_E_WORKSPACE;
+    if (fused ? ((reinterpret_cast<uintptr_t>(j.xa) | reinterpret_cast<uintptr_t>(j.xb)) & 7u) != 0
+              : (reinterpret_cast<uintptr_t>(j.x) & 7u) != 0)
+        return HQQ_E_ALIGN;
+    W3Params p = {};
+    if (j.ix) {
+        p.table = static_cast<const LayerRecord *>(j.ix->table);
+        p.sel = j.ix->sel;
+        p.stride = j.ix->stride, p.first = j.ix->first;
+    } else {
+        for (int i = 0; i < j.NL; ++i)
+            fill_layer_record(p.layer[i], j.layers[i]);
+        p.bias = static_cast<const f16 *>(l->bias);
+    }
+    p.lper = j.lper > 0 ? j.lper : 1;
+    p.counter = static_cast<int *>(ws);
+    p.part = pl.BK > 1 ? reinterpret_cast<float *>(static_cast<char *>(ws) + kCounterBytes) : nullptr;
+    p.part_lstride = (int64_t)pl.BK * 2 * l->N;
+    p.y_lstride = j.y_lstride;
+    p.accumulate = j.ep.accumulate;
+    p.N = (int)l->N, p.K = (int)l->K, p.G = pl.G, p.P = pl.P, p.NW = pl.NW, p.RB = pl.RB;
+    p.NS = pl.NS, p.KS = pl.KS, p.S = pl.S, p.SB = pl.SB, p.BK = pl.BK;
+    const dim3 grid((unsigned)pl.BK, (unsigned)pl.RB, (unsigned)(pl.P * j.NL));
+    for (int64_t m0 = 0; m0 < M; m0 += 2) { // passes of two batch rows; later passes find the weights in the caches
+        const int mb = M - m0 >= 2 ? 2 : 1;
+        if (fused)
+            p.xa = j.xa + m0 * l->K, p.xb = j.xb + m0 * l->K;
+        else
+            p.x = j.x + m0 * l->K;
+        p.y = j.y + m0 * l->N, p.M = mb;
+        p.row_scale = j.ep.row_scale ? j.ep.row_scale + m0 : nullptr;
+        if (mb == 1) {
+            if (pl.q8)
+                launch_xmode<1, true>(p, fused, grid, s);
+            else
+                launch_xmode<1, false>(p, fused, grid, s);
+        } else {
+            if (pl.q8)
+                launch_xmode<2, true>(p, fused, grid, s);
+            else
+                launch_xmode<2, false>(p, fused, grid, s);
+        }
+        int rc = launch_status();
+        if (rc != HQQ_OK)
+            return rc;
+    }
+    return HQQ_OK;
 }
 
 } // namespace
@@ -326,59 +498,62 @@ bool make_plan(const hqq_linear *l, int64_t M, W3Plan &pl)
 bool vec3_supported(const hqq_linear *l, int64_t M)
 {
     W3Plan pl;
-    return M <= 16 && make_plan(l, M, pl);
+    return M <= 16 && make_plan(l, M, 1, pl);
 }
 
 size_t vec3_workspace_bytes(const hqq_linear *l, int64_t M)
 {
     W3Plan pl;
-    if (!make_plan(l, M, pl))
+    if (!make_plan(l, M, 1, pl))
         return 0;
-    return kCounterBytes + (size_t)pl.BK * 2 * (size_t)l->N * sizeof(float);
+    return job_workspace_bytes(pl, l, 1);
 }
 
 int launch_vec3_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s)
 {
+    W3Job j = {};
+    j.layers[0] = l, j.NL = 1, j.x = x, j.y = y;
+    return run_job(j, M, ws, ws_bytes, s);
+}
+
+// The expert FFN of 3-bit layers in two launches: both gate projections (of one expert, or of the experts sel[0] and
+// sel[1] of a record table), then the down projection reading silu(a) * b.
+bool vec3_ffn_supported(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, int64_t M, int n_experts)
+{
     W3Plan pl;
-    if (!make_plan(l, M, pl))
+    return M >= 1 && M <= 16 && same_layout(w1, w3) && !w1->bias && !w3->bias && make_plan(w1, M, 2 * n_experts, pl) &&
+           make_plan(w3, M, 2 * n_experts, pl) && make_plan(w2, M, 1, pl) && w2->K == w1->N && w2->N == w1->K;
+}
+
+size_t vec3_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2, int64_t M, int n_experts)
+{
+    W3Plan a, b;
+    if (!make_plan(w1, M, 2 * n_experts, a) || !make_plan(w2, M, 1, b))
+        return 0;
+    const size_t ga = job_workspace_bytes(a, w1, 2 * n_experts), gb = job_workspace_bytes(b, w2, 1);
+    return ga > gb ? ga : gb;
+}
+
+// ab: the gate outputs, layer l (w1 then w3 of each expert) at ab + l * ab_lstride, each (M, N)
+int launch_vec3_gate(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *ab, int64_t ab_lstride,
+                     int n_experts, void *ws, size_t ws_bytes, hipStream_t s, const StripIndex *ix)
+{
+    if (n_experts < 1 || n_experts > 2 || (n_experts == 2 && !ix) || ab_lstride < M * w1->N)
         return HQQ_E_UNSUPPORTED;
-    if (pl.BK > 1 && (!ws || ws_bytes < vec3_workspace_bytes(l, M)))
-        return HQQ_E_WORKSPACE;
-    if (reinterpret_cast<uintptr_t>(x) & 7u)
-        return HQQ_E_ALIGN;
-    W3Params p = {};
-    p.codes = static_cast<const uint8_t *>(l->codes);
-    p.sq = static_cast<const uint8_t *>(l->scale.data);
-    p.zq = static_cast<const uint8_t *>(l->zero.data);
-    p.s_ms = static_cast<const f16 *>(l->scale.meta_scale), p.s_mz = static_cast<const f16 *>(l->scale.meta_zero);
-    p.z_ms = static_cast<const f16 *>(l->zero.meta_scale), p.z_mz = static_cast<const f16 *>(l->zero.meta_zero);
-    p.s_cols = (uint32_t)l->scale.meta_cols;
-    p.s_inv = p.s_cols ? (uint32_t)(0xFFFFFFFFull / p.s_cols) : 0;
-    p.bias = static_cast<const f16 *>(l->bias);
-    p.counter = static_cast<int *>(ws);
-    p.part = pl.BK > 1 ? reinterpret_cast<float *>(static_cast<char *>(ws) + kCounterBytes) : nullptr;
-    p.N = (int)l->N, p.K = (int)l->K, p.G = pl.G, p.P = pl.P, p.NW = pl.NW, p.RB = pl.RB;
-    p.NS = pl.NS, p.KS = pl.KS, p.SB = pl.SB, p.BK = pl.BK;
-    const dim3 grid((unsigned)pl.BK, (unsigned)pl.RB, (unsigned)pl.P), block(kW3Waves * 64);
-    for (int64_t m0 = 0; m0 < M; m0 += 2) { // passes of two batch rows; later passes find the weights in the caches
-        const int mb = M - m0 >= 2 ? 2 : 1;
-        p.x = x + m0 * l->K, p.y = y + m0 * l->N, p.M = mb;
-        if (mb == 1) {
-            if (pl.q8)
-                gemv_w3_kernel<1, true><<<grid, block, 0, s>>>(p);
-            else
-                gemv_w3_kernel<1, false><<<grid, block, 0, s>>>(p);
-        } else {
-            if (pl.q8)
-                gemv_w3_kernel<2, true><<<grid, block, 0, s>>>(p);
-            else
-                gemv_w3_kernel<2, false><<<grid, block, 0, s>>>(p);
-        }
-        int rc = launch_status();
-        if (rc != HQQ_OK)
-            return rc;
-    }
-    return HQQ_OK;
+    W3Job j = {};
+    j.layers[0] = w1, j.layers[1] = w3, j.layers[2] = w1, j.layers[3] = w3;
+    j.NL = 2 * n_experts, j.ix = ix, j.lper = 2;
+    j.x = x, j.y = ab, j.y_lstride = ab_lstride;
+    return run_job(j, M, ws, ws_bytes, s);
+}
+
+int launch_vec3_down(const hqq_linear *w2, const f16 *a, const f16 *b, int64_t M, f16 *y, void *ws, size_t ws_bytes,
+                     const SmallBatchEpilogue &ep, hipStream_t s, const StripIndex *ix)
+{
+    W3Job j = {};
+    j.layers[0] = w2, j.NL = 1, j.ix = ix, j.lper = 1;
+    j.xa = a, j.xb = b, j.y = y, j.ep = ep;
+    return run_job(j, M, ws, ws_bytes, s);
 }
 
 } // namespace hqq

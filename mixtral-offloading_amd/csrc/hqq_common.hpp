@@ -112,6 +112,30 @@ int launch_smallbatch_gate_up(const hqq_linear *w1, const hqq_linear *w3, const 
 // slabs of 256 columns per wave, in-block gate epilogue
 bool strip_supported(const hqq_linear *l, int64_t M);
 size_t strip_workspace_bytes(const hqq_linear *l, int64_t M);
+// What a decode kernel needs to know of a layer besides its shape; also the record of a device-side expert table.
+struct LayerRecord {
+    const uint8_t *codes;
+    const uint8_t *sq, *zq; // 8-bit tables, or fp16 tables
+    const f16 *s_ms, *s_mz; // meta of the scale table
+    const f16 *z_ms, *z_mz; // meta of the zero table
+    uint32_t s_cols, z_cols, s_inv, z_inv; // meta columns and floor(2^32 / columns)
+};
+static_assert(sizeof(LayerRecord) == 72, "the record is read as 18 words");
+inline void fill_layer_record(LayerRecord &L, const hqq_linear *l)
+{
+    L.codes = static_cast<const uint8_t *>(l->codes);
+    L.sq = static_cast<const uint8_t *>(l->scale.data);
+    L.zq = static_cast<const uint8_t *>(l->zero.data);
+    L.s_ms = static_cast<const f16 *>(l->scale.meta_scale);
+    L.s_mz = static_cast<const f16 *>(l->scale.meta_zero);
+    L.z_ms = static_cast<const f16 *>(l->zero.meta_scale);
+    L.z_mz = static_cast<const f16 *>(l->zero.meta_zero);
+    L.s_cols = (uint32_t)l->scale.meta_cols;
+    L.z_cols = (uint32_t)l->zero.meta_cols;
+    L.s_inv = L.s_cols ? (uint32_t)(0xFFFFFFFFull / L.s_cols) : 0;
+    L.z_inv = L.z_cols ? (uint32_t)(0xFFFFFFFFull / L.z_cols) : 0;
+}
+
 // Indexed launch: the layer records come from a device table of strip_record_bytes() records, record
 // sel[0] * stride + first (+ 1 for the second projection of the gate); the descriptors passed alongside only give
 // the shape, which every record of the table must share.
@@ -155,6 +179,14 @@ int launch_tile_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x
 bool vec3_supported(const hqq_linear *l, int64_t M);
 size_t vec3_workspace_bytes(const hqq_linear *l, int64_t M);
 int launch_vec3_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s);
+// 3-bit expert FFN in two launches: the gate projections of n_experts experts (ab: layer l at ab + l * ab_lstride,
+// w1 then w3 of each expert; two experts only from a record table), then the down projection reading silu(a) * b
+bool vec3_ffn_supported(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, int64_t M, int n_experts);
+size_t vec3_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2, int64_t M, int n_experts);
+int launch_vec3_gate(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *ab, int64_t ab_lstride,
+                     int n_experts, void *ws, size_t ws_bytes, hipStream_t s, const StripIndex *ix = nullptr);
+int launch_vec3_down(const hqq_linear *w2, const f16 *a, const f16 *b, int64_t M, f16 *y, void *ws, size_t ws_bytes,
+                     const SmallBatchEpilogue &ep, hipStream_t s, const StripIndex *ix = nullptr);
 int launch_router_top2(const f16 *x, const f16 *w, int n_experts, int64_t hidden, int *sel, f16 *weights, f16 *logits,
                        hipStream_t s);
 int launch_add_rmsnorm(f16 *x, const f16 *delta, const f16 *weight, float eps, f16 *y, int64_t hidden, hipStream_t s);

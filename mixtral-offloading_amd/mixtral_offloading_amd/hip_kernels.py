@@ -239,6 +239,12 @@ def expert_pair_supported(table: ExpertTable) -> bool:
     return _lib.lib.hqq_expert_pair_ffn_workspace_bytes(w1.ref, w2.ref, w3.ref) > 0
 
 
+def moe_pair_routed_supported(table: ExpertTable, hidden: int, n_experts: int) -> bool:
+    """Whether ``moe_pair_routed`` takes this layer: the two-launch pair, 2- or 4-bit experts, a row of at most 4096."""
+    return (expert_pair_supported(table) and table.shape[0].nbits != 3 and hidden <= 4096 and hidden % 8 == 0
+            and 2 <= n_experts <= 8)
+
+
 def expert_pair_ffn_indexed(table: ExpertTable, expert_index: torch.Tensor, x: torch.Tensor, out: torch.Tensor,
                             row_scale: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
     """``out (+)= sum_e expert_ffn_{expert_index[e]}(x) * row_scale[e]`` over the two active experts of one token

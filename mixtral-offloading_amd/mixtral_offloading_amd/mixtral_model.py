@@ -140,7 +140,7 @@ class DecodeGraph:
                 [(m._expert[0].w1._desc(), m._expert[0].w2._desc(), m._expert[0].w3._desc()) for m in mods]))
         # the two active experts in two launches, q / k / v in one, where the shapes allow
         self.pair = all(hip_kernels.expert_pair_supported(t) for t in self.tables)
-        self.routed = self.pair and cfg.hidden_size <= 4096 and cfg.hidden_size % 8 == 0 and 2 <= cfg.num_local_experts <= 8
+        self.routed = all(hip_kernels.moe_pair_routed_supported(t, cfg.hidden_size, cfg.num_local_experts) for t in self.tables)
         self.qkv = [hip_kernels.LinearGroup([p._desc() for p in (l.self_attn.q_proj, l.self_attn.k_proj, l.self_attn.v_proj)])
                     for l in model.model.layers]
         self.cache = model.new_cache(max_len)

@@ -77,22 +77,23 @@ def test_add_rmsnorm_router_equals_the_two_calls(n_experts, hidden):
             assert float((rw1.float() - rw2.float()).abs().max()) <= 2e-3
 
 
+@pytest.mark.parametrize("nbits,hidden,ffn,gs", [(2, 512, 1024, 16), (3, 768, 1280, 64)])
 @pytest.mark.parametrize("m", [1, 2, 4])
-def test_expert_ffn_indexed_equals_direct(m):
+def test_expert_ffn_indexed_equals_direct(m, nbits, hidden, ffn, gs):
     from mixtral_offloading_amd import hip_kernels
     rng = np.random.default_rng(17 + m)
     experts = []
     for e in range(4):
-        w1, _ = o.random_layer(rng, 1024, 512, 2, 16)
-        w3, _ = o.random_layer(rng, 1024, 512, 2, 16)
-        w2, _ = o.random_layer(rng, 512, 1024, 2, 16)
+        w1, _ = o.random_layer(rng, ffn, hidden, nbits, gs)
+        w3, _ = o.random_layer(rng, ffn, hidden, nbits, gs)
+        w2, _ = o.random_layer(rng, hidden, ffn, nbits, gs)
         experts.append((desc_of(w1), desc_of(w2), desc_of(w3)))
     table = hip_kernels.ExpertTable(experts)
-    x = to_dev(rng.standard_normal((m, 512)).astype(np.float16))
+    x = to_dev(rng.standard_normal((m, hidden)).astype(np.float16))
     rw = to_dev(rng.uniform(0.2, 0.8, size=(m,)).astype(np.float16))
     for e in (2, 0, 3):
         idx = torch.tensor([e], dtype=torch.int32, device="cuda")
-        base = to_dev(rng.standard_normal((m, 512)).astype(np.float16))
+        base = to_dev(rng.standard_normal((m, hidden)).astype(np.float16))
         want = base.clone()
         hip_kernels.expert_ffn(*experts[e], x, out=want, row_scale=rw, accumulate=True)
         got = base.clone()
@@ -105,7 +106,7 @@ def test_expert_ffn_indexed_equals_direct(m):
 
 # (nbits, hidden, ffn, group size, quantised tables): K of the down projections split over one and several blocks
 PAIR_SHAPES = [(2, 512, 1024, 16, True), (2, 1024, 3584, 16, True), (4, 512, 2048, 64, True), (2, 256, 768, 16, False),
-               (2, 4096, 14336, 16, True)]
+               (2, 4096, 14336, 16, True), (3, 768, 1280, 64, True), (3, 1024, 2560, 32, False), (3, 4096, 14336, 64, True)]
 
 
 @pytest.mark.parametrize("shape", PAIR_SHAPES, ids=lambda s: "w%d_h%d_f%d_g%d_%s" % (s[0], s[1], s[2], s[3], "q" if s[4] else "f16"))
@@ -244,19 +245,29 @@ def test_matmul_group_refuses_mixed_layers():
     assert not hip_kernels.LinearGroup([desc_of(a), desc_of(b)]).supported
 
 
-def test_graph_decode_matches_eager_logits():
+@pytest.mark.parametrize("ffn_bits", [2, 3])
+def test_graph_decode_matches_eager_logits(ffn_bits):
     """Each replayed step must give the logits of the eager forward at the same position (same kernels for the
-    quantized linears; attention over the masked full cache instead of the sliced one)."""
+    quantized linears; attention over the masked full cache instead of the sliced one).  With 3-bit experts the
+    step takes the norm + router launch and the three-launch expert pair instead of the routed pair."""
     from mixtral_offloading_amd import build_model as bm
+    from mixtral_offloading_amd.hqq_core import BaseQuantizeConfig
     from mixtral_offloading_amd.mixtral_model import DecodeGraph
-    cfg = bm.mixtral_config(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
-                            num_key_value_heads=2, vocab_size=128, num_local_experts=8)
+    qc = bm.default_quant_config()
+    if ffn_bits == 2:
+        cfg = bm.mixtral_config(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                                num_key_value_heads=2, vocab_size=128, num_local_experts=8)
+    else:
+        cfg = bm.mixtral_config(hidden_size=1024, intermediate_size=1280, num_hidden_layers=2, num_attention_heads=8,
+                                num_key_value_heads=2, vocab_size=128, num_local_experts=8)
+        qc = bm.QuantConfig(ffn_config=BaseQuantizeConfig(nbits=3, group_size=64, quant_zero=True, quant_scale=True),
+                            attn_config=qc.attn_config)
     off = bm.OffloadConfig(main_size=16, offload_size=0, buffer_size=1, offload_per_layer=0)
-    model = bm.build_model(torch.device("cuda:0"), bm.default_quant_config(), off, model_config=cfg, seed=5,
-                           max_positions=64)
+    model = bm.build_model(torch.device("cuda:0"), qc, off, model_config=cfg, seed=5, max_positions=64)
     prompt = torch.randint(0, 128, (9,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(2))
     steps = 6
     dec = DecodeGraph(model, prompt.numel() + steps + 4)
+    assert dec.pair and dec.routed == (ffn_bits == 2)
     first = dec.prefill(prompt)
     dec.capture()
     # eager reference driven with the graph's own tokens

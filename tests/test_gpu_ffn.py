@@ -18,6 +18,9 @@ SHAPES = [
     (4, 512, 1024, 64, True),    # four row blocks per tile
     (4, 256, 512, 32, False),    # fp16 tables
     (2, 768, 1280, 16, False),
+    (3, 768, 1280, 64, True),    # 3-bit: both gate projections in one launch, silu(a) * b applied by the down projection
+    (3, 1024, 2560, 32, True),   # K of the down projection split over blocks
+    (3, 1280, 768, 64, False),   # fp16 tables
 ]
 
 
@@ -52,15 +55,16 @@ def test_expert_ffn_against_oracle(shape, m):
         assert_matmul_close(y, ref, atol, rtol=2e-2)
 
 
-@pytest.mark.parametrize("m", [1, 2, 4])
-def test_expert_ffn_row_scale_and_accumulate(m):
+@pytest.mark.parametrize("nbits,hidden,ffn,gs", [(2, 512, 1792, 16), (3, 768, 1280, 64)])
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+def test_expert_ffn_row_scale_and_accumulate(m, nbits, hidden, ffn, gs):
     """Routing weight and the index_add_ of the reference (src/custom_layers.py:308-312) as the FFN's epilogue."""
     from mixtral_offloading_amd import hip_kernels
     rng = np.random.default_rng(7 + m)
-    w1, w2, w3 = _ffn_case(rng, 2, 512, 1792, 16, True)
-    x = rng.standard_normal((m, 512)).astype(np.float16)
+    w1, w2, w3 = _ffn_case(rng, nbits, hidden, ffn, gs, True)
+    x = rng.standard_normal((m, hidden)).astype(np.float16)
     rw = rng.uniform(0.1, 0.9, size=(m,)).astype(np.float16)
-    base = rng.standard_normal((m, 512)).astype(np.float16)
+    base = rng.standard_normal((m, hidden)).astype(np.float16)
     d1, d2, d3 = desc_of(w1), desc_of(w2), desc_of(w3)
     plain = hip_kernels.expert_ffn(d1, d2, d3, to_dev(x))
     out = to_dev(base.copy())
@@ -70,13 +74,14 @@ def test_expert_ffn_row_scale_and_accumulate(m):
     assert torch.equal(out, want)
 
 
+@pytest.mark.parametrize("nbits,gs", [(2, 16), (3, 64)])
 @pytest.mark.parametrize("m", [1, 2, 4, 8])
-def test_ffn_entry_point_equals_its_three_steps(m):
+def test_ffn_entry_point_equals_its_three_steps(m, nbits, gs):
     """hqq_expert_ffn rounds where the reference's three layers do (fp16 after each matmul, fp16 silu * up): it gives
     the bits that two hqq_matmul_transpose calls, torch's silu * up and a third call give, whatever kernels it picks."""
     from mixtral_offloading_amd import hip_kernels
     rng = np.random.default_rng(11 + m)
-    w1, w2, w3 = _ffn_case(rng, 2, 1024, 3584, 16, True)
+    w1, w2, w3 = _ffn_case(rng, nbits, 1024, 3584 if nbits == 2 else 2560, gs, True)
     x = to_dev(rng.standard_normal((m, 1024)).astype(np.float16))
     d1, d2, d3 = desc_of(w1), desc_of(w2), desc_of(w3)
     whole = hip_kernels.expert_ffn(d1, d2, d3, x)
