@@ -141,9 +141,10 @@ int hqq_expert_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq
 
 /* ---- both experts of one token in two launches instead of four: y (+)= sum over e < 2 of
  *      fp16(FFN_{expert_index[e]}(x)) * row_scale[e], the loop body of src/custom_layers.py:298-312 for the two
- *      active experts of a single token, each product and the sum rounded to fp16 as index_add_ on fp16 tensors
- *      rounds them (what two hqq_expert_ffn_indexed calls give, the second accumulating, up to the order in which the
- *      fp32 partial sums over K are added).  One launch
+ *      active experts of a single token (what two hqq_expert_ffn_indexed calls give, the second accumulating, up to
+ *      the order in which the fp32 partial sums over K are added and, where K of the down projection is split over
+ *      blocks, up to one fp16 rounding: the weighted sum of both experts is then formed in higher precision and
+ *      rounded once, where index_add_ on fp16 tensors rounds each product and the sum).  One launch
  *      computes silu(w1 x) * w3 x of both experts, one both down projections and their weighted sum (3-bit experts:
  *      three launches -- the four gate projections, then one down projection per expert that applies silu(a) * b
  *      as it reads them, the second adding into y).  x is one row

@@ -9,7 +9,30 @@ namespace gemv {
 
 constexpr int kSlab = 256;           // columns per wave
 constexpr float kXsScale = 32.0f;    // xs = 32 * s * x keeps small activations out of the fp16 subnormal range
-constexpr size_t kCounterBytes = 64 * 1024; // head of the workspace: one arrival counter per tile
+// Head of every workspace, zero between launches: one arrival counter per tile, then the accumulation slots of the
+// split-K decode launches (one 64-bit word per output of the launch).
+constexpr size_t kCounterBytes = 64 * 1024;
+constexpr size_t kSlotBytes = 512 * 1024;
+constexpr size_t kHeadBytes = kCounterBytes + kSlotBytes;
+// A slot holds the sum of the K blocks' partial results as a fixed-point number (34 fractional bits, magnitudes up
+// to 2^17 per contribution, at most 8 of them) and, above bit 56, the number of blocks that have added theirs.
+// Integer addition is exact, so the total does not depend on the order of arrival; the block whose addition
+// completes a slot reads the total out of the value its own atomic returns, writes the output and clears the slot:
+// one trip to memory instead of three (partial sums, arrival counter, partial sums again).
+constexpr int kSlotFracBits = 34;
+constexpr float kSlotLimit = 131071.0f;
+__device__ __forceinline__ unsigned long long slot_term(float v)
+{
+    v = v < -kSlotLimit ? -kSlotLimit : (v > kSlotLimit ? kSlotLimit : v); // NaN passes and converts to 0
+    const long long fx = (long long)__builtin_rintf(v * (float)(1ull << kSlotFracBits)); // exact scaling by 2^34
+    return (1ull << 56) + (unsigned long long)fx;
+}
+__device__ __forceinline__ int slot_count(unsigned long long word) { return (int)((word + (1ull << 55)) >> 56); }
+__device__ __forceinline__ float slot_total(unsigned long long word, int count)
+{
+    const long long fx = (long long)(word - ((unsigned long long)count << 56));
+    return (float)((double)fx * (1.0 / (double)(1ull << kSlotFracBits)));
+}
 
 enum { TK_U8_COLS = 1, TK_U8_SCALAR = 2, TK_F16 = 3 };
 

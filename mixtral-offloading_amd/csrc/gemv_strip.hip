@@ -12,8 +12,11 @@
 // per lane, and for the table lanes 16 scale bytes, 16 zero bytes, their fp16 meta values and x -- and the loads of
 // up to D slabs are in flight before the first arithmetic.  When the block holds all of K (BK == 1: every Mixtral
 // projection with K = 4096, gate included) it applies the epilogue itself: no workspace, no atomics.  Otherwise
-// (K = 14336) the BK blocks of a tile store fp32 partial sums with device-scope stores and the block that arrives
-// last at the tile's counter adds them in a fixed order.
+// (K = 14336) the BK blocks of a tile add their results into one 64-bit accumulation slot per output (fixed point,
+// so the sum is exact and independent of the order of arrival) with a returning device-scope atomic; the block
+// whose addition completes a slot writes that output.  The gate epilogue with K over several blocks (not a
+// Mixtral shape) instead stores fp32 partial sums with device-scope stores, and the block that arrives last at the
+// tile's counter adds them in a fixed order.
 //
 // Lane roles inside a slab.  Code lanes: (rr = lane & 15, kg = lane >> 4) own packed row jp + (16*rb + rr)*GP,
 // bytes 64*s + 16*kg .. +15 for step s.  Table lanes: (ti = lane >> 4 < F, kq = lane & 15) own table row F*jp + ti,
@@ -36,7 +39,8 @@ using StripLayer = LayerRecord;
 // the gates of two experts in one launch).
 constexpr int kMaxGroups = 4;
 struct StripGroup {
-    int z_begin, GP, N, pad;
+    int z_begin, GP, N;
+    int slot_begin; // first accumulation slot of the group: slot (slot_begin + n * MT + m) belongs to output (m, n)
     f16 *y;
     const f16 *bias;
     float *part[2]; // [BK][M][N] per layer
@@ -61,6 +65,7 @@ struct StripParams {
     int BK;       // blocks along K per tile
     int NL;       // layers per block (2: fused gate, or the down projections of two experts)
     int *counter; // one per tile, zero between launches
+    unsigned long long *slots; // EPI 0 and 2 with K over several blocks: accumulation slots instead of partial sums (or null)
     const f16 *row_scale;
     int rs_lstride; // EPI 2: layer l scales by row_scale[l * rs_lstride + m]
     int accumulate;
@@ -499,7 +504,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
             continue;
         const int r = 16 * rb + r_t;
         const int64_t n = (int64_t)F * (jp + (int64_t)r * GP); // outputs n .. n+F-1
-        if (!alone) {
+        if (!alone && (EPI == 1 || !p.slots)) {
             // device-scope stores: written through the (per-XCD, mutually non-coherent) L2 so that the finishing
             // block, which may run on another XCD, can read them without any cache-wide flush
             float *dst = (l_t ? Gd.part[1] : Gd.part[0]) + ((int64_t)kb * M + m_t) * N + n;
@@ -508,7 +513,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
                 __hip_atomic_store(dst + i, o[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             continue;
         }
-        if constexpr (EPI != 0) {
+        if (EPI != 0 || !alone) {
             float *dst = &fin_lds[l_t][r_t][m_t][0];
 #pragma unroll
             for (int i = 0; i < F; ++i)
@@ -572,6 +577,42 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
             }
         }
         return;
+    }
+
+    // ---------------------------------------------------------------- accumulation slots: one atomic per output
+    if constexpr (EPI != 1) {
+        if (p.slots) {
+            __syncthreads();
+            for (int u = threadIdx.x; u < 16 * MT * F; u += WAVES * 64) {
+                const int i = u % F, m_t = (u / F) % MT, r_t = u / (F * MT);
+                if (m_t >= M)
+                    continue;
+                const int r = 16 * rb + r_t;
+                const int64_t n = (int64_t)F * (jp + (int64_t)r * GP) + i;
+                unsigned long long *slot = p.slots + (Gd.slot_begin + n * MT + m_t);
+                // EPI 2: the routing weights are applied to the block's partial results in fp32, so the two experts
+                // share a slot and the weighted sum is rounded to fp16 once
+                float term = fin_lds[0][r_t][m_t][i];
+                if constexpr (EPI == 2)
+                    term = term * (float)p.row_scale[m_t] + fin_lds[1][r_t][m_t][i] * (float)p.row_scale[p.rs_lstride + m_t];
+                const unsigned long long mine = slot_term(term);
+                const unsigned long long before = __hip_atomic_fetch_add(slot, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (slot_count(before) != p.BK - 1)
+                    continue;
+                // this addition completed the slot: leave it ready for the next launch, write the output
+                __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                f16 val = (f16)slot_total(before + mine, p.BK);
+                if constexpr (EPI == 0) {
+                    if (Gd.bias)
+                        val = val + Gd.bias[n];
+                    if (p.row_scale)
+                        val = val * p.row_scale[m_t];
+                }
+                f16 *dst = Gd.y + (int64_t)m_t * N + n;
+                *dst = p.accumulate ? (f16)(*dst + val) : val;
+            }
+            return;
+        }
     }
 
     // ---------------------------------------------------------------- the block that arrives last finishes the tile
@@ -865,14 +906,15 @@ int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t
     if (!plan_job(j, M, pl, per_group, part_bytes))
         return HQQ_E_UNSUPPORTED;
     const bool alone = pl.BK == 1;
-    if (!alone && (!ws || ws_bytes < kCounterBytes + part_bytes))
+    if (!alone && (!ws || ws_bytes < kHeadBytes + part_bytes))
         return HQQ_E_WORKSPACE;
     if (j.EPI == 2 && !j.row_scale)
         return HQQ_E_NULL;
     StripParams p = {};
     char *base = static_cast<char *>(ws);
-    char *part = base + kCounterBytes;
+    char *part = base + kHeadBytes;
     int z = 0;
+    int64_t slot = 0;
     for (int g = 0; g < kMaxGroups; ++g) {
         StripGroup &G = p.grp[g];
         if (g >= j.NG) {
@@ -881,6 +923,8 @@ int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t
         }
         const hqq_linear *a = j.shape[g * j.NL];
         G.z_begin = z, G.GP = per_group[g].GP, G.N = (int)a->N;
+        G.slot_begin = (int)slot;
+        slot += a->N * pl.MT;
         G.y = j.y[g];
         G.bias = j.EPI == 0 ? static_cast<const f16 *>(a->bias) : nullptr;
         for (int l = 0; l < j.NL; ++l) {
@@ -906,6 +950,10 @@ int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t
     p.x = j.x, p.x_lstride = (int)j.x_lstride, p.M = (int)M, p.K = (int)j.shape[0]->K;
     p.RB = pl.RB, p.NS = pl.NS, p.KS = pl.KS, p.BK = pl.BK, p.NL = j.NL;
     p.counter = reinterpret_cast<int *>(base);
+    // plain or weighted-pair epilogue, K over at most eight blocks, every output of the launch has a slot: no
+    // partial sums
+    if (!alone && ((j.EPI == 0 && j.NL == 1) || (j.EPI == 2 && j.NL == 2 && j.NG == 1)) && pl.BK <= 8 && slot * (int64_t)sizeof(unsigned long long) <= (int64_t)kSlotBytes)
+        p.slots = reinterpret_cast<unsigned long long *>(base + kCounterBytes);
     p.row_scale = j.row_scale, p.rs_lstride = j.rs_lstride, p.accumulate = j.accumulate;
     if (j.norm_weight) {
         // every launch shape the planner can pick for these jobs has the fused-norm form except blocks under four waves
@@ -952,7 +1000,7 @@ size_t strip_workspace_bytes(const hqq_linear *l, int64_t M)
     if (!make_plan(l, M, 1, pl))
         return 0;
     // sized for the worst split the planner may choose for this shape (one slab per wave and block)
-    return kCounterBytes + (size_t)pl.NS * (size_t)M * (size_t)l->N * sizeof(float);
+    return kHeadBytes + (size_t)pl.NS * (size_t)M * (size_t)l->N * sizeof(float);
 }
 
 int launch_strip_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
@@ -1049,18 +1097,18 @@ size_t strip_job_workspace_bytes(const hqq_linear *const *layers, int count, int
     size_t part = 0;
     if (!plan_job(j, M, pl, per_group, part))
         return 0;
-    return kCounterBytes + part;
+    return kHeadBytes + part;
 }
 
 int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s)
 {
-    const size_t n = (ws_bytes < kCounterBytes ? ws_bytes : kCounterBytes) / 4;
+    const size_t n = (ws_bytes < kHeadBytes ? ws_bytes : kHeadBytes) / 4;
     if (n == 0)
         return HQQ_OK;
     zero_words_kernel<<<16, 256, 0, s>>>(static_cast<uint32_t *>(ws), n);
     return launch_status();
 }
 
-size_t workspace_head_bytes() { return kCounterBytes; }
+size_t workspace_head_bytes() { return kHeadBytes; }
 
 } // namespace hqq

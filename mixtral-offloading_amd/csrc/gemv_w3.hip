@@ -15,8 +15,10 @@
 // leaves xs in LDS; the zero term is a dot product per table row, summed over the wave at the end.
 //
 // The waves of a block split K (two slabs each); when K needs several blocks (or the window count alone would leave
-// most of the chip idle) the blocks of a tile store fp32 partial sums with device-scope stores and the block that
-// arrives last at the tile's counter adds them in a fixed order.  Batches above two rows run as passes of two.
+// most of the chip idle) the blocks of a tile add their results into one 64-bit fixed-point accumulation slot per
+// output with a returning device-scope atomic, and the block whose addition completes a slot writes that output
+// (launches with more outputs than there are slots store fp32 partial sums instead, and the block that arrives
+// last at the tile's counter adds them in a fixed order).  Batches above two rows run as passes of two.
 //
 // A launch may hold up to four layers of one shape (blockIdx.z = layer * P + window): the two projections of an
 // expert's gate, or those of two experts.  Their records come from the kernel arguments or from a device table
@@ -51,6 +53,7 @@ struct W3Params {
     float *part; // layer l: part + l * part_lstride, [BK][M][N]
     int64_t part_lstride;
     int *counter;
+    unsigned long long *slots; // K over several blocks: one accumulation slot per output of the launch (or null)
     int M, N, K, G, P, NW, RB;
     int NS; // K / 256
     int KS; // waves of a block that have slabs
@@ -301,12 +304,22 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
         const int64_t n = 10 * wr_t + i_t;
         if (m_t >= M || wr_t >= p.NW || n >= p.N)
             continue;
-        if (alone)
+        if (alone) {
             finish(m_t, n, v);
-        else
+        } else if (p.slots) {
+            // the K blocks add into the output's slot; the block whose addition completes it writes the output
+            unsigned long long *slot = p.slots + (((int64_t)layer * p.N + n) * MT + m_t);
+            const unsigned long long mine = slot_term(v);
+            const unsigned long long before = __hip_atomic_fetch_add(slot, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (slot_count(before) == p.BK - 1) {
+                __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                finish(m_t, n, slot_total(before + mine, p.BK));
+            }
+        } else {
             __hip_atomic_store(partl + ((int64_t)kb * M + m_t) * p.N + n, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
-    if (alone)
+    if (alone || p.slots)
         return;
 
     // the block that arrives last at the tile's counter adds the partial sums in a fixed order
@@ -423,7 +436,7 @@ template <int MT, bool Q8> void launch_xmode(const W3Params &p, bool fused, dim3
 
 size_t job_workspace_bytes(const W3Plan &pl, const hqq_linear *l, int NL)
 {
-    return kCounterBytes + (pl.BK > 1 ? (size_t)NL * pl.BK * 2 * (size_t)l->N * sizeof(float) : 0);
+    return kHeadBytes + (pl.BK > 1 ? (size_t)NL * pl.BK * 2 * (size_t)l->N * sizeof(float) : 0);
 }
 
 int run_job(const W3Job &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
@@ -460,7 +473,9 @@ int run_job(const W3Job &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
     }
     p.lper = j.lper > 0 ? j.lper : 1;
     p.counter = static_cast<int *>(ws);
-    p.part = pl.BK > 1 ? reinterpret_cast<float *>(static_cast<char *>(ws) + kCounterBytes) : nullptr;
+    p.part = pl.BK > 1 ? reinterpret_cast<float *>(static_cast<char *>(ws) + kHeadBytes) : nullptr;
+    if (pl.BK > 1 && pl.BK <= 8 && (size_t)j.NL * (size_t)l->N * 2 * sizeof(unsigned long long) <= kSlotBytes)
+        p.slots = reinterpret_cast<unsigned long long *>(static_cast<char *>(ws) + kCounterBytes);
     p.part_lstride = (int64_t)pl.BK * 2 * l->N;
     p.y_lstride = j.y_lstride;
     p.accumulate = j.ep.accumulate;
