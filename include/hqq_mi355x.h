@@ -96,11 +96,12 @@ int hqq_dequantize(const hqq_linear *l, void *w_out_f16, void *stream);
  *      triton_matmul3_transpose (src/triton_kernels.py:133-191, 321-380, 511-564) together with the meta expansion of
  *      forward_triton (src/custom_layers.py:55-92).  x is fp16 (M, K) contiguous, y is fp16 (M, N).  fp32 accumulation.
  *      `workspace` must hold hqq_matmul_workspace_bytes(l, M) bytes, 256-byte aligned.  It holds split-K partial sums
- *      and, in its first 64 KiB, per-tile arrival counters: call hqq_workspace_init once after allocating it (or
- *      zero-fill it); every call leaves the counters at zero again, so one workspace serves any sequence of calls
- *      that are ordered on a stream.  Calls that overlap in time need separate workspaces.                          */
+ *      and, in its first 576 KiB, per-tile arrival counters and per-output accumulation slots that must start at
+ *      zero: call hqq_workspace_init once after allocating it (or zero-fill it); every call leaves that head at zero
+ *      again, so one workspace serves any sequence of calls that are ordered on a stream.  Calls that overlap in
+ *      time need separate workspaces.                                                                               */
 size_t hqq_matmul_workspace_bytes(const hqq_linear *l, int64_t M);
-/* zero the counter head of a workspace with a small fill kernel (safe under stream capture)                          */
+/* zero the head (counters and slots) of a workspace with a small fill kernel (safe under stream capture)            */
 int hqq_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
 /* same, with the kernel family forced (-1 = automatic choice, else 0..3 as hqq_matmul_kernel_family reports):
  * HQQ_E_UNSUPPORTED when that family does not take the configuration.  For tests and profiling.                    */
