@@ -245,32 +245,49 @@ struct TileWeightRegs {
 // NFW: waves that share a packed table row, each taking F / NFW of its fields (1: a wave owns all fields; 2: the block
 // is eight waves, every weight is still rebuilt once, and a wave holds half the accumulators -- what lets two waves
 // share a SIMD at the 128-column batch tile).
-template <int NBITS, int BM, int SKIND, int ZKIND, int NFW>
-__global__ __launch_bounds__(kWaves * NFW * 64) void gemm_tile2_kernel(TileParams p)
+// JW packed table rows per block, KW parts of the block's K range worked on by different waves: at the narrowest
+// batch tile a block is one packed row and eight K parts, which meet in LDS, so that a projection with K = 4096
+// needs neither partial sums in memory nor a finishing launch.  G2 (with JW = 2): the two "rows" of the block are the
+// two projections of a gate for the same packed row; they share the x tile, and when the block holds all of K the
+// first projection's wave applies silu(a) * b itself.
+template <int NBITS, int BM, int SKIND, int ZKIND, int NFW, int JW = kWaves, int KW = 1, bool G2 = false>
+__global__ __launch_bounds__(JW * NFW * KW * 64) void gemm_tile2_kernel(TileParams p)
 {
+    static_assert(!G2 || (JW == 2 && NFW == 1 && KW > 1), "the gate form is two projections by several K parts");
     constexpr int F = 8 / NBITS;
     constexpr int FW = F / NFW;       // fields per wave
-    constexpr int NW = kWaves * NFW;  // waves per block
+    constexpr int NWK = JW * NFW;     // waves per K part
+    constexpr int NW = NWK * KW;      // waves per block
     constexpr int MB = BM / 16;
     constexpr int XP = BM + 2;
-    constexpr int XCH = (BM * 8 + NW * 64 - 1) / (NW * 64);
+    // With K parts every wave stages an x tile of its own and the steps of the loop need no block barrier: the
+    // waves of a block share nothing until their sums meet at the end.
+    constexpr bool PRIV = KW > 1;
+    constexpr int XT = PRIV ? 64 : NWK * 64; // threads that stage one x tile
+    constexpr int XCH = (BM * 8 + XT - 1) / XT;
     constexpr int TAB = FW * 2 * 4 * 8; // halves per wave and table: entry ((i*2 + h)*4 + kg) of 8 halves
-    __shared__ __attribute__((aligned(16))) f16 x_lds[2][8 * XP * 8];
+    __shared__ __attribute__((aligned(16))) f16 x_lds[2][PRIV ? NW : 1][8 * XP * 8];
     __shared__ __attribute__((aligned(16))) f16 s_lds[2][NW][TAB];
     __shared__ __attribute__((aligned(16))) f16 z_lds[2][NW][TAB];
+    __shared__ float red_lds[KW > 1 ? (KW - 1) * NWK : 1][KW > 1 ? FW * MB * 4 : 1][KW > 1 ? 64 : 1];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kpart = wave / NWK, wl = wave - kpart * NWK; // K part of the block, wave inside the part
+    const int tk = PRIV ? lane : (int)threadIdx.x;         // thread among those that stage its x tile
+    const int xi = PRIV ? wave : 0;                        // which x tile
     const int jall = blockIdx.x / p.KSP, ks = blockIdx.x - jall * p.KSP;
-    const bool second = jall >= p.JB; // block-uniform: the selections below are scalar
-    const int jblk = jall - (second ? p.JB : 0);
-    const int jp = jblk * kWaves + wave / NFW;
-    const int f0 = (wave % NFW) * FW; // first field of this wave
+    // second projection of a gate: a block of its own (block-uniform), or with G2 the block's odd waves
+    const bool second = G2 ? (wl & 1) != 0 : jall >= p.JB;
+    const int jblk = jall - (!G2 && second ? p.JB : 0);
+    const int jp = G2 ? jblk : jblk * JW + wl / NFW;
+    const int f0 = (wl % NFW) * FW; // first field of this wave
     const Table &sc_t = second ? p.sc_b : p.sc, &zr_t = second ? p.zr_b : p.zr;
     const uint32_t sc_inv = second ? p.sc_b_inv : p.sc_inv;
-    const int s_begin = ks * p.KTS;
-    const int s_end = s_begin + p.KTS < p.KT ? s_begin + p.KTS : p.KT;
-    const int s_last = s_end - 1;
+    const int s_begin = (ks * KW + kpart) * p.KTS; // KTS: steps per K part
+    const int s_stop = s_begin + p.KTS;            // the same trip count for every wave of the block
+    const int s_end = s_stop < p.KT ? s_stop : p.KT;
+    const int s_last = s_end > 0 ? s_end - 1 : 0;
     const int rb = blockIdx.y;
     const int m0 = blockIdx.z * BM;
     const int K = p.K;
@@ -296,7 +313,7 @@ __global__ __launch_bounds__(kWaves * NFW * 64) void gemm_tile2_kernel(TileParam
     int xdst[XCH];
 #pragma unroll
     for (int c = 0; c < XCH; ++c) {
-        const int ch = (int)threadIdx.x + c * NW * 64;
+        const int ch = tk + c * XT;
         const int chc = ch < BM * 8 ? ch : BM * 8 - 1;
         int m = m0 + chc / 8;
         m = m < p.M ? m : p.M - 1;
@@ -347,8 +364,8 @@ __global__ __launch_bounds__(kWaves * NFW * 64) void gemm_tile2_kernel(TileParam
             o.y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
             o.z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
             o.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
-            if (XCH * NW * 64 == BM * 8 || (int)threadIdx.x + c * NW * 64 < BM * 8)
-                *reinterpret_cast<u32x4 *>(&x_lds[buf][xdst[c]]) = o;
+            if (XCH * XT == BM * 8 || tk + c * XT < BM * 8)
+                *reinterpret_cast<u32x4 *>(&x_lds[buf][xi][xdst[c]]) = o;
         }
         if (tlane) {
             f16x2 s01, s23, z01, z23;
@@ -388,7 +405,7 @@ __global__ __launch_bounds__(kWaves * NFW * 64) void gemm_tile2_kernel(TileParam
             f16x8 B[MB];
 #pragma unroll
             for (int b = 0; b < MB; ++b)
-                B[b] = *reinterpret_cast<const f16x8 *>(&x_lds[buf][(((h * 4 + kg) * XP) + b * 16 + rr) * 8]);
+                B[b] = *reinterpret_cast<const f16x8 *>(&x_lds[buf][xi][(((h * 4 + kg) * XP) + b * 16 + rr) * 8]);
 #pragma unroll
             for (int i = 0; i < FW; ++i) {
                 const u32x4 S = *reinterpret_cast<const u32x4 *>(&s_lds[buf][wave][((i * 2 + h) * 4 + kg) * 8]);
@@ -427,7 +444,16 @@ __global__ __launch_bounds__(kWaves * NFW * 64) void gemm_tile2_kernel(TileParam
     u32x4 cw = T0.cw;
     issue_x(X0, s_begin + 2);
     issue(T0, s_begin + 4);
-    __syncthreads();
+    auto staged = [&]() __attribute__((always_inline)) { // what was staged is visible to those who read it
+        if constexpr (PRIV) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        } else {
+            __syncthreads();
+        }
+    };
+    staged();
     auto step = [&](Regs &Tn, XRegs &Xn, int buf, int s) __attribute__((always_inline)) {
         if (s < s_end)
             compute(cw, buf);
@@ -435,13 +461,66 @@ __global__ __launch_bounds__(kWaves * NFW * 64) void gemm_tile2_kernel(TileParam
         cw = Tn.cw;
         issue_x(Xn, s + 3);
         issue(Tn, s + 5);
-        __syncthreads();
+        staged();
     };
-    for (int s = s_begin; s < s_end; s += 4) {
+    for (int s = s_begin; s < (KW > 1 ? s_stop : s_end); s += 4) {
         step(T1, X1, 0, s);
         step(T2, X0, 1, s + 1);
         step(T3, X1, 0, s + 2);
         step(T0, X0, 1, s + 3);
+    }
+
+    if constexpr (KW > 1) {
+        // the K parts of the block meet in LDS: part 0 adds the others' sums in a fixed order and goes on alone
+        if (kpart > 0) {
+#pragma unroll
+            for (int i = 0; i < FW; ++i)
+#pragma unroll
+                for (int b = 0; b < MB; ++b)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        red_lds[(kpart - 1) * NWK + wl][(i * MB + b) * 4 + v][lane] = acc[i][b][v];
+        }
+        __syncthreads();
+        if (kpart > 0)
+            return;
+        for (int q = 0; q < KW - 1; ++q)
+#pragma unroll
+            for (int i = 0; i < FW; ++i)
+#pragma unroll
+                for (int b = 0; b < MB; ++b)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        acc[i][b][v] += red_lds[q * NWK + wl][(i * MB + b) * 4 + v][lane];
+        if constexpr (G2) {
+            if (!p.part) {
+                // Both projections are complete in this block.  The second one's wave hands its sums over through
+                // the LDS rows only it has read; the first one's wave rounds both to fp16, applies SiLU in fp32
+                // rounded once and multiplies in fp16 (the reference's three ops, src/custom_layers.py:253-256).
+                if (second) {
+#pragma unroll
+                    for (int i = 0; i < FW; ++i)
+#pragma unroll
+                        for (int b = 0; b < MB; ++b)
+#pragma unroll
+                            for (int v = 0; v < 4; ++v)
+                                red_lds[1][(i * MB + b) * 4 + v][lane] = acc[i][b][v];
+                }
+                __syncthreads(); // the two waves that are left
+                if (second)
+                    return;
+#pragma unroll
+                for (int i = 0; i < FW; ++i)
+#pragma unroll
+                    for (int b = 0; b < MB; ++b)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            const float u = (float)(f16)acc[i][b][v];
+                            const f16 h = (f16)(u / (1.0f + __expf(-u))) * (f16)red_lds[1][(i * MB + b) * 4 + v][lane];
+                            acc[i][b][v] = (float)h; // exact: the store below rounds an fp16 value to fp16
+                        }
+            }
+        }
     }
 
     // D layout: column = batch column (lane & 15) of block b, rows r = 4*(lane>>4) + v
@@ -580,6 +659,7 @@ size_t rewrite_bytes(const hqq_linear *l)
 
 struct TilePlan {
     int F, GP, RB, KT, BM, KSP, KTS;
+    int JW, KW; // packed table rows per block, K parts per block
     int kinds; // 1: 8-bit tables as HQQ writes them, 3: fp16 tables (both run the pipelined kernel), 0: anything else
 };
 
@@ -626,6 +706,24 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl, int nl = 1)
     const int64_t mtiles = (M + pl.BM - 1) / pl.BM;
     if (mtiles > 65535)
         return false;
+    pl.JW = kWaves, pl.KW = 1;
+    if (pl.BM == 16 && pl.kinds != 0 && !(tuning_overrides() && std::getenv("HQQ_TILE_KW1"))) {
+        // the narrowest batch tile: a block is one packed row, its eight waves split the block's K range.  Blocks
+        // along K only until the chip is covered, with at least four steps (256 columns) per wave.
+        pl.JW = nl == 2 ? 2 : 1, pl.KW = nl == 2 ? 4 : 8; // a gate: both projections of a packed row in one block
+        const int64_t rows = (int64_t)pl.GP * pl.RB * mtiles;
+        int64_t kb = (224 + rows - 1) / rows;
+        if (kb > pl.KT / (4 * pl.KW))
+            kb = pl.KT / (4 * pl.KW);
+        if (kb < 1)
+            kb = 1;
+        if (tuning_overrides())
+            if (const char *e = std::getenv("HQQ_TILE_KSP"))
+                kb = std::atoi(e);
+        pl.KTS = (int)((pl.KT + kb * pl.KW - 1) / (kb * pl.KW));
+        pl.KSP = (pl.KT + pl.KTS * pl.KW - 1) / (pl.KTS * pl.KW);
+        return (int64_t)pl.GP * pl.KSP <= 0x7fffffff;
+    }
     // K is split over blocks until every SIMD has a wave (two for batches up to 128 rows, whose partial sums are
     // small), with at least eight steps per block.  Measured at Mixtral shapes: a split beyond that, which leaves
     // waves over for a partly filled round, costs 20-40 %.
@@ -652,6 +750,22 @@ template <int NBITS, int BM> void launch_tile2_kinds(const TileParams &p, const 
 {
     // the widest batch tile runs with two waves per packed table row (half the accumulators each)
     constexpr int NFW = BM == 128 ? 2 : 1;
+    if constexpr (BM == 16) {
+        if (pl.KW == 8) {
+            if (pl.kinds == 1)
+                gemm_tile2_kernel<NBITS, BM, TK_U8_COLS, TK_U8_SCALAR, 1, 1, 8><<<grid, 8 * 64, 0, s>>>(p);
+            else
+                gemm_tile2_kernel<NBITS, BM, TK_F16, TK_F16, 1, 1, 8><<<grid, 8 * 64, 0, s>>>(p);
+            return;
+        }
+        if (pl.KW == 4) {
+            if (pl.kinds == 1)
+                gemm_tile2_kernel<NBITS, BM, TK_U8_COLS, TK_U8_SCALAR, 1, 2, 4, true><<<grid, 8 * 64, 0, s>>>(p);
+            else
+                gemm_tile2_kernel<NBITS, BM, TK_F16, TK_F16, 1, 2, 4, true><<<grid, 8 * 64, 0, s>>>(p);
+            return;
+        }
+    }
     if (pl.kinds == 1)
         gemm_tile2_kernel<NBITS, BM, TK_U8_COLS, TK_U8_SCALAR, NFW><<<grid, kWaves * NFW * 64, 0, s>>>(p);
     else
@@ -697,7 +811,7 @@ static size_t tile_job_bytes(const hqq_linear *l, int64_t M, int nl)
     const hqq_linear v = tile_view(l);
     if (!make_plan(&v, M, pl, nl))
         return 0;
-    const bool partial = pl.KSP > 1 || nl == 2;
+    const bool partial = pl.KSP > 1 || (nl == 2 && pl.KW == 1);
     const size_t one = partial ? (((size_t)pl.KSP * (size_t)M * (size_t)l->N * sizeof(float) + 255) & ~(size_t)255) : 0;
     const size_t body = nl * (one + rewrite_bytes(l));
     return body ? workspace_head_bytes() + body : 0;
@@ -717,7 +831,7 @@ static int tile_job(const hqq_linear *la, const hqq_linear *lb, const f16 *x, in
     const size_t need = tile_job_bytes(la, M, nl);
     if (need > 0 && (!ws || ws_bytes < need))
         return HQQ_E_WORKSPACE;
-    const bool partial = pl.KSP > 1 || nl == 2;
+    const bool partial = pl.KSP > 1 || (nl == 2 && pl.KW == 1);
     const size_t one = partial ? (((size_t)pl.KSP * (size_t)M * (size_t)la->N * sizeof(float) + 255) & ~(size_t)255) : 0;
     char *body = static_cast<char *>(ws) + workspace_head_bytes();
     if (la->nbits == 3) {
@@ -739,13 +853,15 @@ static int tile_job(const hqq_linear *la, const hqq_linear *lb, const f16 *x, in
     p.codes_b = static_cast<const uint8_t *>(view[1].codes);
     p.sc_b = make_table(view[1].scale), p.zr_b = make_table(view[1].zero);
     p.sc_b_inv = view[1].scale.meta_cols > 0 ? (uint32_t)(0xFFFFFFFFull / (uint64_t)view[1].scale.meta_cols) : 0;
-    p.JB = pl.GP / kWaves;
+    p.JB = pl.GP / pl.JW;
     p.part_lstride = (int64_t)(one / sizeof(float));
     p.x = x, p.bias = nl == 1 ? static_cast<const f16 *>(l->bias) : nullptr, p.y = y;
     p.M = (int)M, p.N = (int)l->N, p.K = (int)l->K, p.GP = pl.GP, p.KT = pl.KT;
     p.KSP = pl.KSP, p.KTS = pl.KTS;
     p.part = partial ? reinterpret_cast<float *>(body) : nullptr;
-    const dim3 grid((unsigned)(pl.GP / kWaves * pl.KSP * nl), (unsigned)pl.RB, (unsigned)((M + pl.BM - 1) / pl.BM));
+    // blocks along x: packed rows (per projection, unless a block holds both) by K blocks
+    const int jrows = pl.KW == 4 ? pl.GP : pl.GP / pl.JW * nl;
+    const dim3 grid((unsigned)(jrows * pl.KSP), (unsigned)pl.RB, (unsigned)((M + pl.BM - 1) / pl.BM));
     if (pl.kinds != 0) {
         launch_tile2(p, pl, l->nbits, grid, s);
     } else if (l->nbits == 2) {
