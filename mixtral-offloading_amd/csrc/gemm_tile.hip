@@ -707,7 +707,7 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl, int nl = 1)
     if (mtiles > 65535)
         return false;
     pl.JW = kWaves, pl.KW = 1;
-    if (pl.BM == 16 && pl.kinds != 0 && !(tuning_overrides() && std::getenv("HQQ_TILE_KW1"))) {
+    if (pl.BM <= 32 && pl.kinds != 0 && !(tuning_overrides() && std::getenv("HQQ_TILE_KW1"))) {
         // the narrowest batch tile: a block is one packed row, its eight waves split the block's K range.  Blocks
         // along K only until the chip is covered, with at least four steps (256 columns) per wave.
         pl.JW = nl == 2 ? 2 : 1, pl.KW = nl == 2 ? 4 : 8; // a gate: both projections of a packed row in one block
@@ -750,7 +750,7 @@ template <int NBITS, int BM> void launch_tile2_kinds(const TileParams &p, const 
 {
     // the widest batch tile runs with two waves per packed table row (half the accumulators each)
     constexpr int NFW = BM == 128 ? 2 : 1;
-    if constexpr (BM == 16) {
+    if constexpr (BM <= 32) {
         if (pl.KW == 8) {
             if (pl.kinds == 1)
                 gemm_tile2_kernel<NBITS, BM, TK_U8_COLS, TK_U8_SCALAR, 1, 1, 8><<<grid, 8 * 64, 0, s>>>(p);
