@@ -269,7 +269,10 @@ __global__ __launch_bounds__(JW * NFW * KW * 64) void gemm_tile2_kernel(TilePara
     __shared__ __attribute__((aligned(16))) f16 x_lds[2][PRIV ? NW : 1][8 * XP * 8];
     __shared__ __attribute__((aligned(16))) f16 s_lds[2][NW][TAB];
     __shared__ __attribute__((aligned(16))) f16 z_lds[2][NW][TAB];
-    __shared__ float red_lds[KW > 1 ? (KW - 1) * NWK : 1][KW > 1 ? FW * MB * 4 : 1][KW > 1 ? 64 : 1];
+    // where the K parts' sums meet after the loop: the memory of the x tiles, which are no longer needed then
+    constexpr int RED_ROWS = FW * MB * 4;
+    static_assert(!PRIV || sizeof(float) * (KW - 1) * NWK * RED_ROWS * 64 <= sizeof(x_lds), "the sums fit the x tiles");
+    float(*red_lds)[RED_ROWS][64] = reinterpret_cast<float(*)[RED_ROWS][64]>(&x_lds[0][0][0]);
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -472,6 +475,7 @@ __global__ __launch_bounds__(JW * NFW * KW * 64) void gemm_tile2_kernel(TilePara
 
     if constexpr (KW > 1) {
         // the K parts of the block meet in LDS: part 0 adds the others' sums in a fixed order and goes on alone
+        __syncthreads(); // every wave is through with its x tiles
         if (kpart > 0) {
 #pragma unroll
             for (int i = 0; i < FW; ++i)
@@ -710,7 +714,9 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl, int nl = 1)
     if (pl.BM <= 32 && pl.kinds != 0 && !(tuning_overrides() && std::getenv("HQQ_TILE_KW1"))) {
         // the narrowest batch tile: a block is one packed row, its eight waves split the block's K range.  Blocks
         // along K only until the chip is covered, with at least four steps (256 columns) per wave.
-        pl.JW = nl == 2 ? 2 : 1, pl.KW = nl == 2 ? 4 : 8; // a gate: both projections of a packed row in one block
+        pl.JW = nl == 2 ? 2 : 1, pl.KW = 8; // a gate: both projections of a packed row in one block of sixteen waves
+        if (nl == 2 && pl.BM == 32)
+            pl.KW = 4; // the wider tile needs more registers than sixteen waves leave each
         const int64_t rows = (int64_t)pl.GP * pl.RB * mtiles;
         int64_t kb = (224 + rows - 1) / rows;
         if (kb > pl.KT / (4 * pl.KW))
@@ -751,6 +757,15 @@ template <int NBITS, int BM> void launch_tile2_kinds(const TileParams &p, const 
     // the widest batch tile runs with two waves per packed table row (half the accumulators each)
     constexpr int NFW = BM == 128 ? 2 : 1;
     if constexpr (BM <= 32) {
+        if constexpr (BM == 16) {
+            if (pl.KW == 8 && pl.JW == 2) {
+                if (pl.kinds == 1)
+                    gemm_tile2_kernel<NBITS, BM, TK_U8_COLS, TK_U8_SCALAR, 1, 2, 8, true><<<grid, 16 * 64, 0, s>>>(p);
+                else
+                    gemm_tile2_kernel<NBITS, BM, TK_F16, TK_F16, 1, 2, 8, true><<<grid, 16 * 64, 0, s>>>(p);
+                return;
+            }
+        }
         if (pl.KW == 8) {
             if (pl.kinds == 1)
                 gemm_tile2_kernel<NBITS, BM, TK_U8_COLS, TK_U8_SCALAR, 1, 1, 8><<<grid, 8 * 64, 0, s>>>(p);
@@ -860,7 +875,7 @@ static int tile_job(const hqq_linear *la, const hqq_linear *lb, const f16 *x, in
     p.KSP = pl.KSP, p.KTS = pl.KTS;
     p.part = partial ? reinterpret_cast<float *>(body) : nullptr;
     // blocks along x: packed rows (per projection, unless a block holds both) by K blocks
-    const int jrows = pl.KW == 4 ? pl.GP : pl.GP / pl.JW * nl;
+    const int jrows = pl.JW == 2 ? pl.GP : pl.GP / pl.JW * nl;
     const dim3 grid((unsigned)(jrows * pl.KSP), (unsigned)pl.RB, (unsigned)((M + pl.BM - 1) / pl.BM));
     if (pl.kinds != 0) {
         launch_tile2(p, pl, l->nbits, grid, s);
