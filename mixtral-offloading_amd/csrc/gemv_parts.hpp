@@ -23,7 +23,8 @@ constexpr int kSlotFracBits = 34;
 constexpr float kSlotLimit = 131071.0f;
 __device__ __forceinline__ unsigned long long slot_term(float v)
 {
-    v = v < -kSlotLimit ? -kSlotLimit : (v > kSlotLimit ? kSlotLimit : v); // NaN passes and converts to 0
+    // beyond the fp16 range the output is infinite either way; a NaN takes the same way out (it cannot be added)
+    v = v >= -kSlotLimit ? (v <= kSlotLimit ? v : kSlotLimit) : (v < -kSlotLimit ? -kSlotLimit : kSlotLimit);
     const long long fx = (long long)__builtin_rintf(v * (float)(1ull << kSlotFracBits)); // exact scaling by 2^34
     return (1ull << 56) + (unsigned long long)fx;
 }

@@ -172,3 +172,24 @@ def test_full_size_against_dequantize_then_matmul(nbits, n, k, gs, m):
     # that hold scale*x in fp16 may differ by an fp16 rounding of a few tiny terms)
     y2 = hip_kernels.matmul(desc, (x * 2).contiguous())
     assert bool(((y2.float() - 2 * y.float()).abs() <= 2.0 ** -9 * (2 * y.float()).abs() + 1e-2 * atol).all())
+
+
+def test_workspace_head_is_left_at_zero():
+    """Launches that split K meet in the head of the workspace (arrival counters, accumulation slots), which they
+    must leave at zero: the next call, of any kernel family, starts from it."""
+    from mixtral_offloading_amd import hip_kernels
+    rng = np.random.default_rng(99)
+    dev = torch.device("cuda:0")
+    cases = [(2, 256, 8192, 16), (4, 128, 6144, 64), (3, 640, 4096, 64), (2, 512, 1024, 16)]
+    for nbits, n, k, gs in cases:
+        layer, _ = o.random_layer(rng, n, k, nbits, gs)
+        d = desc_of(layer)
+        for m in (1, 2, 4, 8, 40):
+            x = rng.standard_normal((m, k)).astype(np.float16)
+            ref = o.matmul_transpose(x, layer)
+            for rep in range(2):
+                y = hip_kernels.matmul(d, to_dev(x)).cpu().numpy()
+                assert_matmul_close(y, ref, o.matmul_tolerance(x, layer))
+    torch.cuda.synchronize()
+    head = hip_kernels.workspace(dev, 1)[: 576 * 1024]
+    assert head.numel() == 576 * 1024 and not bool(head.any())
