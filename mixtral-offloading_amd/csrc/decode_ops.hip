@@ -197,23 +197,40 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restr
     }
     __syncthreads();
 
-    // scores: one position per thread, the key row read as 16-byte pieces, q broadcast from LDS
+    // scores: LPK threads share a key row (16 bytes each, so a wave's load covers whole rows), four passes of
+    // KROWS rows in flight; the pieces of a dot product meet through lane exchanges
     const float inv = 1.0f / __builtin_sqrtf((float)HD);
     float mx = -3.0e38f;
-    for (int64_t l = tid; l <= pos; l += NT) {
-        const f16 *krow = l == pos ? k_lds : cache_k + ((int64_t)kv * max_len + l) * HD;
-        float acc = 0.f;
+    {
+        constexpr int LPK = HD / 8, KROWS = NT / LPK;
+        const int ksub = tid / LPK, kc = tid % LPK;
+        const f16x8 qq = *reinterpret_cast<const f16x8 *>(q_lds + 8 * kc);
+        for (int64_t l0 = 0; l0 <= pos; l0 += 4 * KROWS) {
+            f16x8 kk[4];
 #pragma unroll
-        for (int c = 0; c < HD / 8; ++c) {
-            const f16x8 kk = *reinterpret_cast<const f16x8 *>(krow + 8 * c);
-            const f16x8 qq = *reinterpret_cast<const f16x8 *>(q_lds + 8 * c);
+            for (int u = 0; u < 4; ++u) {
+                const int64_t l = l0 + u * KROWS + ksub;
+                const int64_t lc = l <= pos ? l : pos;
+                const f16 *krow = lc == pos ? k_lds : cache_k + ((int64_t)kv * max_len + lc) * HD;
+                kk[u] = *reinterpret_cast<const f16x8 *>(krow + 8 * kc);
+            }
 #pragma unroll
-            for (int t = 0; t < 8; ++t)
-                acc += (float)kk[t] * (float)qq[t];
+            for (int u = 0; u < 4; ++u) {
+                float acc = 0.f;
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    acc += (float)kk[u][t] * (float)qq[t];
+#pragma unroll
+                for (int off = LPK / 2; off > 0; off >>= 1)
+                    acc += __shfl_xor(acc, off, 64);
+                const int64_t l = l0 + u * KROWS + ksub;
+                if (kc == 0 && l <= pos) {
+                    const float sc = (float)(f16)acc * inv;
+                    score_lds[l] = sc;
+                    mx = fmaxf(mx, sc);
+                }
+            }
         }
-        const float sc = (float)(f16)acc * inv;
-        score_lds[l] = sc;
-        mx = fmaxf(mx, sc);
     }
     // block max
 #pragma unroll
