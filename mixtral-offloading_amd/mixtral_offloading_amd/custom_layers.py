@@ -235,6 +235,21 @@ class SparseMoeWrapper(nn.Module):
         self.experts = expert_cache
 
     @torch.inference_mode()
+    def forward_routed(self, hidden_states: torch.Tensor, selected: torch.Tensor, weights: torch.Tensor,
+                       out: torch.Tensor) -> torch.Tensor:
+        """One token whose router has already run on the device (``hip_kernels.add_rmsnorm_router``): ``selected``
+        int32[2] and ``weights`` fp16[2] are device tensors.  The host reads the choice (the one synchronisation of the
+        layer, as the cache is driven from the host), loads what is missing and runs the experts into ``out``."""
+        chosen = selected.cpu().tolist()
+        first = True
+        for (_layer_index, expert_idx), expert_layer in self.experts.load_experts(
+                *((self.layer_id, expert_idx) for expert_idx in sorted(set(chosen))), unordered=True):
+            k = chosen.index(expert_idx)
+            expert_layer(hidden_states, out=out, row_scale=weights[k:k + 1], accumulate=not first)
+            first = False
+        return out
+
+    @torch.inference_mode()
     def forward(self, hidden_states: torch.Tensor):
         batch_size, sequence_length, hidden_dim = hidden_states.shape
         hidden_states = hidden_states.reshape(-1, hidden_dim)

@@ -264,9 +264,70 @@ class MixtralForCausalLM(nn.Module):
         return [(torch.zeros((cfg.num_key_value_heads, L, hd), **mk), torch.zeros((cfg.num_key_value_heads, L, hd), **mk))
                 for _ in range(cfg.num_hidden_layers)]
 
+    def _token_state(self):
+        """Buffers and grouped projections of the single-token step, made once."""
+        st = getattr(self, "_token_bufs", None)
+        if st is None:
+            from . import hip_kernels
+
+            cfg, mk = self.config, dict(device=self.device)
+            row = lambda n: torch.zeros((1, n), dtype=torch.float16, **mk)  # noqa: E731
+            st = dict(x=row(cfg.hidden_size), x2=row(cfg.hidden_size), xn=row(cfg.hidden_size), moe=row(cfg.hidden_size),
+                      att=row(cfg.hidden_size), sel=torch.zeros(2, dtype=torch.int32, **mk),
+                      rw=torch.zeros(2, dtype=torch.float16, **mk), pos=torch.zeros(1, dtype=torch.int64, **mk),
+                      qkv=[hip_kernels.LinearGroup([p._desc() for p in (l.self_attn.q_proj, l.self_attn.k_proj, l.self_attn.v_proj)])
+                           for l in self.model.layers])
+            self._token_bufs = st
+        return st
+
+    @torch.inference_mode()
+    def forward_token(self, token: torch.Tensor, cache, start: int) -> torch.Tensor:
+        """One new token through the launches of the graph step (grouped q/k/v with the norm folded in, the attention
+        kernel, norm + router in one launch, the fused expert FFN), but with the experts picked up from the expert cache
+        by the host: one synchronisation per layer, which is what lets experts be offloaded.  Returns logits (1, vocab)."""
+        from . import hip_kernels
+
+        cfg, st = self.config, self._token_state()
+        if cfg.num_experts_per_tok != 2 or not (0 <= start < min(cache[0][0].shape[1], self.rotary.cos.shape[0])):
+            raise ValueError("the single-token step takes top-2 routing and a position inside the cache")
+        eps = cfg.rms_norm_eps
+        x, spare, xn, moe = st["x"], st["x2"], st["xn"], st["moe"]
+        st["pos"].fill_(start)
+        x.copy_(self.model.embed_tokens(token.view(1)))
+        delta = None
+        for layer, (ck, cv), qkv in zip(self.model.layers, cache, st["qkv"]):
+            attn = layer.self_attn
+            if qkv.supported:
+                q, k, v = hip_kernels.matmul_group_norm(qkv, x, delta, layer.input_layernorm.weight, eps, spare)
+                x, spare = spare, x
+            else:
+                hip_kernels.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps, xn)
+                q, k, v = attn.q_proj(xn), attn.k_proj(xn), attn.v_proj(xn)
+            out = hip_kernels.attention_decode(q, k, v, self.rotary.cos, self.rotary.sin, st["pos"], ck, cv, st["att"])
+            hip_kernels.add_rmsnorm_router(x, attn.o_proj(out), layer.post_attention_layernorm.weight, eps, xn,
+                                           layer.block_sparse_moe.gate.weight, st["sel"], st["rw"])
+            layer.block_sparse_moe.forward_routed(xn, st["sel"], st["rw"], moe)
+            delta = moe
+        hip_kernels.add_rmsnorm(x, delta, self.model.norm.weight, eps, xn)
+        return self.lm_head(xn)
+
+    def _token_step_ok(self, cache) -> bool:
+        cfg = self.config
+        hd = cfg.hidden_size // cfg.num_attention_heads
+        return (cfg.num_experts_per_tok == 2 and 2 <= cfg.num_local_experts <= 16 and hd in (64, 128)
+                and cfg.hidden_size % 8 == 0 and hasattr(self.model.layers[0].block_sparse_moe, "forward_routed")
+                and cache[0][0].is_contiguous() and cache[0][0].shape[1] <= 16000)
+
     @torch.inference_mode()
     def forward(self, input_ids: torch.Tensor, cache, start: int) -> torch.Tensor:
         """input_ids (T,), one sequence; returns logits (T, vocab)."""
+        if input_ids.numel() == 1 and self._token_step_ok(cache):
+            return self.forward_token(input_ids, cache, start)
+        return self.forward_tokens(input_ids, cache, start)
+
+    @torch.inference_mode()
+    def forward_tokens(self, input_ids: torch.Tensor, cache, start: int) -> torch.Tensor:
+        """Any number of tokens of one sequence, layer by layer with torch ops around the quantized linears."""
         x = self.model.embed_tokens(input_ids)
         for layer, (ck, cv) in zip(self.model.layers, cache):
             x = layer(x, self.rotary, ck, cv, start)

@@ -206,3 +206,26 @@ def test_checkpoint_round_trip(tmp_path, layout, ffn_bits, ffn_group):
     prompt = torch.randint(0, cfg.vocab_size, (7,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(1))
     assert torch.equal(model.generate(prompt, 6), again.generate(prompt, 6))
     assert torch.equal(model.forward(prompt, model.new_cache(16), 0), again.forward(prompt, again.new_cache(16), 0))
+
+
+@pytest.mark.parametrize("offload_per_layer", [0, 6])
+def test_single_token_step_equals_the_layerwise_forward(offload_per_layer):
+    """``forward`` of one token takes the fused launches of the decode step (experts still fetched through the cache
+    by the host); it must give what the layer-by-layer path gives for the same token and cache."""
+    model, cfg = _small_setup(layers=2, offload_per_layer=offload_per_layer, main_per_layer=8 - offload_per_layer, seed=4)
+    g = torch.Generator(device="cuda").manual_seed(8)
+    prompt = torch.randint(0, cfg.vocab_size, (11,), device="cuda", generator=g)
+    cache_a, cache_b = model.new_cache(32), model.new_cache(32)
+    model.forward(prompt, cache_a, 0)
+    model.forward(prompt, cache_b, 0)
+    tok = torch.randint(0, cfg.vocab_size, (1,), device="cuda", generator=g)
+    for pos in range(11, 17):
+        fused = model.forward_token(tok, cache_a, pos).float()
+        plain = model.forward_tokens(tok, cache_b, pos).float()
+        assert fused.shape == plain.shape == (1, cfg.vocab_size)
+        assert float((fused - plain).abs().max()) <= 2e-2 * float(plain.abs().max()) + 1e-3
+        tok = plain[-1].argmax().view(1)
+    for (ka, va), (kb, vb) in zip(cache_a, cache_b):  # both paths appended the same keys and values
+        assert float((ka.float() - kb.float()).abs().max()) <= 2e-2 and float((va.float() - vb.float()).abs().max()) <= 2e-2
+    with pytest.raises(ValueError):
+        model.forward_token(tok, cache_a, 32)  # past the cache
