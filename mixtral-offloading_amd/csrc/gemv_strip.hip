@@ -746,7 +746,8 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl, int64_t ti
     } else {
         // One slab per wave unless a block that holds all of K would then need more than eight waves; K is split over
         // several blocks only when a single block cannot hold it or there would be too few blocks to cover the chip.
-        if (KS * NL > max_waves && (pl.NS + 1) / 2 * NL <= max_waves) {
+        // (two-layer blocks always take two slabs per wave: half the blocks along K, half the partial sums)
+        if (KS * NL > max_waves && ((pl.NS + 1) / 2 * NL <= max_waves || (NL == 2 && pl.NS >= 2))) {
             S = 2;
             KS = (pl.NS + 1) / 2;
         }
