@@ -295,8 +295,11 @@ class MixtralForCausalLM(nn.Module):
         st["pos"].fill_(start)
         x.copy_(self.model.embed_tokens(token.view(1)))
         delta = None
-        for layer, (ck, cv), qkv in zip(self.model.layers, cache, st["qkv"]):
+        for i, (layer, (ck, cv)) in enumerate(zip(self.model.layers, cache)):
             attn = layer.self_attn
+            qkv = st["qkv"][i]
+            if qkv.descs[0] is not attn.q_proj._desc():  # the layer's tensors were replaced since the group was made
+                qkv = st["qkv"][i] = hip_kernels.LinearGroup([p._desc() for p in (attn.q_proj, attn.k_proj, attn.v_proj)])
             if qkv.supported:
                 q, k, v = hip_kernels.matmul_group_norm(qkv, x, delta, layer.input_layernorm.weight, eps, spare)
                 x, spare = spare, x
