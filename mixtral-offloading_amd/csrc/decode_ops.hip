@@ -177,14 +177,16 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restr
     __shared__ float acc_lds[NT / (HD / 8)][HD];
     const int h = blockIdx.x, kv = h / group;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // the new token's q, k and v do not depend on the position: their loads go out before it is waited for
+    const int d = tid < HD ? tid : 0, dr = d < HD / 2 ? d + HD / 2 : d - HD / 2;
+    const f16 qa = q_in[h * HD + d], qb = q_in[h * HD + dr];
+    const f16 ka = k_in[kv * HD + d], kb = k_in[kv * HD + dr];
+    const f16 vnew = v_in[kv * HD + d];
     const int64_t pos = pos_p[0];
     if (pos < 0 || pos >= max_len) // the position lives in device memory: a step past the cache must not write past it
         return;
     const f16 *cs = cos_t + pos * HD, *sn = sin_t + pos * HD;
     if (tid < HD) {
-        const int d = tid, o = d < HD / 2 ? d + HD / 2 : d - HD / 2;
-        const f16 qa = q_in[h * HD + d], qb = q_in[h * HD + o];
-        const f16 ka = k_in[kv * HD + d], kb = k_in[kv * HD + o];
         const f16 qr = d < HD / 2 ? -qb : qb, kr = d < HD / 2 ? -kb : kb;
         const f16 qrot = (f16)(qa * cs[d]) + (f16)(qr * sn[d]);
         const f16 krot = (f16)(ka * cs[d]) + (f16)(kr * sn[d]);
@@ -192,7 +194,7 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restr
         k_lds[d] = krot;
         if (h % group == 0) {
             cache_k[((int64_t)kv * max_len + pos) * HD + d] = krot;
-            cache_v[((int64_t)kv * max_len + pos) * HD + d] = v_in[kv * HD + d];
+            cache_v[((int64_t)kv * max_len + pos) * HD + d] = vnew;
         }
     }
     __syncthreads();
@@ -232,6 +234,17 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restr
             }
         }
     }
+    // the value rows of the first four passes do not depend on the scores: requested now, used after the softmax
+    constexpr int LPR = HD / 8, ROWS = NT / LPR;
+    const int rsub = tid / LPR, c8 = tid % LPR;
+    f16x8 vfirst[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t l = u * ROWS + rsub;
+        const int64_t lc = l <= pos ? l : pos;
+        const f16 *vrow = lc == pos ? v_in + kv * HD : cache_v + ((int64_t)kv * max_len + lc) * HD;
+        vfirst[u] = *reinterpret_cast<const f16x8 *>(vrow + 8 * c8);
+    }
     // block max
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1)
@@ -261,8 +274,6 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restr
 
     // output: LPR threads share a value row (16 bytes each), the block covers ROWS rows per pass and four passes
     // are in flight; the ROWS partial outputs meet in LDS
-    constexpr int LPR = HD / 8, ROWS = NT / LPR;
-    const int rsub = tid / LPR, c8 = tid % LPR;
     float o[8];
 #pragma unroll
     for (int t = 0; t < 8; ++t)
@@ -274,8 +285,12 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restr
         for (int u = 0; u < 4; ++u) {
             const int64_t l = l0 + u * ROWS + rsub;
             const int64_t lc = l <= pos ? l : pos;
-            const f16 *vrow = lc == pos ? v_in + kv * HD : cache_v + ((int64_t)kv * max_len + lc) * HD;
-            vv[u] = *reinterpret_cast<const f16x8 *>(vrow + 8 * c8);
+            if (l0 == 0) {
+                vv[u] = vfirst[u];
+            } else {
+                const f16 *vrow = lc == pos ? v_in + kv * HD : cache_v + ((int64_t)kv * max_len + lc) * HD;
+                vv[u] = *reinterpret_cast<const f16x8 *>(vrow + 8 * c8);
+            }
             pr[u] = l <= pos ? (float)(f16)(score_lds[lc] * rs) : 0.f;
         }
 #pragma unroll
