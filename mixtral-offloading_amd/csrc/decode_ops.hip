@@ -186,6 +186,17 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restr
     if (pos < 0 || pos >= max_len) // the position lives in device memory: a step past the cache must not write past it
         return;
     const f16 *cs = cos_t + pos * HD, *sn = sin_t + pos * HD;
+    // the cached key rows of the first four passes only need the position: requested before the rope table arrives
+    // (the row of the new token itself is taken from LDS later)
+    constexpr int LPK = HD / 8, KROWS = NT / LPK;
+    const int ksub = tid / LPK, kc = tid % LPK;
+    f16x8 kfirst[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t l = u * KROWS + ksub;
+        const int64_t lc = l <= pos ? l : pos;
+        kfirst[u] = *reinterpret_cast<const f16x8 *>(cache_k + ((int64_t)kv * max_len + lc) * HD + 8 * kc);
+    }
     if (tid < HD) {
         const f16 qr = d < HD / 2 ? -qb : qb, kr = d < HD / 2 ? -kb : kb;
         const f16 qrot = (f16)(qa * cs[d]) + (f16)(qr * sn[d]);
@@ -204,8 +215,6 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restr
     const float inv = 1.0f / __builtin_sqrtf((float)HD);
     float mx = -3.0e38f;
     {
-        constexpr int LPK = HD / 8, KROWS = NT / LPK;
-        const int ksub = tid / LPK, kc = tid % LPK;
         const f16x8 qq = *reinterpret_cast<const f16x8 *>(q_lds + 8 * kc);
         for (int64_t l0 = 0; l0 <= pos; l0 += 4 * KROWS) {
             f16x8 kk[4];
@@ -213,8 +222,12 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restr
             for (int u = 0; u < 4; ++u) {
                 const int64_t l = l0 + u * KROWS + ksub;
                 const int64_t lc = l <= pos ? l : pos;
-                const f16 *krow = lc == pos ? k_lds : cache_k + ((int64_t)kv * max_len + lc) * HD;
-                kk[u] = *reinterpret_cast<const f16x8 *>(krow + 8 * kc);
+                if (lc == pos)
+                    kk[u] = *reinterpret_cast<const f16x8 *>(k_lds + 8 * kc);
+                else if (l0 == 0)
+                    kk[u] = kfirst[u];
+                else
+                    kk[u] = *reinterpret_cast<const f16x8 *>(cache_k + ((int64_t)kv * max_len + lc) * HD + 8 * kc);
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
