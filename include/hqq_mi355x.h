@@ -119,8 +119,12 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
                    void *y_f16, const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
                    void *stream);
 
-/* ---- h = silu(w1 x) * (w3 x), fp16 (M, ffn): the first half of the expert FFN as one fused pass over both weight
- *      matrices (src/custom_layers.py:254).  Workspace: 2 * hqq_matmul_workspace_bytes(w1, M).                        */
+/* ---- h = silu(w1 x) * (w3 x), fp16 (M, ffn): the first half of the expert FFN (src/custom_layers.py:254), both
+ *      projections rounded to fp16 as the reference's two layers round them, SiLU in fp32 rounded once, the product in
+ *      fp16.  One fused pass over both weight matrices where a kernel family has one for the batch (2- and 4-bit
+ *      layers of one kind), else both projections followed by an elementwise pass.  Layers without bias.
+ *      Workspace: hqq_gate_up_workspace_bytes(w1, w3, M), 256-byte aligned, head zeroed as for hqq_matmul_transpose.  */
+size_t hqq_gate_up_workspace_bytes(const hqq_linear *w1, const hqq_linear *w3, int64_t M);
 int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, int64_t M, void *h_f16, void *workspace,
                 size_t workspace_bytes, void *stream);
 

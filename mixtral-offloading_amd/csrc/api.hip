@@ -216,6 +216,25 @@ size_t hqq_expert_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2
     return ffn_matmul_scratch(w1, w2, w3, M) + 3 * align256((size_t)M * w1->N * 2) + align256((size_t)M * w2->N * 2);
 }
 
+// workspace of the gate: [matmul scratch, counters first][a, b: M x N fp16 each (unfused paths only)]
+static size_t gate_matmul_scratch(const hqq_linear *w1, const hqq_linear *w3, int64_t M)
+{
+    size_t mm = hqq_matmul_workspace_bytes(w1, M); // already sized for the fused decode pass over two layers
+    const size_t m3 = hqq_matmul_workspace_bytes(w3, M), g = tile_gate_workspace_bytes(w1, w3, M);
+    mm = m3 > mm ? m3 : mm;
+    mm = g > mm ? g : mm;
+    const size_t v = vec3_gate_workspace_bytes(w1, M);
+    mm = v > mm ? v : mm;
+    return align256(mm);
+}
+
+size_t hqq_gate_up_workspace_bytes(const hqq_linear *w1, const hqq_linear *w3, int64_t M)
+{
+    if (validate_linear(w1) != HQQ_OK || validate_linear(w3) != HQQ_OK || M <= 0 || w1->N != w3->N || w1->K != w3->K)
+        return 0;
+    return gate_matmul_scratch(w1, w3, M) + 2 * align256((size_t)M * w1->N * 2);
+}
+
 int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, int64_t M, void *h_f16, void *workspace,
                 size_t workspace_bytes, void *stream)
 {
@@ -228,13 +247,37 @@ int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, i
         return HQQ_OK;
     if (!x_f16 || !h_f16)
         return HQQ_E_NULL;
-    if (!smallbatch_supported(w1, M) || !smallbatch_supported(w3, M) || w1->bias || w3->bias ||
-        w1->nbits != w3->nbits || w1->group_size != w3->group_size)
-        return HQQ_E_UNSUPPORTED;
+    if (w1->bias || w3->bias)
+        return HQQ_E_UNSUPPORTED; // the reference's experts have none (src/custom_layers.py:253-256)
     if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return HQQ_E_WORKSPACE;
-    return launch_smallbatch_gate_up(w1, w3, (const f16 *)x_f16, M, (f16 *)h_f16, workspace, workspace_bytes,
-                                     (hipStream_t)stream);
+    hipStream_t s = (hipStream_t)stream;
+    const f16 *x = (const f16 *)x_f16;
+    f16 *h = (f16 *)h_f16;
+    const bool alike = w1->nbits == w3->nbits && w1->group_size == w3->group_size;
+    // one fused launch where a kernel family has one for the batch; the decode kernels need no more workspace than
+    // they check for themselves
+    const bool prefer_tile = tile_supported(w1, M) && tile_supported(w3, M) && !strip_supported(w1, M);
+    if (alike && !prefer_tile && smallbatch_supported(w1, M) && smallbatch_supported(w3, M))
+        return launch_smallbatch_gate_up(w1, w3, x, M, h, workspace, workspace_bytes, s);
+    if (prefer_tile && tile_gate_supported(w1, w3, M))
+        return launch_tile_gate_up(w1, w3, x, M, h, workspace, workspace_bytes, s);
+    // otherwise both projections (3-bit decode batches: in one launch), then silu(a) * b
+    if (workspace_bytes < hqq_gate_up_workspace_bytes(w1, w3, M))
+        return HQQ_E_WORKSPACE;
+    char *p = static_cast<char *>(workspace);
+    const size_t mm_bytes = gate_matmul_scratch(w1, w3, M), mid = align256((size_t)M * w1->N * 2);
+    f16 *a = (f16 *)(p + mm_bytes), *b = (f16 *)(p + mm_bytes + mid);
+    if (pick_family(w1, M) == FAM_VEC3 && pick_family(w3, M) == FAM_VEC3 && vec3_gate_supported(w1, w3, M)) {
+        if ((rc = launch_vec3_gate(w1, w3, x, M, a, (int64_t)(mid / 2), 1, p, mm_bytes, s)) != HQQ_OK)
+            return rc;
+    } else {
+        if ((rc = run_matmul(w1, x, M, a, p, mm_bytes, pick_family(w1, M), s)) != HQQ_OK)
+            return rc;
+        if ((rc = run_matmul(w3, x, M, b, p, mm_bytes, pick_family(w3, M), s)) != HQQ_OK)
+            return rc;
+    }
+    return launch_silu_mul(a, b, h, M * w1->N, s);
 }
 
 int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *x_f16, int64_t M,

@@ -549,6 +549,19 @@ size_t vec3_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2, int6
     return ga > gb ? ga : gb;
 }
 
+bool vec3_gate_supported(const hqq_linear *w1, const hqq_linear *w3, int64_t M)
+{
+    W3Plan pl;
+    return M >= 1 && M <= 16 && same_layout(w1, w3) && !w1->bias && !w3->bias && make_plan(w1, M, 2, pl) &&
+           make_plan(w3, M, 2, pl);
+}
+
+size_t vec3_gate_workspace_bytes(const hqq_linear *w1, int64_t M)
+{
+    W3Plan pl;
+    return make_plan(w1, M, 2, pl) ? job_workspace_bytes(pl, w1, 2) : 0;
+}
+
 // ab: the gate outputs, layer l (w1 then w3 of each expert) at ab + l * ab_lstride, each (M, N)
 int launch_vec3_gate(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *ab, int64_t ab_lstride,
                      int n_experts, void *ws, size_t ws_bytes, hipStream_t s, const StripIndex *ix)

@@ -197,6 +197,21 @@ def expert_ffn(w1: LinearDesc, w2: LinearDesc, w3: LinearDesc, x: torch.Tensor, 
     return out
 
 
+def gate_up(w1: LinearDesc, w3: LinearDesc, x: torch.Tensor) -> torch.Tensor:
+    """``silu(w1 x) * (w3 x)``, the first half of the expert FFN (reference src/custom_layers.py:254)."""
+    assert x.dtype == torch.float16 and x.is_contiguous() and x.shape[-1] == w1.K == w3.K and w1.N == w3.N
+    xv = x.view(-1, w1.K)
+    M = xv.shape[0]
+    out = torch.empty((M, w1.N), dtype=torch.float16, device=x.device)
+    if M == 0:
+        return out
+    with torch.cuda.device(x.device):
+        ws = workspace(x.device, _lib.lib.hqq_gate_up_workspace_bytes(w1.ref, w3.ref, M))
+        _lib.check(_lib.lib.hqq_gate_up(w1.ref, w3.ref, xv.data_ptr(), M, out.data_ptr(), ws.data_ptr(), ws.numel(),
+                                        _lib.current_stream_ptr(x.device)), "hqq_gate_up")
+    return out
+
+
 class ExpertTable:
     """Device-resident table of the experts of one MoE layer for ``expert_ffn_indexed``: three records per expert
     (w1, w3, w2).  ``experts`` is a list of (w1, w2, w3) ``LinearDesc`` triples that all share one shape."""

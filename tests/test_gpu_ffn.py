@@ -114,3 +114,44 @@ def test_full_size_ffn_against_dequantize_then_matmul(m):
         atol = 4e-3 * h.float().norm(dim=1)[:, None] * wc.norm(dim=1)[None, :]
         bound = 2e-2 * ref.abs() + atol
         assert bool((err <= bound).all()), float((err / bound).max())
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "w%d_h%d_f%d_g%d_%s" % (s[0], s[1], s[2], s[3], "q" if s[4] else "f16"))
+@pytest.mark.parametrize("m", [1, 2, 4, 7, 16, 40])
+def test_gate_up_entry_point(shape, m):
+    """hqq_gate_up against the numpy oracle's silu(x w1^T) * (x w3^T) (reference src/custom_layers.py:254), and
+    against the two projections done one by one on the GPU followed by torch's silu * up: the fused kernels round where
+    those three steps round, so the two agree to an fp16 ulp of the larger values."""
+    from mixtral_offloading_amd import hip_kernels
+    nbits, hidden, ffn, gs, qt = shape
+    rng = np.random.default_rng(3 * hidden + ffn + m)
+    w1, _, w3 = _ffn_case(rng, nbits, hidden, ffn, gs, qt)
+    x = rng.standard_normal((m, hidden)).astype(np.float16)
+    d1, d3 = desc_of(w1), desc_of(w3)
+    a = o.matmul_transpose(x, w1)
+    b = o.matmul_transpose(x, w3)
+    want = (o.silu_f16(a).astype(np.float32) * b.astype(np.float32)).astype(np.float16)
+    ta, tb = o.matmul_tolerance(x, w1), o.matmul_tolerance(x, w3)
+    # |d(silu(a) b)| <= |b| |da| * max|silu'| + |silu(a)| |db|, max|silu'| < 1.1
+    atol = 1.1 * np.abs(b.astype(np.float32)) * ta + np.abs(o.silu_f16(a).astype(np.float32)) * tb + 1e-3
+    xd = to_dev(x)
+    for rep in range(2):
+        got = hip_kernels.gate_up(d1, d3, xd)
+        assert_matmul_close(got.cpu().numpy(), want, atol, rtol=2e-2)
+    steps = torch.nn.functional.silu(hip_kernels.matmul(d1, xd).float()).half() * hip_kernels.matmul(d3, xd)
+    err = (got.float() - steps.float()).abs().max().item()
+    assert err <= 4e-3 * steps.float().abs().max().item() + 1e-3, err
+
+
+def test_gate_up_refuses_bias_and_mismatched_layers():
+    from mixtral_offloading_amd import _lib, hip_kernels
+    rng = np.random.default_rng(5)
+    w1, _ = o.random_layer(rng, 512, 256, 2, 16)
+    w3, _ = o.random_layer(rng, 512, 256, 2, 16)
+    other, _ = o.random_layer(rng, 768, 256, 2, 16)
+    x = to_dev(rng.standard_normal((2, 256)).astype(np.float16))
+    with pytest.raises(_lib.HqqError):
+        hip_kernels.gate_up(desc_of(w1, bias=np.zeros(512, np.float16)), desc_of(w3), x)
+    with pytest.raises(AssertionError):
+        hip_kernels.gate_up(desc_of(w1), desc_of(other), x)
+    assert hip_kernels.gate_up(desc_of(w1), desc_of(w3), x[:0]).shape == (0, 512)

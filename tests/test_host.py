@@ -54,6 +54,15 @@ def test_argument_errors_without_touching_the_gpu():
     assert lib.hqq_matmul_group(ptrs, 1, 1 << 20, ys, None, 0, None) == -5  # no workspace
     assert lib.hqq_expert_pair_ffn_indexed(ctypes.byref(ok), ctypes.byref(ok), ctypes.byref(ok), None, None, None, None,
                                            None, 0, None, 0, None) == -3  # w2 must map ffn -> hidden
+    other = _lib.HqqLinear()
+    other.nbits, other.group_size, other.N, other.K, other.codes = 4, 64, 512, 512, 1 << 20
+    other.scale.data = other.zero.data = 1 << 21
+    assert lib.hqq_gate_up(ctypes.byref(ok), ctypes.byref(other), 1 << 20, 1, 1 << 22, 1 << 23, 1 << 20, None) == -3
+    assert lib.hqq_gate_up_workspace_bytes(ctypes.byref(ok), ctypes.byref(other), 1) == 0
+    assert lib.hqq_gate_up(ctypes.byref(ok), ctypes.byref(ok), None, 1, 1 << 22, 1 << 23, 1 << 20, None) == -1
+    assert lib.hqq_gate_up(ctypes.byref(ok), ctypes.byref(ok), None, 0, None, None, 0, None) == 0  # empty batch
+    assert lib.hqq_gate_up(ctypes.byref(ok), ctypes.byref(ok), 1 << 20, 1, 1 << 22, None, 0, None) == -5  # no workspace
+    assert lib.hqq_gate_up_workspace_bytes(ctypes.byref(ok), ctypes.byref(ok), 3) > 0
     assert lib.hqq_add_rmsnorm_router(None, None, None, 1e-5, None, 4096, None, 8, None, None, None, None) == -1
     assert lib.hqq_add_rmsnorm_router(1 << 20, None, 1 << 21, 1e-5, 1 << 22, 4096, 1 << 23, 17, 1 << 24, 1 << 25, None,
                                       None) == -3  # more than 16 experts
