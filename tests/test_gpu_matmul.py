@@ -193,3 +193,26 @@ def test_workspace_head_is_left_at_zero():
     torch.cuda.synchronize()
     head = hip_kernels.workspace(dev, 1)[: 576 * 1024]
     assert head.numel() == 576 * 1024 and not bool(head.any())
+
+
+def test_workspace_init_makes_a_dirty_workspace_usable():
+    """A caller that brings its own workspace zeroes its head with hqq_workspace_init (a small kernel, so it may be
+    recorded into a graph); the split-K launches then work on it."""
+    from mixtral_offloading_amd import _lib
+    rng = np.random.default_rng(123)
+    layer, _ = o.random_layer(rng, 256, 8192, 2, 16)
+    d = desc_of(layer)
+    stream = _lib.current_stream_ptr(torch.device("cuda:0"))
+    for m in (1, 4):
+        x = rng.standard_normal((m, 8192)).astype(np.float16)
+        need = int(_lib.lib.hqq_matmul_workspace_bytes(d.ref, m))
+        ws = torch.full((need,), 0xFF, dtype=torch.uint8, device="cuda")
+        assert _lib.lib.hqq_workspace_init(ws.data_ptr() + 1, need - 1, stream) == -5  # misaligned
+        assert _lib.lib.hqq_workspace_init(ws.data_ptr(), need, stream) == 0
+        assert not bool(ws[: 576 * 1024].any()) and bool((ws[576 * 1024:] == 0xFF).all())
+        xd, y = to_dev(x), torch.empty((m, 256), dtype=torch.float16, device="cuda")
+        for rep in range(2):
+            _lib.check(_lib.lib.hqq_matmul_transpose(d.ref, xd.data_ptr(), m, y.data_ptr(), ws.data_ptr(), need, stream),
+                       "hqq_matmul_transpose")
+            assert_matmul_close(y.cpu().numpy(), o.matmul_transpose(x, layer), o.matmul_tolerance(x, layer))
+        assert not bool(ws[: 576 * 1024].any())
