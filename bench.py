@@ -118,7 +118,7 @@ def random_desc(nbits, n, k, gs, seed, dev):
 
 
 def survey_section(dev):
-    """Every kernel of the path at the BASELINE shapes: microseconds per launch by HIP events (cache-cold: each
+    """Every kernel of the path at the Mixtral-8x7B shapes: microseconds per launch by HIP events (cache-cold: each
     timing rotates over more than 256 MB of distinct inputs) and the rate that follows from its algorithmic bytes."""
     import torch
 
@@ -190,7 +190,7 @@ def survey_section(dev):
 
 
 def decode_section(dev, tokens_resident=256, tokens_offload=48):
-    """Tokens per second of the whole model (BASELINE configs[4]); every figure is measured between synchronisations
+    """Tokens per second of the whole model; every figure is measured between synchronisations
     around the decode loop, prompt processing excluded."""
     import gc
 
@@ -233,7 +233,7 @@ def decode_section(dev, tokens_resident=256, tokens_offload=48):
             out["all_experts_resident_graph_tok_s"] = round(tokens_resident / (time.perf_counter() - t0), 1)
             out["all_experts_resident_graph_tokens"] = tokens_resident
             del dec
-            # the same step with a 512-token KV cache (BASELINE configs[3]): 64 tokens after a 512-token prompt
+            # the same step with a 512-token KV cache: 64 tokens after a 512-token prompt
             ctx = torch.randint(0, cfg.vocab_size, (512,), device=dev, generator=gen)
             dec = DecodeGraph(model, 512 + 64 + 4)
             dec.prefill(ctx)
@@ -301,7 +301,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the whole-model decode section")
     ap.add_argument("--survey", action="store_true",
-                    help="also time every kernel of the path (packers, de-quantiser, 2/3/4-bit matmuls at the BASELINE "
+                    help="also time every kernel of the path (packers, de-quantiser, 2/3/4-bit matmuls at the Mixtral-8x7B "
                          "shapes and batches) and add the table as 'kernels'")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain 256 MiB device copies, so that a counter run can scale FETCH_SIZE / WRITE_SIZE "

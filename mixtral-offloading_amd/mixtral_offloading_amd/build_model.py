@@ -1,7 +1,7 @@
 """Model assembly with the reference's entry points (``src/build_model.py``):
 ``OffloadConfig``, ``QuantConfig``, ``replace_attn_layers``, ``make_empty_expert``,
 ``build_model``.  Without a ``state_path`` the model gets seeded random weights of the
-Mixtral architecture, quantised on the GPU (the BASELINE configurations); with one, the
+Mixtral architecture, quantised on the GPU (what the benchmark runs on); with one, the
 expert and trunk tensors are read from the reference's safetensors shards."""
 from __future__ import annotations
 
