@@ -19,6 +19,24 @@ from ._lib import HqqLinear, HqqTable
 _workspaces = {}
 
 
+class _Stay:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_STAY = _Stay()
+
+
+def _on(device: torch.device):
+    """Context that makes ``device`` current for the launches inside; free when it already is."""
+    if device.index is None or torch.cuda.current_device() == device.index:
+        return _STAY
+    return torch.cuda.device(device)
+
+
 def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     """Per (device, stream) scratch for split-K partial sums; grows on demand.
     Calls on one stream are ordered, so sharing it between them is safe."""
@@ -104,7 +122,7 @@ def matmul(desc: LinearDesc, a: torch.Tensor, family: int = -1) -> torch.Tensor:
     M = x.shape[0]
     c = torch.empty((M, desc.N), device=a.device, dtype=torch.float16)
     if M > 0:
-        with torch.cuda.device(a.device):
+        with _on(a.device):
             need = _lib.lib.hqq_matmul_workspace_bytes(desc.ref, M)
             ws = workspace(a.device, need)
             _lib.check(_lib.lib.hqq_matmul_transpose_ex(desc.ref, x.data_ptr(), M, c.data_ptr(), ws.data_ptr(),
@@ -154,7 +172,7 @@ triton_matmul3_transpose = hip_matmul3_transpose
 
 def dequantize(desc: LinearDesc) -> torch.Tensor:
     w = torch.empty((desc.N, desc.K), dtype=torch.float16, device=desc.device)
-    with torch.cuda.device(desc.device):
+    with _on(desc.device):
         _lib.check(_lib.lib.hqq_dequantize(desc.ref, w.data_ptr(), _lib.current_stream_ptr(desc.device)),
                    "hqq_dequantize")
     return w
@@ -164,7 +182,7 @@ def table_to_f16(values: torch.Tensor, meta: dict) -> torch.Tensor:
     """``Quantizer.dequantize`` of an 8-bit scale / zero table (reference src/custom_layers.py:63-66)."""
     t, keep = _table(values, meta)
     out = torch.empty(meta["shape"] if "shape" in meta else values.shape, dtype=torch.float16, device=values.device)
-    with torch.cuda.device(values.device):
+    with _on(values.device):
         _lib.check(_lib.lib.hqq_table_to_f16(ctypes.byref(t), values.numel(), out.data_ptr(),
                                              _lib.current_stream_ptr(values.device)), "hqq_table_to_f16")
     del keep
@@ -187,7 +205,7 @@ def expert_ffn(w1: LinearDesc, w2: LinearDesc, w3: LinearDesc, x: torch.Tensor, 
     if row_scale is not None:
         row_scale = row_scale.to(torch.float16).contiguous()
         assert row_scale.numel() == M
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         need = _lib.lib.hqq_expert_ffn_workspace_bytes(w1.ref, w2.ref, w3.ref, M)
         ws = workspace(x.device, need)
         _lib.check(_lib.lib.hqq_expert_ffn(w1.ref, w2.ref, w3.ref, xv.data_ptr(), M, out.data_ptr(),
@@ -205,7 +223,7 @@ def gate_up(w1: LinearDesc, w3: LinearDesc, x: torch.Tensor) -> torch.Tensor:
     out = torch.empty((M, w1.N), dtype=torch.float16, device=x.device)
     if M == 0:
         return out
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         ws = workspace(x.device, _lib.lib.hqq_gate_up_workspace_bytes(w1.ref, w3.ref, M))
         _lib.check(_lib.lib.hqq_gate_up(w1.ref, w3.ref, xv.data_ptr(), M, out.data_ptr(), ws.data_ptr(), ws.numel(),
                                         _lib.current_stream_ptr(x.device)), "hqq_gate_up")
@@ -237,7 +255,7 @@ def expert_ffn_indexed(table: ExpertTable, expert_index: torch.Tensor, x: torch.
     assert expert_index.dtype == torch.int32 and expert_index.is_cuda
     M = x.numel() // w1.K
     assert out.is_contiguous() and out.numel() == M * w2.N and out.dtype == torch.float16
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         need = _lib.lib.hqq_expert_ffn_workspace_bytes(w1.ref, w2.ref, w3.ref, M)
         ws = workspace(x.device, need)
         _lib.check(_lib.lib.hqq_expert_ffn_indexed(w1.ref, w2.ref, w3.ref, table.table.data_ptr(),
@@ -270,7 +288,7 @@ def expert_pair_ffn_indexed(table: ExpertTable, expert_index: torch.Tensor, x: t
     assert expert_index.dtype == torch.int32 and expert_index.is_cuda and expert_index.numel() >= 2
     assert row_scale.dtype == torch.float16 and row_scale.is_cuda and row_scale.numel() >= 2
     assert out.is_contiguous() and out.numel() == w2.N and out.dtype == torch.float16
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         need = _lib.lib.hqq_expert_pair_ffn_workspace_bytes(w1.ref, w2.ref, w3.ref)
         ws = workspace(x.device, need)
         _lib.check(_lib.lib.hqq_expert_pair_ffn_indexed(w1.ref, w2.ref, w3.ref, table.table.data_ptr(),
@@ -293,7 +311,7 @@ def moe_pair_routed(table: ExpertTable, x: torch.Tensor, delta: Optional[torch.T
     assert gate_weight.is_contiguous() and sel.dtype == torch.int32 and sel.numel() >= 2
     assert weights.dtype == torch.float16 and weights.numel() >= 2
     assert out.is_contiguous() and out.numel() == w2.N and out.dtype == torch.float16
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         need = _lib.lib.hqq_expert_pair_ffn_workspace_bytes(w1.ref, w2.ref, w3.ref)
         ws = workspace(x.device, need)
         _lib.check(_lib.lib.hqq_moe_pair_routed(w1.ref, w2.ref, w3.ref, table.table.data_ptr(), x.data_ptr(),
@@ -321,7 +339,7 @@ class LinearGroup:
         assert x.dtype == torch.float16 and x.is_contiguous() and x.numel() == d0.K and x.device == d0.device
         outs = [torch.empty((1, d.N), device=x.device, dtype=torch.float16) for d in self.descs]
         ys = (ctypes.c_void_p * len(outs))(*[o.data_ptr() for o in outs])
-        with torch.cuda.device(x.device):
+        with _on(x.device):
             ws = workspace(x.device, self.need)
             _lib.check(_lib.lib.hqq_matmul_group(self._ptrs, len(outs), x.data_ptr(), ys, ws.data_ptr(), ws.numel(),
                                                  _lib.current_stream_ptr(x.device)), "hqq_matmul_group")
@@ -338,7 +356,7 @@ def matmul_group_norm(group: LinearGroup, x: torch.Tensor, delta: Optional[torch
     assert weight.dtype == torch.float16 and weight.numel() == d0.K
     outs = [torch.empty((1, d.N), device=x.device, dtype=torch.float16) for d in group.descs]
     ys = (ctypes.c_void_p * len(outs))(*[o.data_ptr() for o in outs])
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         ws = workspace(x.device, group.need)
         _lib.check(_lib.lib.hqq_matmul_group_norm(group._ptrs, len(outs), x.data_ptr(),
                                                   delta.data_ptr() if delta is not None else None, weight.data_ptr(),
@@ -354,7 +372,7 @@ def router_top2(x: torch.Tensor, gate_weight: torch.Tensor, sel: torch.Tensor, w
     n_experts, hidden = gate_weight.shape
     assert x.dtype == torch.float16 and gate_weight.dtype == torch.float16 and x.numel() == hidden
     assert sel.dtype == torch.int32 and sel.numel() >= 2 and weights.dtype == torch.float16 and weights.numel() >= 2
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         _lib.check(_lib.lib.hqq_router_top2(x.data_ptr(), gate_weight.data_ptr(), n_experts, hidden, sel.data_ptr(),
                                             weights.data_ptr(), logits.data_ptr() if logits is not None else None,
                                             _lib.current_stream_ptr(x.device)), "hqq_router_top2")
@@ -364,7 +382,7 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
                 out: torch.Tensor) -> torch.Tensor:
     """``x += delta`` (when given) then ``out = weight * rmsnorm(x)`` for one token."""
     assert x.dtype == torch.float16 and x.is_contiguous() and out.dtype == torch.float16 and x.numel() == weight.numel()
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         _lib.check(_lib.lib.hqq_add_rmsnorm(x.data_ptr(), delta.data_ptr() if delta is not None else None,
                                             weight.data_ptr(), float(eps), out.data_ptr(), x.numel(),
                                             _lib.current_stream_ptr(x.device)), "hqq_add_rmsnorm")
@@ -379,7 +397,7 @@ def add_rmsnorm_router(x: torch.Tensor, delta: Optional[torch.Tensor], weight: t
     assert x.dtype == torch.float16 and x.is_contiguous() and out.dtype == torch.float16 and x.numel() == weight.numel()
     assert gate_weight.dtype == torch.float16 and gate_weight.is_contiguous() and x.numel() == hidden
     assert sel.dtype == torch.int32 and sel.numel() >= 2 and weights.dtype == torch.float16 and weights.numel() >= 2
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         _lib.check(_lib.lib.hqq_add_rmsnorm_router(x.data_ptr(), delta.data_ptr() if delta is not None else None,
                                                    weight.data_ptr(), float(eps), out.data_ptr(), hidden,
                                                    gate_weight.data_ptr(), n_experts, sel.data_ptr(), weights.data_ptr(),
@@ -396,7 +414,7 @@ def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: tor
     assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous() and cache_k.is_contiguous() and cache_v.is_contiguous()
     assert pos.dtype == torch.int64 and pos.is_cuda and cos.shape[-1] == hd and cos.is_contiguous() and sin.is_contiguous()
     assert out.numel() == n_heads * hd and k.numel() == n_kv * hd == v.numel()
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         _lib.check(_lib.lib.hqq_attention_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), cos.data_ptr(), sin.data_ptr(),
                                                  pos.data_ptr(), cache_k.data_ptr(), cache_v.data_ptr(), max_len, n_heads,
                                                  n_kv, hd, out.data_ptr(), _lib.current_stream_ptr(q.device)),
