@@ -151,8 +151,7 @@ int hqq_expert_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq
  *      blocks, up to one fp16 rounding: the weighted sum of both experts is then formed in higher precision and
  *      rounded once, where index_add_ on fp16 tensors rounds each product and the sum).  One launch
  *      computes silu(w1 x) * w3 x of both experts, one both down projections and their weighted sum (3-bit experts:
- *      three launches -- the four gate projections, then one down projection per expert that applies silu(a) * b
- *      as it reads them, the second adding into y).  x is one row
+ *      the four gate projections, then both down projections, which apply silu(a) * b as they read them).  x is one row
  *      (hidden fp16), expert_index two device int32, row_scale two device fp16.  Table as for
  *      hqq_expert_ffn_indexed.  HQQ_E_UNSUPPORTED when the shapes do not fit the decode kernel (the workspace query
  *      then returns 0): call hqq_expert_ffn_indexed twice instead.                                                 */

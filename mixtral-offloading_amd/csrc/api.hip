@@ -460,6 +460,11 @@ int hqq_expert_pair_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, cons
         const int64_t ls = (int64_t)(mid / 2);
         if ((rc = launch_vec3_gate(w1, w3, (const f16 *)x_f16, 1, h0, ls, 2, p, mm_bytes, s, &gate)) != HQQ_OK)
             return rc;
+        // both down projections in one launch where K is split over blocks (their results then meet in the
+        // outputs' accumulation slots), else one launch per expert, the second adding into y
+        rc = launch_vec3_down_pair(w2, h0, ls, (f16 *)y_f16, (const f16 *)row_scale_f16, accumulate, p, mm_bytes, s, down);
+        if (rc != HQQ_E_UNSUPPORTED)
+            return rc;
         const StripIndex down1 = {device_table, expert_index + 1, 3, 2};
         SmallBatchEpilogue ep;
         ep.row_scale = (const f16 *)row_scale_f16;

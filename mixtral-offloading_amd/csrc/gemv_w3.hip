@@ -44,11 +44,14 @@ struct W3Params {
     const int *sel;
     int stride, first, lper;
     const f16 *x;       // XMODE 0: (M, K)
-    const f16 *xa, *xb; // XMODE 1: x = silu(xa) * xb, both (M, K)
+    const f16 *xa, *xb; // XMODE 1: x = silu(xa) * xb, both (M, K); layer l reads them x_lstride elements further
+    int64_t x_lstride;
     f16 *y;             // layer l writes y + l * y_lstride
     int64_t y_lstride;
     const f16 *bias;      // single layer from the kernel arguments only
     const f16 *row_scale; // optional multiplier per batch row
+    int pair; // the layers of the launch are the down projections of two experts: y (+)= sum over l of
+              // row_scale[l] * o_l, formed in the outputs' accumulation slots and rounded to fp16 once
     int accumulate;       // add into y
     float *part; // layer l: part + l * part_lstride, [BK][M][N]
     int64_t part_lstride;
@@ -117,7 +120,7 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
     } else {
         R = p.layer[__builtin_amdgcn_readfirstlane(layer)];
     }
-    f16 *const yl = p.y + (int64_t)layer * p.y_lstride;
+    f16 *const yl = p.y + (int64_t)(p.pair ? 0 : layer) * p.y_lstride;
     float *const partl = p.part + (int64_t)layer * p.part_lstride;
     const int M = MT == 1 ? 1 : p.M;
     const int K = p.K;
@@ -181,8 +184,8 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
         for (int m = 0; m < MT; ++m) {
             const uint32_t at = (uint32_t)((m < M ? m : 0) * K) + k0 + (uint32_t)(4 * lane);
             if constexpr (XMODE) {
-                xg[m] = gload<u32x2>(p.xa + at);
-                xr[m] = gload<u32x2>(p.xb + at);
+                xg[m] = gload<u32x2>(p.xa + (int64_t)layer * p.x_lstride + at);
+                xr[m] = gload<u32x2>(p.xb + (int64_t)layer * p.x_lstride + at);
             } else {
                 xr[m] = gload<u32x2>(p.x + at);
             }
@@ -290,7 +293,7 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
         f16 val = (f16)v;
         if (p.bias)
             val = val + p.bias[n];
-        if (p.row_scale)
+        if (p.row_scale && !p.pair)
             val = val * p.row_scale[m_t];
         f16 *dst = yl + (int64_t)m_t * p.N + n;
         *dst = p.accumulate ? (f16)(*dst + val) : val;
@@ -308,12 +311,14 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
             finish(m_t, n, v);
         } else if (p.slots) {
             // the K blocks add into the output's slot; the block whose addition completes it writes the output
-            unsigned long long *slot = p.slots + (((int64_t)layer * p.N + n) * MT + m_t);
-            const unsigned long long mine = slot_term(v);
+            // (a pair of experts shares the slots: every block's result enters with its expert's routing weight)
+            const int arrivals = p.pair ? 2 * p.BK : p.BK;
+            unsigned long long *slot = p.slots + (((int64_t)(p.pair ? 0 : layer) * p.N + n) * MT + m_t);
+            const unsigned long long mine = slot_term(p.pair ? v * (float)p.row_scale[layer] : v);
             const unsigned long long before = __hip_atomic_fetch_add(slot, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (slot_count(before) == p.BK - 1) {
+            if (slot_count(before) == arrivals - 1) {
                 __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                finish(m_t, n, slot_total(before + mine, p.BK));
+                finish(m_t, n, slot_total(before + mine, arrivals));
             }
         } else {
             __hip_atomic_store(partl + ((int64_t)kb * M + m_t) * p.N + n, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -421,6 +426,8 @@ struct W3Job {
     const StripIndex *ix; // records from a device table: layer l is record sel[l / lper] * stride + first + l % lper
     int lper;
     const f16 *x, *xa, *xb; // x, or xa and xb (x = silu(xa) * xb)
+    int64_t x_lstride;      // xa, xb of layer l (paired down projections)
+    int pair;
     f16 *y;
     int64_t y_lstride;
     SmallBatchEpilogue ep;
@@ -474,8 +481,12 @@ int run_job(const W3Job &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
     p.lper = j.lper > 0 ? j.lper : 1;
     p.counter = static_cast<int *>(ws);
     p.part = pl.BK > 1 ? reinterpret_cast<float *>(static_cast<char *>(ws) + kHeadBytes) : nullptr;
-    if (pl.BK > 1 && pl.BK <= 8 && (size_t)j.NL * (size_t)l->N * 2 * sizeof(unsigned long long) <= kSlotBytes)
+    if (pl.BK > 1 && pl.BK * (j.pair ? 2 : 1) <= 14 &&
+        (size_t)(j.pair ? 1 : j.NL) * (size_t)l->N * 2 * sizeof(unsigned long long) <= kSlotBytes)
         p.slots = reinterpret_cast<unsigned long long *>(static_cast<char *>(ws) + kCounterBytes);
+    if (j.pair && (!p.slots || M != 1 || j.NL != 2 || !fused || !j.ep.row_scale))
+        return HQQ_E_UNSUPPORTED; // the shared slots are what joins the two experts
+    p.pair = j.pair, p.x_lstride = j.x_lstride;
     p.part_lstride = (int64_t)pl.BK * 2 * l->N;
     p.y_lstride = j.y_lstride;
     p.accumulate = j.ep.accumulate;
@@ -545,8 +556,15 @@ size_t vec3_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2, int6
     W3Plan a, b;
     if (!make_plan(w1, M, 2 * n_experts, a) || !make_plan(w2, M, 1, b))
         return 0;
-    const size_t ga = job_workspace_bytes(a, w1, 2 * n_experts), gb = job_workspace_bytes(b, w2, 1);
-    return ga > gb ? ga : gb;
+    size_t need = job_workspace_bytes(a, w1, 2 * n_experts);
+    const size_t gb = job_workspace_bytes(b, w2, 1);
+    need = gb > need ? gb : need;
+    W3Plan c;
+    if (n_experts == 2 && make_plan(w2, M, 2, c)) { // both down projections in one launch
+        const size_t gc = job_workspace_bytes(c, w2, 2);
+        need = gc > need ? gc : need;
+    }
+    return need;
 }
 
 bool vec3_gate_supported(const hqq_linear *w1, const hqq_linear *w3, int64_t M)
@@ -582,6 +600,19 @@ int launch_vec3_down(const hqq_linear *w2, const f16 *a, const f16 *b, int64_t M
     j.layers[0] = w2, j.NL = 1, j.ix = ix, j.lper = 1;
     j.xa = a, j.xb = b, j.y = y, j.ep = ep;
     return run_job(j, M, ws, ws_bytes, s);
+}
+
+// Both down projections of a token's two experts (records sel[0] and sel[1]) in one launch:
+// y (+)= rw[0] * w2_0(silu(a0) * b0) + rw[1] * w2_1(silu(a1) * b1), expert e reading a, b at ab + 2 * e * ab_lstride
+// and ab + (2 * e + 1) * ab_lstride.  HQQ_E_UNSUPPORTED when K fits one block (the caller makes two launches).
+int launch_vec3_down_pair(const hqq_linear *w2, const f16 *ab, int64_t ab_lstride, f16 *y, const f16 *row_scale,
+                          int accumulate, void *ws, size_t ws_bytes, hipStream_t s, const StripIndex &ix)
+{
+    W3Job j = {};
+    j.layers[0] = w2, j.layers[1] = w2, j.NL = 2, j.ix = &ix, j.lper = 1, j.pair = 1;
+    j.xa = ab, j.xb = ab + ab_lstride, j.x_lstride = 2 * ab_lstride, j.y = y;
+    j.ep.row_scale = row_scale, j.ep.accumulate = accumulate;
+    return run_job(j, 1, ws, ws_bytes, s);
 }
 
 } // namespace hqq

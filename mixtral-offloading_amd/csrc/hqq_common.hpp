@@ -183,6 +183,8 @@ int launch_vec3_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, voi
 // w1 then w3 of each expert; two experts only from a record table), then the down projection reading silu(a) * b
 bool vec3_ffn_supported(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, int64_t M, int n_experts);
 size_t vec3_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2, int64_t M, int n_experts);
+int launch_vec3_down_pair(const hqq_linear *w2, const f16 *ab, int64_t ab_lstride, f16 *y, const f16 *row_scale,
+                          int accumulate, void *ws, size_t ws_bytes, hipStream_t s, const StripIndex &ix);
 bool vec3_gate_supported(const hqq_linear *w1, const hqq_linear *w3, int64_t M);
 size_t vec3_gate_workspace_bytes(const hqq_linear *w1, int64_t M);
 int launch_vec3_gate(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *ab, int64_t ab_lstride,
