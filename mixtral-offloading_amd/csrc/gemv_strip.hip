@@ -121,6 +121,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     __shared__ f16 rw_lds[2];
     // ROUTED launches: the normed row, written once by the prologue and read by every slab (hidden <= 4096)
     __shared__ __attribute__((aligned(16))) f16 xn_lds[ROUTED ? 4096 : 8];
+    // ROUTED launches: the records of both gate projections of every expert, fetched while the router runs, so that
+    // the chosen ones are at hand when it is done (one trip to memory less in front of the first weight load)
+    constexpr int REC_WORDS = sizeof(StripLayer) / 4, REC_ALL = 8 * 2 * REC_WORDS;
+    constexpr int REC_PER = (REC_ALL + WAVES * 64 - 1) / (WAVES * 64);
+    __shared__ uint32_t rec_lds[ROUTED ? REC_ALL : 1];
 
     const int lane = threadIdx.x & 63;
     // the wave index as a scalar: what depends on it (the layer, its record, the K range) then lives in scalar
@@ -144,8 +149,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
         // on: with an LDS array of its own the block no longer fits twice into a compute unit
         static_assert(!ROUTED || sizeof(code_lds) >= sizeof(NormRouteLds<8>), "router scratch does not fit the staging buffer");
         NormRouteLds<8> &route_lds = *reinterpret_cast<NormRouteLds<8> *>(&code_lds[0][0]);
+        uint32_t recw[REC_PER];
+#pragma unroll
+        for (int q = 0; q < REC_PER; ++q) {
+            const int t = (int)threadIdx.x + q * WAVES * 64;
+            const int tc = t < p.n_experts * 2 * REC_WORDS ? t : 0; // spare threads repeat word 0
+            const int ex = tc / (2 * REC_WORDS), rem = tc - ex * 2 * REC_WORDS, ly = rem / REC_WORDS, w = rem - ly * REC_WORDS;
+            recw[q] = gload<uint32_t>(reinterpret_cast<const uint32_t *>(p.table + (ex * p.table_stride + p.table_first + ly * p.first_lstride)) + w);
+        }
         rnorm = norm_route_block<2, 8>(p.x, p.norm_delta, p.norm_weight, p.norm_eps, writer ? p.x_sum : nullptr, xn_lds, p.K,
                                        p.gate_w, p.n_experts, sel_lds, rw_lds, nullptr, route_lds);
+#pragma unroll
+        for (int q = 0; q < REC_PER; ++q) {
+            const int t = (int)threadIdx.x + q * WAVES * 64;
+            if (t < p.n_experts * 2 * REC_WORDS)
+                rec_lds[t] = recw[q];
+        }
         __syncthreads();
         if (writer && threadIdx.x < 2) {
             p.sel_out[threadIdx.x] = sel_lds[threadIdx.x];
@@ -158,9 +177,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
         // one word of the record per lane, then broadcast: the record's address is known only now
         const int sel_at = g * p.sel_gstride + layer * p.sel_lstride;
         const int e = __builtin_amdgcn_readfirstlane(ROUTED ? sel_lds[sel_at] : p.sel[sel_at]);
-        const uint32_t *src =
-            reinterpret_cast<const uint32_t *>(p.table + (e * p.table_stride + p.table_first + layer * p.first_lstride));
-        const uint32_t word = src[lane < 18 ? lane : 0];
+        uint32_t word;
+        if constexpr (ROUTED) {
+            word = rec_lds[(e * 2 + layer) * REC_WORDS + (lane < 18 ? lane : 0)];
+        } else {
+            const uint32_t *src =
+                reinterpret_cast<const uint32_t *>(p.table + (e * p.table_stride + p.table_first + layer * p.first_lstride));
+            word = src[lane < 18 ? lane : 0];
+        }
         uint32_t rec[18];
 #pragma unroll
         for (int i = 0; i < 18; ++i)
