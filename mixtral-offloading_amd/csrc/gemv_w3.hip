@@ -91,7 +91,8 @@ __device__ __forceinline__ f16 silu_mul(f16 a, f16 b)
 }
 
 // Q8: scale u8 + per-column meta, zero u8 + whole-tensor meta; else fp16 tables.  XMODE 1: x = silu(xa) * xb
-template <int MT, bool Q8, int XMODE>
+// S: slabs per wave (1 or 2)
+template <int MT, bool Q8, int XMODE, int S>
 __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
 {
     constexpr int NT = kW3Waves * 64;
@@ -137,112 +138,114 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
         for (int m = 0; m < MT; ++m)
             acc[i][m] = zacc[i][m] = 0.f;
 
-    const int slab_lo = kb * p.SB + wave * p.S;
+    const int slab_lo = kb * p.SB + wave * S;
     int slab_hi = (kb + 1) * p.SB;
     if (slab_hi > p.NS)
         slab_hi = p.NS;
 
-    for (int sl = 0; sl < p.S; ++sl) {
-        const int slab = slab_lo + sl;
-        if (wave >= p.KS || slab >= slab_hi)
-            break;
-        const uint32_t k0 = (uint32_t)slab * kSlab;
-        // Every load of the slab is issued before any of its arithmetic, in the order the arithmetic needs them
-        // (loads retire in issue order): zero meta, tables, x, codes.
-        // Whole-tensor meta of the zero table: the address is the same in every lane but written so that the
-        // compiler does not see it (lane >> 6 is zero): a load it knows to be uniform is moved to scalar registers
-        // at once, which waits for it before any weight load has been issued.
-        uint32_t zms_raw = 0, zmz_raw = 0;
-        if constexpr (Q8) {
-            zms_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_ms) + (lane >> 6));
-            zmz_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_mz) + (lane >> 6));
-        }
-        // ------------------------------------------------------------ loads: tables and x (lane l: columns 4l..4l+3), codes
+    // What a slab's table phase reads: tables, their per-column meta, the zero table's whole-tensor meta, x.
+    struct Tab {
         uint32_t sraw[10][2], zraw[10][2];
         u32x2 msr[10], mzr[10];
+        u32x2 xr[MT], xg[XMODE ? MT : 1];
+        uint32_t zms_raw, zmz_raw;
+    };
+    // Every load of a slab is issued in the order the arithmetic needs them (loads retire in issue order): zero meta,
+    // tables, x, then the codes.  Whole-tensor meta of the zero table: the address is the same in every lane but
+    // written so that the compiler does not see it (lane >> 6 is zero): a load it knows to be uniform is moved to
+    // scalar registers at once, which waits for it before any weight load has been issued.
+    auto load_tab = [&](Tab &T, int slab) __attribute__((always_inline)) {
+        const uint32_t k0 = (uint32_t)slab * kSlab;
+        T.zms_raw = T.zmz_raw = 0;
+        if constexpr (Q8) {
+            T.zms_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_ms) + (lane >> 6));
+            T.zmz_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_mz) + (lane >> 6));
+        }
 #pragma unroll
         for (int i = 0; i < 10; ++i) {
             uint32_t j = j0 + (uint32_t)i; // (10*w0 + i) mod G; G >= 10
             j -= j >= (uint32_t)p.G ? (uint32_t)p.G : 0u;
             const uint32_t ce = j * (uint32_t)K + k0 + (uint32_t)(4 * lane);
             if constexpr (Q8) {
-                sraw[i][0] = gload<uint32_t>(R.sq + ce);
-                zraw[i][0] = gload<uint32_t>(R.zq + ce);
+                T.sraw[i][0] = gload<uint32_t>(R.sq + ce);
+                T.zraw[i][0] = gload<uint32_t>(R.zq + ce);
                 uint32_t cm = ce - __umulhi(ce, R.s_inv) * R.s_cols; // ce mod cols; the quotient estimate is at most 2 short
                 cm -= cm >= R.s_cols ? R.s_cols : 0;
                 cm -= cm >= R.s_cols ? R.s_cols : 0;
-                msr[i] = gload<u32x2>(R.s_ms + cm);
-                mzr[i] = gload<u32x2>(R.s_mz + cm);
+                T.msr[i] = gload<u32x2>(R.s_ms + cm);
+                T.mzr[i] = gload<u32x2>(R.s_mz + cm);
             } else {
                 const u32x2 a = gload<u32x2>(reinterpret_cast<const f16 *>(R.sq) + ce);
                 const u32x2 b = gload<u32x2>(reinterpret_cast<const f16 *>(R.zq) + ce);
-                sraw[i][0] = a.x, sraw[i][1] = a.y, zraw[i][0] = b.x, zraw[i][1] = b.y;
+                T.sraw[i][0] = a.x, T.sraw[i][1] = a.y, T.zraw[i][0] = b.x, T.zraw[i][1] = b.y;
             }
         }
-        u32x2 xr[MT], xg[XMODE ? MT : 1];
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             const uint32_t at = (uint32_t)((m < M ? m : 0) * K) + k0 + (uint32_t)(4 * lane);
             if constexpr (XMODE) {
-                xg[m] = gload<u32x2>(p.xa + (int64_t)layer * p.x_lstride + at);
-                xr[m] = gload<u32x2>(p.xb + (int64_t)layer * p.x_lstride + at);
+                T.xg[m] = gload<u32x2>(p.xa + (int64_t)layer * p.x_lstride + at);
+                T.xr[m] = gload<u32x2>(p.xb + (int64_t)layer * p.x_lstride + at);
             } else {
-                xr[m] = gload<u32x2>(p.x + at);
+                T.xr[m] = gload<u32x2>(p.x + at);
             }
         }
-        u32x4 cw[16];
+    };
+    auto load_codes = [&](u32x4(&cw)[16], int slab) __attribute__((always_inline)) {
 #pragma unroll
         for (int m = 0; m < 16; ++m)
-            cw[m] = gload<u32x4>(R.codes + (code_base + 4u * k0 + (uint32_t)(64 * m)));
-        __builtin_amdgcn_sched_barrier(0); // nothing below moves above the loads, no load sinks into the arithmetic
-        if constexpr (Q8) // the meta values become opaque here, so no use of them is hoisted above the loads
-            asm volatile("" : "+v"(zms_raw), "+v"(zmz_raw));
-
-        // ------------------------------------------------------------ table phase: xs into LDS, zero term accumulated
-        if constexpr (XMODE) {
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                const f16x2 a01 = as_h2(xg[m].x), a23 = as_h2(xg[m].y), b01 = as_h2(xr[m].x), b23 = as_h2(xr[m].y);
-                xr[m].x = as_u32((f16x2){silu_mul(a01.x, b01.x), silu_mul(a01.y, b01.y)});
-                xr[m].y = as_u32((f16x2){silu_mul(a23.x, b23.x), silu_mul(a23.y, b23.y)});
-            }
-        }
-        {
-            const f16x2 k1024 = {(f16)1024.0f, (f16)1024.0f};
-            const f16x2 k32 = {(f16)kXsScale, (f16)kXsScale};
-            const f16x2 zms = as_h2(zms_raw * 0x10001u), zmz = as_h2(zmz_raw * 0x10001u);
-#pragma unroll
-            for (int i = 0; i < 10; ++i) {
-                f16x2 s01, s23, z01, z23;
-                if constexpr (Q8) {
-                    // bytes -> fp16 exactly (0x6400 | b is 1024 + b), then fp16(fp16(q - mz) * ms) as the reference does
-                    const f16x2 q01 = as_h2(__builtin_amdgcn_perm(0x64646464u, sraw[i][0], 0x04010400u)) - k1024;
-                    const f16x2 q23 = as_h2(__builtin_amdgcn_perm(0x64646464u, sraw[i][0], 0x04030402u)) - k1024;
-                    s01 = (q01 - as_h2(mzr[i].x)) * as_h2(msr[i].x);
-                    s23 = (q23 - as_h2(mzr[i].y)) * as_h2(msr[i].y);
-                    const f16x2 y01 = as_h2(__builtin_amdgcn_perm(0x64646464u, zraw[i][0], 0x04010400u)) - k1024;
-                    const f16x2 y23 = as_h2(__builtin_amdgcn_perm(0x64646464u, zraw[i][0], 0x04030402u)) - k1024;
-                    z01 = (y01 - zmz) * zms;
-                    z23 = (y23 - zmz) * zms;
-                } else {
-                    s01 = as_h2(sraw[i][0]), s23 = as_h2(sraw[i][1]);
-                    z01 = as_h2(zraw[i][0]), z23 = as_h2(zraw[i][1]);
-                }
-                s01 = s01 * k32, s23 = s23 * k32;
-#pragma unroll
-                for (int m = 0; m < MT; ++m) {
-                    const f16x2 a01 = s01 * as_h2(xr[m].x), a23 = s23 * as_h2(xr[m].y);
-                    zacc[i][m] = __builtin_amdgcn_fdot2(z01, a01, zacc[i][m], false);
-                    zacc[i][m] = __builtin_amdgcn_fdot2(z23, a23, zacc[i][m], false);
-                    *reinterpret_cast<f16x4 *>(&xs_lds[wave][lane][m][i][0]) = (f16x4){a01.x, a01.y, a23.x, a23.y};
-                }
-            }
-        }
+            cw[m] = gload<u32x4>(R.codes + (code_base + 4u * ((uint32_t)slab * kSlab) + (uint32_t)(64 * m)));
+    };
+    auto wave_sync = [&]() __attribute__((always_inline)) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-        // ------------------------------------------------------------ codes: per pair of words and field, perm + and + dot2
+    };
+    // table phase: xs into LDS, zero term accumulated
+    auto table_phase = [&](Tab &T) __attribute__((always_inline)) {
+        if constexpr (Q8) // the meta values become opaque here, so no use of them is hoisted above the loads
+            asm volatile("" : "+v"(T.zms_raw), "+v"(T.zmz_raw));
+        if constexpr (XMODE) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const f16x2 a01 = as_h2(T.xg[m].x), a23 = as_h2(T.xg[m].y), b01 = as_h2(T.xr[m].x), b23 = as_h2(T.xr[m].y);
+                T.xr[m].x = as_u32((f16x2){silu_mul(a01.x, b01.x), silu_mul(a01.y, b01.y)});
+                T.xr[m].y = as_u32((f16x2){silu_mul(a23.x, b23.x), silu_mul(a23.y, b23.y)});
+            }
+        }
+        const f16x2 k1024 = {(f16)1024.0f, (f16)1024.0f};
+        const f16x2 k32 = {(f16)kXsScale, (f16)kXsScale};
+        const f16x2 zms = as_h2(T.zms_raw * 0x10001u), zmz = as_h2(T.zmz_raw * 0x10001u);
+#pragma unroll
+        for (int i = 0; i < 10; ++i) {
+            f16x2 s01, s23, z01, z23;
+            if constexpr (Q8) {
+                // bytes -> fp16 exactly (0x6400 | b is 1024 + b), then fp16(fp16(q - mz) * ms) as the reference does
+                const f16x2 q01 = as_h2(__builtin_amdgcn_perm(0x64646464u, T.sraw[i][0], 0x04010400u)) - k1024;
+                const f16x2 q23 = as_h2(__builtin_amdgcn_perm(0x64646464u, T.sraw[i][0], 0x04030402u)) - k1024;
+                s01 = (q01 - as_h2(T.mzr[i].x)) * as_h2(T.msr[i].x);
+                s23 = (q23 - as_h2(T.mzr[i].y)) * as_h2(T.msr[i].y);
+                const f16x2 y01 = as_h2(__builtin_amdgcn_perm(0x64646464u, T.zraw[i][0], 0x04010400u)) - k1024;
+                const f16x2 y23 = as_h2(__builtin_amdgcn_perm(0x64646464u, T.zraw[i][0], 0x04030402u)) - k1024;
+                z01 = (y01 - zmz) * zms;
+                z23 = (y23 - zmz) * zms;
+            } else {
+                s01 = as_h2(T.sraw[i][0]), s23 = as_h2(T.sraw[i][1]);
+                z01 = as_h2(T.zraw[i][0]), z23 = as_h2(T.zraw[i][1]);
+            }
+            s01 = s01 * k32, s23 = s23 * k32;
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const f16x2 a01 = s01 * as_h2(T.xr[m].x), a23 = s23 * as_h2(T.xr[m].y);
+                zacc[i][m] = __builtin_amdgcn_fdot2(z01, a01, zacc[i][m], false);
+                zacc[i][m] = __builtin_amdgcn_fdot2(z23, a23, zacc[i][m], false);
+                *reinterpret_cast<f16x4 *>(&xs_lds[wave][lane][m][i][0]) = (f16x4){a01.x, a01.y, a23.x, a23.y};
+            }
+        }
+        wave_sync();
+    };
+    // codes: per pair of words and field, perm + and + dot2
+    auto code_phase = [&](const u32x4(&cw)[16]) __attribute__((always_inline)) {
 #pragma unroll
         for (int m = 0; m < 16; ++m) {
             const int q = 4 * m + c;
@@ -268,9 +271,46 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
                 }
             }
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        wave_sync();
+    };
+
+    if (wave < p.KS && slab_lo < slab_hi) {
+        Tab T;
+        u32x4 c0[16];
+        load_tab(T, slab_lo);
+        load_codes(c0, slab_lo);
+        __builtin_amdgcn_sched_barrier(0); // nothing below moves above the loads, no load sinks into the arithmetic
+        table_phase(T);
+        if constexpr (S == 2 && MT == 1) {
+            // The second slab's loads go out before the first slab's codes are worked on (unconditionally: a wave
+            // whose second slab lies past its range re-reads the first and skips the arithmetic), its tables into
+            // the registers the first slab's table phase has just released.
+            const bool two = slab_lo + 1 < slab_hi;
+            const int s1 = two ? slab_lo + 1 : slab_lo;
+            u32x4 c1[16];
+            load_tab(T, s1);
+            load_codes(c1, s1);
+            __builtin_amdgcn_sched_barrier(0);
+            code_phase(c0);
+            if (two) {
+                table_phase(T);
+                code_phase(c1);
+            }
+        } else if constexpr (S == 2) {
+            // two batch rows leave no registers for a second set of codes: one slab after the other
+            code_phase(c0);
+            const bool two = slab_lo + 1 < slab_hi;
+            const int s1 = two ? slab_lo + 1 : slab_lo;
+            load_tab(T, s1);
+            load_codes(c0, s1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (two) {
+                table_phase(T);
+                code_phase(c0);
+            }
+        } else {
+            code_phase(c0);
+        }
     }
 
     // ---------------------------------------------------------------- wave result: sum over the column lanes, zero term removed
@@ -433,12 +473,20 @@ struct W3Job {
     SmallBatchEpilogue ep;
 };
 
-template <int MT, bool Q8> void launch_xmode(const W3Params &p, bool fused, dim3 grid, hipStream_t s)
+template <int MT, bool Q8, int S> void launch_slabs(const W3Params &p, bool fused, dim3 grid, hipStream_t s)
 {
     if (fused)
-        gemv_w3_kernel<MT, Q8, 1><<<grid, dim3(kW3Waves * 64), 0, s>>>(p);
+        gemv_w3_kernel<MT, Q8, 1, S><<<grid, dim3(kW3Waves * 64), 0, s>>>(p);
     else
-        gemv_w3_kernel<MT, Q8, 0><<<grid, dim3(kW3Waves * 64), 0, s>>>(p);
+        gemv_w3_kernel<MT, Q8, 0, S><<<grid, dim3(kW3Waves * 64), 0, s>>>(p);
+}
+
+template <int MT, bool Q8> void launch_xmode(const W3Params &p, bool fused, dim3 grid, hipStream_t s)
+{
+    if (p.S == 2)
+        launch_slabs<MT, Q8, 2>(p, fused, grid, s);
+    else
+        launch_slabs<MT, Q8, 1>(p, fused, grid, s);
 }
 
 size_t job_workspace_bytes(const W3Plan &pl, const hqq_linear *l, int NL)
