@@ -9,14 +9,18 @@ pytestmark = pytest.mark.gpu
 
 
 def _small_setup(layers=2, hidden=256, ffn=512, experts=8, vocab=128, offload_per_layer=6, main_per_layer=2,
-                 buffers=2, seed=0):
+                 buffers=2, seed=0, ffn_bits=2):
     from mixtral_offloading_amd import build_model as bm
+    from mixtral_offloading_amd.hqq_core import BaseQuantizeConfig
     cfg = bm.mixtral_config(hidden_size=hidden, intermediate_size=ffn, num_hidden_layers=layers, num_attention_heads=4,
                             num_key_value_heads=2, vocab_size=vocab, num_local_experts=experts)
     off = bm.OffloadConfig(main_size=layers * main_per_layer, offload_size=layers * offload_per_layer,
                            buffer_size=buffers, offload_per_layer=offload_per_layer)
-    model = bm.build_model(torch.device("cuda:0"), bm.default_quant_config(), off, model_config=cfg, seed=seed,
-                           max_positions=256)
+    qc = bm.default_quant_config()
+    if ffn_bits != 2:
+        qc = bm.QuantConfig(ffn_config=BaseQuantizeConfig(nbits=ffn_bits, group_size=64, quant_zero=True, quant_scale=True),
+                            attn_config=qc.attn_config)
+    model = bm.build_model(torch.device("cuda:0"), qc, off, model_config=cfg, seed=seed, max_positions=256)
     return model, cfg
 
 
@@ -144,10 +148,15 @@ def test_cache_error_paths():
         c.add_expert((0, 100), c.slots[0], eviction_group=0, offload=True)
 
 
-def test_generate_offloaded_equals_resident():
-    """Greedy decoding with a 2-expert cache per layer gives the same tokens as with every expert resident."""
-    model_off, cfg = _small_setup(layers=2, offload_per_layer=6, main_per_layer=2, buffers=2, seed=11)
-    model_res, _ = _small_setup(layers=2, offload_per_layer=0, main_per_layer=8, buffers=1, seed=11)
+@pytest.mark.parametrize("ffn_bits,hidden,ffn", [(2, 256, 512), (3, 256, 512), (3, 1024, 1280), (4, 256, 512)])
+def test_generate_offloaded_equals_resident(ffn_bits, hidden, ffn):
+    """Greedy decoding with a 2-expert cache per layer gives the same tokens as with every expert resident (2-, 3- and
+    4-bit experts; 3-bit ones at a size the decode kernel does not take, which run on the general kernel, and at one
+    it does)."""
+    model_off, cfg = _small_setup(layers=2, hidden=hidden, ffn=ffn, offload_per_layer=6, main_per_layer=2, buffers=2, seed=11,
+                                  ffn_bits=ffn_bits)
+    model_res, _ = _small_setup(layers=2, hidden=hidden, ffn=ffn, offload_per_layer=0, main_per_layer=8, buffers=1, seed=11,
+                                ffn_bits=ffn_bits)
     prompt = torch.randint(0, cfg.vocab_size, (9,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(2))
     a = model_off.generate(prompt, 12)
     b = model_res.generate(prompt, 12)
