@@ -346,6 +346,12 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
     }
     if (!row_scale_f16 && !accumulate)
         return run_matmul(w2, h, M, y, mm, mm_bytes, pick_family(w2, M), s);
+    if (pick_family(w2, M) == FAM_TILE && tile_epilogue_supported(w2, M)) {
+        SmallBatchEpilogue ep; // the routing weight and the accumulation in the matmul's own epilogue
+        ep.row_scale = (const f16 *)row_scale_f16;
+        ep.accumulate = accumulate;
+        return launch_tile_matmul(w2, h, M, y, mm, mm_bytes, s, &ep);
+    }
     if ((rc = run_matmul(w2, h, M, t, mm, mm_bytes, pick_family(w2, M), s)) != HQQ_OK)
         return rc;
     return launch_scale_store(t, y, (const f16 *)row_scale_f16, accumulate, M, w2->N, s);

@@ -48,6 +48,9 @@ struct TileParams {
     uint32_t sc_b_inv;
     int JB;
     int64_t part_lstride;
+    // pipelined kernel and its finishing pass only: y = o (+ bias) (* row_scale[m]) (+ y), each step rounded to fp16
+    const f16 *row_scale;
+    int accumulate;
 };
 
 template <int NBITS> struct WField {
@@ -550,13 +553,17 @@ __global__ __launch_bounds__(JW * NFW * KW * 64) void gemm_tile2_kernel(TilePara
                 continue;
             }
             f16 o[FW];
+            f16 *dst = p.y + (int64_t)m * p.N + n;
 #pragma unroll
             for (int i = 0; i < FW; ++i) {
                 o[i] = (f16)acc[i][b][v];
                 if (p.bias)
                     o[i] = o[i] + p.bias[n + i];
+                if (p.row_scale)
+                    o[i] = o[i] * p.row_scale[m];
+                if (p.accumulate)
+                    o[i] = dst[i] + o[i];
             }
-            f16 *dst = p.y + (int64_t)m * p.N + n;
             if constexpr (FW == 4)
                 *reinterpret_cast<f16x4 *>(dst) = (f16x4){o[0], o[1], o[2], o[3]};
             else if constexpr (FW == 2)
@@ -574,7 +581,8 @@ __global__ __launch_bounds__(JW * NFW * KW * 64) void gemm_tile2_kernel(TilePara
 template <int F, bool GATE>
 __global__ __launch_bounds__(256) void tile_finish_kernel(const float *__restrict__ part, int KSP, int M, int N,
                                                            const f16 *__restrict__ bias, f16 *__restrict__ y,
-                                                           int64_t lstride)
+                                                           int64_t lstride, const f16 *__restrict__ row_scale,
+                                                           int accumulate)
 {
     __shared__ f16 t_lds[16][16][F];
     const int NG = N / F;
@@ -604,6 +612,8 @@ __global__ __launch_bounds__(256) void tile_finish_kernel(const float *__restric
                 } else if (bias) {
                     v = v + bias[F * g + i];
                 }
+                if (row_scale)
+                    v = v * row_scale[m];
                 t_lds[threadIdx.x & 15][gl][i] = v;
             }
         }
@@ -615,7 +625,7 @@ __global__ __launch_bounds__(256) void tile_finish_kernel(const float *__restric
             f16 *dst = y + (int64_t)m * N + F * g;
 #pragma unroll
             for (int i = 0; i < F; ++i)
-                dst[i] = t_lds[threadIdx.x >> 4][gl][i];
+                dst[i] = accumulate ? (f16)(dst[i] + t_lds[threadIdx.x >> 4][gl][i]) : t_lds[threadIdx.x >> 4][gl][i];
         }
     }
 }
@@ -834,7 +844,7 @@ static size_t tile_job_bytes(const hqq_linear *l, int64_t M, int nl)
 
 // one layer (lb == nullptr) or the two projections of a gate: y = x W^T (+ bias), or y = silu(x Wa^T) * (x Wb^T)
 static int tile_job(const hqq_linear *la, const hqq_linear *lb, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
-                    hipStream_t s)
+                    hipStream_t s, const SmallBatchEpilogue *ep = nullptr)
 {
     const int nl = lb ? 2 : 1;
     TilePlan pl;
@@ -842,6 +852,9 @@ static int tile_job(const hqq_linear *la, const hqq_linear *lb, const f16 *x, in
     if (!make_plan(&view[0], M, pl, nl) || (reinterpret_cast<uintptr_t>(x) & 15u))
         return HQQ_E_UNSUPPORTED;
     if (nl == 2 && pl.kinds == 0)
+        return HQQ_E_UNSUPPORTED;
+    const bool scaled = ep && (ep->row_scale || ep->accumulate);
+    if (scaled && (pl.kinds == 0 || nl == 2))
         return HQQ_E_UNSUPPORTED;
     const size_t need = tile_job_bytes(la, M, nl);
     if (need > 0 && (!ws || ws_bytes < need))
@@ -873,6 +886,7 @@ static int tile_job(const hqq_linear *la, const hqq_linear *lb, const f16 *x, in
     p.x = x, p.bias = nl == 1 ? static_cast<const f16 *>(l->bias) : nullptr, p.y = y;
     p.M = (int)M, p.N = (int)l->N, p.K = (int)l->K, p.GP = pl.GP, p.KT = pl.KT;
     p.KSP = pl.KSP, p.KTS = pl.KTS;
+    p.row_scale = scaled ? ep->row_scale : nullptr, p.accumulate = scaled ? ep->accumulate : 0;
     p.part = partial ? reinterpret_cast<float *>(body) : nullptr;
     // blocks along x: packed rows (per projection, unless a block holds both) by K blocks
     const int jrows = pl.JW == 2 ? pl.GP : pl.GP / pl.JW * nl;
@@ -900,22 +914,31 @@ static int tile_job(const hqq_linear *la, const hqq_linear *lb, const f16 *x, in
     const dim3 fgrid((unsigned)((l->N / pl.F + 15) / 16), (unsigned)((M + 15) / 16));
     if (nl == 2) {
         if (pl.F == 4)
-            tile_finish_kernel<4, true><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, nullptr, y, p.part_lstride);
+            tile_finish_kernel<4, true><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, nullptr, y, p.part_lstride, nullptr, 0);
         else
-            tile_finish_kernel<2, true><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, nullptr, y, p.part_lstride);
+            tile_finish_kernel<2, true><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, nullptr, y, p.part_lstride, nullptr, 0);
     } else if (pl.F == 4) {
-        tile_finish_kernel<4, false><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, p.bias, y, 0);
+        tile_finish_kernel<4, false><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, p.bias, y, 0, p.row_scale, p.accumulate);
     } else {
-        tile_finish_kernel<2, false><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, p.bias, y, 0);
+        tile_finish_kernel<2, false><<<fgrid, 256, 0, s>>>(p.part, pl.KSP, (int)M, (int)l->N, p.bias, y, 0, p.row_scale, p.accumulate);
     }
     return launch_status();
 }
 
 size_t tile_workspace_bytes(const hqq_linear *l, int64_t M) { return tile_job_bytes(l, M, 1); }
 
-int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s)
+int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s,
+                       const SmallBatchEpilogue *ep)
 {
-    return tile_job(l, nullptr, x, M, y, ws, ws_bytes, s);
+    return tile_job(l, nullptr, x, M, y, ws, ws_bytes, s, ep);
+}
+
+// whether the routing weight and the accumulation can ride in the matmul's own epilogue
+bool tile_epilogue_supported(const hqq_linear *l, int64_t M)
+{
+    TilePlan pl;
+    const hqq_linear v = tile_view(l);
+    return tile_supported(l, M) && make_plan(&v, M, pl) && pl.kinds != 0;
 }
 
 // the two projections of an expert's gate in one launch, silu(a) * b applied by the finishing kernel

@@ -171,7 +171,9 @@ int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s);
 size_t workspace_head_bytes();
 bool tile_supported(const hqq_linear *l, int64_t M);
 size_t tile_workspace_bytes(const hqq_linear *l, int64_t M);
-int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s);
+int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s,
+                       const SmallBatchEpilogue *ep = nullptr);
+bool tile_epilogue_supported(const hqq_linear *l, int64_t M);
 bool tile_gate_supported(const hqq_linear *w1, const hqq_linear *w3, int64_t M);
 size_t tile_gate_workspace_bytes(const hqq_linear *w1, const hqq_linear *w3, int64_t M);
 int launch_tile_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,

@@ -56,7 +56,7 @@ def test_expert_ffn_against_oracle(shape, m):
 
 
 @pytest.mark.parametrize("nbits,hidden,ffn,gs", [(2, 512, 1792, 16), (3, 768, 1280, 64)])
-@pytest.mark.parametrize("m", [1, 2, 3, 4])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 8, 40, 130])
 def test_expert_ffn_row_scale_and_accumulate(m, nbits, hidden, ffn, gs):
     """Routing weight and the index_add_ of the reference (src/custom_layers.py:308-312) as the FFN's epilogue."""
     from mixtral_offloading_amd import hip_kernels
