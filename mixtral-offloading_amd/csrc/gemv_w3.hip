@@ -14,7 +14,8 @@
 // multiplies exactly and accumulates in fp32.  The table phase (lane l owns columns 4l .. 4l+3 of all ten rows)
 // leaves xs in LDS; the zero term is a dot product per table row, summed over the wave at the end.
 //
-// The waves of a block split K (two slabs each); when K needs several blocks (or the window count alone would leave
+// The waves of a block split K (one or two slabs each; with two, the second slab's loads are in flight while the
+// first slab's codes are worked on); when K needs several blocks (or the window count alone would leave
 // most of the chip idle) the blocks of a tile add their results into one 64-bit fixed-point accumulation slot per
 // output with a returning device-scope atomic, and the block whose addition completes a slot writes that output
 // (launches with more outputs than there are slots store fp32 partial sums instead, and the block that arrives
