@@ -216,3 +216,22 @@ def test_workspace_init_makes_a_dirty_workspace_usable():
                        "hqq_matmul_transpose")
             assert_matmul_close(y.cpu().numpy(), o.matmul_transpose(x, layer), o.matmul_tolerance(x, layer))
         assert not bool(ws[: 576 * 1024].any())
+
+
+@pytest.mark.parametrize("nbits,n,k,gs", [(4, 6144, 6144, 64), (4, 1024, 6144, 64), (2, 16384, 6144, 16),
+                                          (2, 6144, 16384, 16), (3, 16384, 6144, 64), (3, 6144, 16384, 64)])
+@pytest.mark.parametrize("m", [1, 2, 4, 16, 64])
+def test_other_model_shapes_against_dequantize_then_matmul(nbits, n, k, gs, m):
+    """The projections of Mixtral-8x22B (hidden 6144, ffn 16384): shapes the launch planners were not tuned on."""
+    from mixtral_offloading_amd import hip_kernels
+    desc = _full_size_layer(nbits, n, k, gs, seed=n + k + nbits)
+    g = torch.Generator(device="cuda").manual_seed(m)
+    x = torch.randn((m, k), device="cuda", generator=g).half()
+    w = hip_kernels.dequantize(desc).float()
+    ref = (x.float() @ w.t())
+    for rep in range(2):
+        y = hip_kernels.matmul(desc, x)
+        atol = 1e-3 * x.float().norm(dim=1)[:, None] * w.norm(dim=1)[None, :]
+        err = (y.float() - ref).abs()
+        bound = 1e-2 * ref.abs() + atol + ref.abs() * 2.0 ** -11
+        assert bool((err <= bound).all()), float((err / bound).max())
