@@ -247,8 +247,8 @@ def test_matmul_group_refuses_mixed_layers():
     assert not hip_kernels.LinearGroup([desc_of(a), desc_of(b)]).supported
 
 
-@pytest.mark.parametrize("ffn_bits", [2, 3])
-def test_graph_decode_matches_eager_logits(ffn_bits):
+@pytest.mark.parametrize("ffn_bits,wide", [(2, False), (3, False), (2, True)])
+def test_graph_decode_matches_eager_logits(ffn_bits, wide):
     """Each replayed step must give the logits of the eager forward at the same position (same kernels for the
     quantized linears; attention over the masked full cache instead of the sliced one).  With 3-bit experts the
     step takes the norm + router launch and the three-launch expert pair instead of the routed pair."""
@@ -256,7 +256,10 @@ def test_graph_decode_matches_eager_logits(ffn_bits):
     from mixtral_offloading_amd.hqq_core import BaseQuantizeConfig
     from mixtral_offloading_amd.mixtral_model import DecodeGraph
     qc = bm.default_quant_config()
-    if ffn_bits == 2:
+    if wide:  # a row longer than the routed launch takes: norm + router in a launch of their own, then the pair
+        cfg = bm.mixtral_config(hidden_size=5120, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=40,
+                                num_key_value_heads=8, vocab_size=128, num_local_experts=4)
+    elif ffn_bits == 2:
         cfg = bm.mixtral_config(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
                                 num_key_value_heads=2, vocab_size=128, num_local_experts=8)
     else:
@@ -264,12 +267,12 @@ def test_graph_decode_matches_eager_logits(ffn_bits):
                                 num_key_value_heads=2, vocab_size=128, num_local_experts=8)
         qc = bm.QuantConfig(ffn_config=BaseQuantizeConfig(nbits=3, group_size=64, quant_zero=True, quant_scale=True),
                             attn_config=qc.attn_config)
-    off = bm.OffloadConfig(main_size=16, offload_size=0, buffer_size=1, offload_per_layer=0)
+    off = bm.OffloadConfig(main_size=2 * cfg.num_local_experts, offload_size=0, buffer_size=1, offload_per_layer=0)
     model = bm.build_model(torch.device("cuda:0"), qc, off, model_config=cfg, seed=5, max_positions=64)
     prompt = torch.randint(0, 128, (9,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(2))
     steps = 6
     dec = DecodeGraph(model, prompt.numel() + steps + 4)
-    assert dec.pair and dec.routed == (ffn_bits == 2)
+    assert dec.pair and dec.routed == (ffn_bits == 2 and not wide)
     first = dec.prefill(prompt)
     dec.capture()
     # eager reference driven with the graph's own tokens
