@@ -384,7 +384,7 @@ def main():
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this command, scaled by a
                      # 256 MiB copy (profiles/gemv_strip_kernel_ffn_2bit_g16_m1.txt); measured at batch 1 only
-                     "traffic": 46305081 if m == 1 else None,
+                     "traffic": 46320457 if m == 1 else None,
                      "kernel": "gemv_strip_kernel<2,1,4,2,8,1,2,1,false,0> as launched by hqq_gate_up (w1 and w3 in one grid, one launch)",
                      "bytes_per_launch": gate_up_bytes(m), "us_per_launch": round(ms_gate * 1e3, 3)},
     }
