@@ -18,6 +18,9 @@
 // Mixtral shape) instead stores fp32 partial sums with device-scope stores, and the block that arrives last at the
 // tile's counter adds them in a fixed order.
 //
+// A gate of three or four rows whose blocks hold all of K is launched as two passes of the two-row kernel (batch
+// rows 0-1 and 2-3) in one grid, the two passes of a tile next to each other in launch order.
+//
 // Lane roles inside a slab.  Code lanes: (rr = lane & 15, kg = lane >> 4) own packed row jp + (16*rb + rr)*GP,
 // bytes 64*s + 16*kg .. +15 for step s.  Table lanes: (ti = lane >> 4 < F, kq = lane & 15) own table row F*jp + ti,
 // columns 16*kq .. 16*kq+15, i.e. step kq >> 2, MFMA lane group kq & 3.
@@ -59,6 +62,7 @@ struct StripParams {
     const f16 *x;
     int x_lstride; // layer l reads x + l * x_lstride (0: every layer reads the same activations)
     int M, K;
+    int passes; // 2 (two-row kernel only): the launch holds every tile twice, the second copy working on batch rows 2, 3
     int RB;
     int NS;       // K / 256
     int KS;       // waves per layer in a block
@@ -132,11 +136,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     // registers, and the record is picked from the kernel arguments without a memory access of its own
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kb = blockIdx.x, rb = blockIdx.y;
+    // Batches of three and four rows run as two passes of the two-row kernel inside one launch: blocks 2z and 2z + 1
+    // are the two passes of tile z, so both ask for the tile's weights at about the same time and memory delivers
+    // them once (how far apart the two are in launch order, 1 to 32 workgroups, made no difference when measured).
+    int bz = (int)blockIdx.z, pass = 0;
+    if constexpr (MT == 2) {
+        if (p.passes == 2) {
+            pass = bz & 1;
+            bz >>= 1;
+        }
+    }
     int g = 0;
     if constexpr (GROUPED) // absent groups begin at INT_MAX
-        g = ((int)blockIdx.z >= p.grp[1].z_begin) + ((int)blockIdx.z >= p.grp[2].z_begin) + ((int)blockIdx.z >= p.grp[3].z_begin);
+        g = (bz >= p.grp[1].z_begin) + (bz >= p.grp[2].z_begin) + (bz >= p.grp[3].z_begin);
     const StripGroup &Gd = p.grp[g]; // g is uniform: the record comes from the kernel arguments by scalar loads
-    const int jp = (int)blockIdx.z - Gd.z_begin;
+    const int jp = bz - Gd.z_begin;
     const int GP = Gd.GP, N = Gd.N;
     const int layer = wave >= p.KS ? 1 : 0;
     const int ks = wave - layer * p.KS;
@@ -208,7 +222,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     }
     const int slab0 = (kb * p.KS + ks) * S;
     const int K = p.K;
-    const int M = MT == 1 ? 1 : p.M;
+    const int M = MT == 1 ? 1 : (p.M - 2 * pass < MT ? p.M - 2 * pass : MT);
 
     const int rr = lane & 15, kg = lane >> 4;
     const int ti = lane >> 4, kq = lane & 15;
@@ -225,7 +239,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     const uint32_t crow = STAGE ? ((uint32_t)jp + (uint32_t)(16 * rb + lrow) * (uint32_t)GP) * (uint32_t)K + (uint32_t)(16 * lchunk)
                                 : ((uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)GP) * (uint32_t)K + (uint32_t)(16 * kg);
     const uint32_t crow_step = STAGE ? 4u * (uint32_t)GP * (uint32_t)K : 64u; // four tile rows further / next step
-    const f16 *xl = p.x + layer * p.x_lstride;
+    const f16 *xl = p.x + layer * p.x_lstride + pass * 2 * K;
 
     auto issue = [&](SlabRegs<MT, SKIND, ZKIND> &r, int slab) __attribute__((always_inline)) {
         const uint32_t k0 = (uint32_t)slab * kSlab;
@@ -507,7 +521,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
 
     // ---------------------------------------------------------------- block tile: 16 lanes per (layer, row, batch row)
     const bool alone = p.BK == 1;
-    const int tile = (int)blockIdx.z * p.RB + rb;
+    const int tile = bz * p.RB + rb;
+    f16 *const y_rows = Gd.y + (int64_t)pass * 2 * N; // the pass's first batch row
     for (int t = threadIdx.x; t < p.NL * 16 * MT * 16; t += WAVES * 64) {
         const int w = t & 15, u = t >> 4;
         const int l_t = u / (16 * MT), r_t = (u / MT) & 15, m_t = u % MT;
@@ -543,7 +558,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
             for (int i = 0; i < F; ++i)
                 dst[i] = o[i];
         } else {
-            f16 *dst = Gd.y + (int64_t)m_t * N + n;
+            f16 *dst = y_rows + (int64_t)m_t * N + n;
             f16 hv[F];
 #pragma unroll
             for (int i = 0; i < F; ++i) {
@@ -585,7 +600,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
                     continue;
                 const int r = 16 * rb + r_t;
                 const int64_t n = (int64_t)F * (jp + (int64_t)r * GP);
-                f16 *dst = Gd.y + (int64_t)m_t * N + n;
+                f16 *dst = y_rows + (int64_t)m_t * N + n;
                 f16 hv[F];
 #pragma unroll
                 for (int i = 0; i < F; ++i) {
@@ -632,7 +647,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
                     if (p.row_scale)
                         val = val * p.row_scale[m_t];
                 }
-                f16 *dst = Gd.y + (int64_t)m_t * N + n;
+                f16 *dst = y_rows + (int64_t)m_t * N + n;
                 *dst = p.accumulate ? (f16)(*dst + val) : val;
             }
             return;
@@ -673,7 +688,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
                     b[i] += __hip_atomic_load(Gd.part[1] + off + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        f16 *dst = Gd.y + (int64_t)m_t * N + n;
+        f16 *dst = y_rows + (int64_t)m_t * N + n;
         f16 hv[F];
 #pragma unroll
         for (int i = 0; i < F; ++i) {
@@ -928,7 +943,13 @@ int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t
 {
     StripPlan pl, per_group[kMaxGroups];
     size_t part_bytes = 0;
-    if (!plan_job(j, M, pl, per_group, part_bytes))
+    // A gate of three or four rows whose blocks hold all of K runs as two passes of the two-row kernel in one launch.
+    int passes = 1;
+    if ((M == 3 || M == 4) && j.EPI == 1 && j.NL == 2 && j.NG == 1 && !j.norm_weight &&
+        !(tuning_overrides() && std::getenv("HQQ_STRIP_NOPASS")) && plan_job(j, 2, pl, per_group, part_bytes) &&
+        pl.BK == 1 && 2 * per_group[0].GP <= 65535)
+        passes = 2;
+    if (passes == 1 && !plan_job(j, M, pl, per_group, part_bytes))
         return HQQ_E_UNSUPPORTED;
     const bool alone = pl.BK == 1;
     if (!alone && (!ws || ws_bytes < kHeadBytes + part_bytes))
@@ -973,6 +994,7 @@ int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t
         p.sel_gstride = j.sel_gstride, p.sel_lstride = j.sel_lstride, p.first_lstride = j.first_lstride;
     }
     p.x = j.x, p.x_lstride = (int)j.x_lstride, p.M = (int)M, p.K = (int)j.shape[0]->K;
+    p.passes = passes;
     p.RB = pl.RB, p.NS = pl.NS, p.KS = pl.KS, p.BK = pl.BK, p.NL = j.NL;
     p.counter = reinterpret_cast<int *>(base);
     // plain or weighted-pair epilogue, K over at most eight blocks, every output of the launch has a slot: no
@@ -990,7 +1012,7 @@ int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t
         p.norm_delta = j.norm_delta, p.norm_weight = j.norm_weight, p.x_sum = j.x_sum, p.norm_eps = j.norm_eps;
         p.gate_w = j.gate_w, p.n_experts = j.n_experts, p.sel_out = j.sel_out, p.rw_out = j.rw_out;
     }
-    const dim3 grid((unsigned)pl.BK, (unsigned)pl.RB, (unsigned)z);
+    const dim3 grid((unsigned)pl.BK, (unsigned)pl.RB, (unsigned)(z * passes));
     const bool two = j.shape[0]->nbits == 2;
     if (j.NG > 1 || j.norm_weight) {
         if (j.EPI == 0 && j.NL == 1)

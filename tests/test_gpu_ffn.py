@@ -92,7 +92,7 @@ def test_ffn_entry_point_equals_its_three_steps(m, nbits, gs):
     assert err <= 2e-3 * steps.float().abs().max().item() + 1e-3, err
 
 
-@pytest.mark.parametrize("m", [1, 2, 4, 8, 16, 128])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 8, 16, 128])
 def test_full_size_ffn_against_dequantize_then_matmul(m):
     """Mixtral shapes (2-bit g16, 4096 -> 14336 -> 4096): the library's bit-exact de-quantiser followed by torch
     matmuls with the reference's fp16 roundings."""
