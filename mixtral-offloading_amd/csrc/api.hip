@@ -50,7 +50,7 @@ static int pick_family(const hqq_linear *l, int64_t M)
 {
     if (strip_supported(l, M)) // decode batches: part of the small-batch family
         return FAM_SMALLBATCH;
-    if (l->nbits == 3 && tile_supported(l, M)) // seven rows and more: 3-bit codes rewritten as 4-bit ones, then the tile kernel
+    if (l->nbits == 3 && tile_supported(l, M)) // five rows and more: 3-bit codes rewritten as 4-bit ones, then the tile kernel
         return FAM_TILE;
     if (vec3_supported(l, M))
         return FAM_VEC3;

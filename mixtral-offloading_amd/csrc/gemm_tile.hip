@@ -822,9 +822,9 @@ void launch_tile2(const TileParams &p, const TilePlan &pl, int nbits, dim3 grid,
 bool tile_supported(const hqq_linear *l, int64_t M)
 {
     TilePlan pl;
-    if (l->nbits == 3) { // below seven rows the 3-bit row kernel, run in passes of two rows, is faster than the rewrite
+    if (l->nbits == 3) { // up to four rows the 3-bit row kernel, run in passes of two rows, is faster than the rewrite
         const hqq_linear v = tile_view(l);
-        return M > 6 && l->N % 2 == 0 && l->K % 4 == 0 && aligned16(l->codes) && make_plan(&v, M, pl);
+        return M > 4 && l->N % 2 == 0 && l->K % 4 == 0 && aligned16(l->codes) && make_plan(&v, M, pl);
     }
     return M > 4 && make_plan(l, M, pl);
 }
