@@ -119,6 +119,18 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
                    void *y_f16, const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
                    void *stream);
 
+/* ---- hqq_expert_ffn for callers that cannot allocate or carry a workspace (code under HIP graph capture, tight
+ *      serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The workspace is an
+ *      array of HQQ_STATIC_SCRATCH_BYTES built into the library's device code (every GPU the library runs on holds it
+ *      until the process ends); the call allocates nothing and returns HQQ_E_WORKSPACE when
+ *      hqq_expert_ffn_workspace_bytes(w1, w2, w3, M) exceeds that size (Mixtral-8x7B experts: batches up to 4 rows at
+ *      any code width, up to 16 rows for 2-bit codes).  Results are hqq_expert_ffn's, bit for bit.  All calls on one
+ *      GPU share the array: calls that overlap in time on one GPU race (order them on one stream, or with events).
+ *      The first call on a GPU records one extra small fill kernel on `stream`.                                    */
+#define HQQ_STATIC_SCRATCH_BYTES ((size_t)16 << 20)
+int hqq_expert_ffn_static(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *x_f16, int64_t M,
+                          void *y_f16, const void *row_scale_f16, int accumulate, void *stream);
+
 /* ---- h = silu(w1 x) * (w3 x), fp16 (M, ffn): the first half of the expert FFN (src/custom_layers.py:254), both
  *      projections rounded to fp16 as the reference's two layers round them, SiLU in fp32 rounded once, the product in
  *      fp16.  One fused pass over both weight matrices where a kernel family has one for the batch (2- and 4-bit

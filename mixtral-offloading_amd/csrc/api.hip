@@ -2,6 +2,8 @@
 // kernel-family dispatch and workspace carving.
 #include "hqq_common.hpp"
 
+#include <mutex>
+
 namespace hqq {
 
 static int validate_table(const hqq_table &t)
@@ -355,6 +357,61 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
     if ((rc = run_matmul(w2, h, M, t, mm, mm_bytes, pick_family(w2, M), s)) != HQQ_OK)
         return rc;
     return launch_scale_store(t, y, (const f16 *)row_scale_f16, accumulate, M, w2->N, s);
+}
+
+// ---- the expert FFN for callers that cannot allocate.  The workspace is a file-scope device array; each GPU holds
+// its own copy at its own address, found once per device with hipGetSymbolAddress (the array's name is only a
+// host-side handle, never a device address).
+constexpr size_t kStaticScratchBytes = HQQ_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+static std::mutex scratch_mutex;
+static void *scratch_ptr[kMaxDevices]; // per device, null until the first call there
+
+// the device address of `scratch` on the current device; the first call on a device also clears the head
+// (counters and accumulation slots) with the fill kernel, on the caller's stream
+static int static_scratch(void **out, hipStream_t s)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return static_cast<int>(e);
+    if (dev < 0 || dev >= kMaxDevices)
+        return HQQ_E_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess)
+            return static_cast<int>(e);
+        if (!ptr || (reinterpret_cast<uintptr_t>(ptr) & 255u))
+            return HQQ_E_ALIGN;
+        const int rc = launch_zero_workspace_head(ptr, kStaticScratchBytes, s);
+        if (rc != HQQ_OK)
+            return rc;
+        scratch_ptr[dev] = ptr;
+    }
+    *out = scratch_ptr[dev];
+    return HQQ_OK;
+}
+
+int hqq_expert_ffn_static(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *x_f16, int64_t M,
+                          void *y_f16, const void *row_scale_f16, int accumulate, void *stream)
+{
+    int rc;
+    if ((rc = validate_linear(w1)) != HQQ_OK || (rc = validate_linear(w2)) != HQQ_OK ||
+        (rc = validate_linear(w3)) != HQQ_OK)
+        return rc;
+    if (M < 0 || w1->N != w3->N || w1->K != w3->K || w2->K != w1->N || w2->N != w1->K)
+        return HQQ_E_SHAPE;
+    if (M == 0)
+        return HQQ_OK;
+    if (hqq_expert_ffn_workspace_bytes(w1, w2, w3, M) > kStaticScratchBytes)
+        return HQQ_E_WORKSPACE; // beyond the built-in scratch: use hqq_expert_ffn with a workspace of the caller's
+    void *ws = nullptr;
+    if ((rc = static_scratch(&ws, (hipStream_t)stream)) != HQQ_OK)
+        return rc;
+    return hqq_expert_ffn(w1, w2, w3, x_f16, M, y_f16, row_scale_f16, accumulate, ws, kStaticScratchBytes, stream);
 }
 
 size_t hqq_expert_record_bytes(void) { return strip_record_bytes(); }

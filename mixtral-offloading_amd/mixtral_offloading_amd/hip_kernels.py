@@ -215,6 +215,25 @@ def expert_ffn(w1: LinearDesc, w2: LinearDesc, w3: LinearDesc, x: torch.Tensor, 
     return out
 
 
+STATIC_SCRATCH_BYTES = 16 << 20  # HQQ_STATIC_SCRATCH_BYTES of include/hqq_mi355x.h
+
+
+def expert_ffn_static(w1: LinearDesc, w2: LinearDesc, w3: LinearDesc, x: torch.Tensor, out: torch.Tensor,
+                      row_scale: Optional[torch.Tensor] = None, accumulate: bool = False) -> torch.Tensor:
+    """``expert_ffn`` on the library's built-in scratch: nothing is allocated, here or in the library, so ``out`` is
+    the caller's.  Raises ``HqqError`` (workspace) when the batch needs more than ``STATIC_SCRATCH_BYTES``."""
+    assert x.dtype == torch.float16 and x.is_contiguous() and x.shape[-1] == w1.K
+    M = x.numel() // w1.K
+    assert out.is_contiguous() and out.numel() == M * w2.N and out.dtype == torch.float16
+    assert row_scale is None or (row_scale.dtype == torch.float16 and row_scale.is_contiguous() and row_scale.numel() == M)
+    with _on(x.device):
+        _lib.check(_lib.lib.hqq_expert_ffn_static(w1.ref, w2.ref, w3.ref, x.data_ptr(), M, out.data_ptr(),
+                                                  row_scale.data_ptr() if row_scale is not None else None,
+                                                  int(accumulate), _lib.current_stream_ptr(x.device)),
+                   "hqq_expert_ffn_static")
+    return out
+
+
 def gate_up(w1: LinearDesc, w3: LinearDesc, x: torch.Tensor) -> torch.Tensor:
     """``silu(w1 x) * (w3 x)``, the first half of the expert FFN (reference src/custom_layers.py:254)."""
     assert x.dtype == torch.float16 and x.is_contiguous() and x.shape[-1] == w1.K == w3.K and w1.N == w3.N
