@@ -224,7 +224,8 @@ int hqq_add_rmsnorm_router(void *x_f16, const void *delta_f16, const void *weigh
  *      reference): q (n_heads*head_dim), k and v (n_kv_heads*head_dim) are the un-rotated projections of the token;
  *      cos / sin are tables [positions][head_dim]; pos[0] (device memory) is the token's position; the rotated key
  *      and the value are written to cache_k / cache_v [n_kv_heads][max_len][head_dim] at pos and positions 0..pos
- *      are attended.  out is (n_heads*head_dim).  head_dim 64 or 128; the caller keeps pos < max_len <= 16000.      */
+ *      are attended.  out is (n_heads*head_dim).  head_dim 64 or 128; the caller keeps pos < max_len <= 16000 and
+ *      cos / sin at least max_len rows long (pos is read on the device and bounded by max_len only).               */
 int hqq_attention_decode(const void *q_f16, const void *k_f16, const void *v_f16, const void *cos_f16, const void *sin_f16,
                          const int64_t *pos, void *cache_k_f16, void *cache_v_f16, int64_t max_len, int32_t n_heads,
                          int32_t n_kv_heads, int32_t head_dim, void *out_f16, void *stream);

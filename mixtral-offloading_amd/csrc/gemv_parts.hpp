@@ -14,25 +14,36 @@ constexpr float kXsScale = 32.0f;    // xs = 32 * s * x keeps small activations 
 constexpr size_t kCounterBytes = 64 * 1024;
 constexpr size_t kSlotBytes = 512 * 1024;
 constexpr size_t kHeadBytes = kCounterBytes + kSlotBytes;
-// A slot holds the sum of the K blocks' partial results as a fixed-point number (34 fractional bits, magnitudes up
-// to 2^17 per contribution, at most 8 of them) and, above bit 56, the number of blocks that have added theirs.
-// Integer addition is exact, so the total does not depend on the order of arrival; the block whose addition
-// completes a slot reads the total out of the value its own atomic returns, writes the output and clears the slot:
-// one trip to memory instead of three (partial sums, arrival counter, partial sums again).
-constexpr int kSlotFracBits = 34;
+// A slot holds the sum of the K blocks' partial results as a fixed-point number (26 fractional bits, kept in bits
+// 8..55; magnitudes up to 2^17 per contribution, at most 15 of them) and, above bit 56, the number of blocks that
+// have added theirs.  Integer addition is exact, so the total does not depend on the order of arrival; the block whose
+// addition completes a slot reads the total out of the value its own atomic returns, writes the output and clears the
+// slot: one trip to memory instead of three (partial sums, arrival counter, partial sums again).
+// A contribution that has no fixed-point form is counted instead, in the low byte: bits 0..3 count those beyond
+// +2^17 (the fp16 result is +inf whatever the others add), bits 4..7 those beyond -2^17, and a NaN counts in both --
+// the total is then +inf, -inf, or NaN when both kinds met, as a floating-point sum of the same terms would be.
+constexpr int kSlotFracBits = 26;
 constexpr float kSlotLimit = 131071.0f;
+constexpr unsigned long long kSlotOne = 1ull << 56;
 __device__ __forceinline__ unsigned long long slot_term(float v)
 {
-    // beyond the fp16 range the output is infinite either way; a NaN takes the same way out (it cannot be added)
-    v = v >= -kSlotLimit ? (v <= kSlotLimit ? v : kSlotLimit) : (v < -kSlotLimit ? -kSlotLimit : kSlotLimit);
-    const long long fx = (long long)__builtin_rintf(v * (float)(1ull << kSlotFracBits)); // exact scaling by 2^34
-    return (1ull << 56) + (unsigned long long)fx;
+    if (!(v <= kSlotLimit)) // beyond +2^17, or NaN
+        return kSlotOne + (v != v ? 0x11ull : 0x01ull);
+    if (v < -kSlotLimit)
+        return kSlotOne + 0x10ull;
+    const long long fx = (long long)__builtin_rintf(v * (float)(1u << kSlotFracBits)) * 256; // exact scaling by 2^26
+    return kSlotOne + (unsigned long long)fx;
 }
 __device__ __forceinline__ int slot_count(unsigned long long word) { return (int)((word + (1ull << 55)) >> 56); }
 __device__ __forceinline__ float slot_total(unsigned long long word, int count)
 {
+    const unsigned flags = (unsigned)word & 0xFFu;
+    if (flags) {
+        const bool pos = (flags & 0x0Fu) != 0, neg = (flags & 0xF0u) != 0;
+        return pos && neg ? __builtin_nanf("") : (pos ? __builtin_inff() : -__builtin_inff());
+    }
     const long long fx = (long long)(word - ((unsigned long long)count << 56));
-    return (float)((double)fx * (1.0 / (double)(1ull << kSlotFracBits)));
+    return (float)((double)fx * (1.0 / (double)(1ull << (kSlotFracBits + 8))));
 }
 
 enum { TK_U8_COLS = 1, TK_U8_SCALAR = 2, TK_F16 = 3 };

@@ -152,11 +152,11 @@ def codes_in_checkpoint_layout(lin: HQQLinearTritonSavable) -> torch.Tensor:
 
 def iterate_experts(model) -> tp.Iterator[tp.Tuple[tp.Tuple[int, int], MixtralBLockSparseTop2MLP_HQQ]]:
     """Every registered expert, in uid order, as a module on the device.  All of them are views of one scratch slab
-    that the next iteration overwrites (filled from the expert's pinned host copy)."""
+    that the next iteration overwrites (filled from the expert's pinned host copy, or from its device slot when it has none)."""
     cache_ = model.expert_cache
     scratch = MixtralExpertWrapper(copy.deepcopy(cache_.slots[0]._expert[0]), cache_.device)
     for uid, info in sorted(cache_.registered_experts.items()):
-        scratch.storage.copy_(info.host_slab.untyped_storage())
+        scratch.storage.copy_(cache_.expert_bytes(uid).untyped_storage())
         yield uid, scratch._expert[0]
 
 

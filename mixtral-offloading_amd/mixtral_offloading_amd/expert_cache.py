@@ -8,7 +8,8 @@ only valid inside the loop.  What is different underneath:
 
 * the policy (which expert a miss evicts, hit / miss counts) is the host-only
   C++ object ``hqq_lru`` of the library, one per eviction group;
-* every expert keeps a pinned host copy for its whole life, so an eviction
+* every expert that can be evicted (any expert of a group with an offloaded
+  member) keeps a pinned host copy for its whole life, so an eviction
   copies nothing back (the reference copies the victim device-to-host,
   ``src/expert_cache.py:189``; weights are immutable, the copy is redundant);
 * host-to-device loads are ``hipMemcpyAsync`` from pinned memory on a side
@@ -39,7 +40,9 @@ class ExpertInfo:
     uid: ExpertUID
     eviction_group: int
     index: int  # index of the expert inside its eviction group
-    host_slab: torch.Tensor  # pinned uint8 copy, kept for the life of the cache
+    # pinned uint8 copy, kept for the life of the cache; None while the expert cannot be evicted (no expert of its
+    # group is offloaded), so that a fully resident model pins nothing
+    host_slab: Optional[torch.Tensor]
 
     @property
     def offloaded(self) -> bool:
@@ -55,6 +58,7 @@ class EvictionGroup:
             raise MemoryError("hqq_lru_create failed")
         self.members: List[ExpertInfo] = []
         self.global_slot: List[int] = []  # local slot -> global device slot
+        self.evictable = False  # true once an expert of the group is offloaded: residents can then be evicted
 
     def __del__(self):
         if getattr(self, "_lru", None):
@@ -105,12 +109,29 @@ class ExpertCache:
         self.group_infos: Dict[int, EvictionGroup] = dict()
         self.n_offloaded = 0
 
+        self._init_device_side()
+        self._used = [False] * len(self.slots)
+        self.bytes_copied = 0
+
+    # ---- the device side, kept apart so that the scheduling above it can be driven on a machine without a GPU
+    def _init_device_side(self) -> None:
         assert self.device.type == "cuda", "experts are cached on a GPU"
         self.copy_stream = torch.cuda.Stream(device=self.device)  # default priority
         self.ready = [torch.cuda.Event() for _ in self.slots]  # load into the slot finished (copy stream)
         self.released = [torch.cuda.Event() for _ in self.slots]  # last use of the slot finished (compute stream)
-        self._used = [False] * len(self.slots)
-        self.bytes_copied = 0
+
+    def _compute_stream(self):
+        return torch.cuda.current_stream(self.device)
+
+    def _alloc_host(self, nbytes: int) -> torch.Tensor:
+        return torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+
+    def _copy_in(self, info: ExpertInfo, slot: int) -> None:
+        dst = self.slots[slot].storage
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.lib.hqq_slab_h2d_async(dst.data_ptr(), info.host_slab.data_ptr(), self.module_size,
+                                                   self.copy_stream.cuda_stream, None), "hqq_slab_h2d_async")
+            self.ready[slot].record(self.copy_stream)
 
     def _check_module(self, module: MixtralExpertWrapper):
         assert isinstance(module.storage, torch.UntypedStorage)
@@ -136,6 +157,11 @@ class ExpertCache:
         assert isinstance(module, self.module_type)
         return self.add_expert_storage(uid, module.storage, eviction_group=eviction_group, offload=offload)
 
+    def _pin(self, source: torch.UntypedStorage) -> torch.Tensor:
+        host = self._alloc_host(self.module_size)
+        host.copy_(torch.as_tensor(source, dtype=torch.uint8, device=source.device))
+        return host
+
     def add_expert_storage(self, uid: ExpertUID, storage: torch.UntypedStorage, eviction_group: int = 0,
                            offload: Optional[bool] = None):
         assert uid not in self.registered_experts, f"expert {uid} already registered"
@@ -146,9 +172,13 @@ class ExpertCache:
         if not to_device:
             if offload is False or self.n_offloaded >= self.offload_size:
                 raise ValueError("Cache is full")
-        host = torch.empty(self.module_size, dtype=torch.uint8, pin_memory=True)
-        host.copy_(torch.as_tensor(storage, dtype=torch.uint8, device=storage.device))
-        info = ExpertInfo(uid, eviction_group, len(group.members), host)
+        # Host copies are pinned only for experts that can leave the device: an expert can be evicted once any expert
+        # of its group is offloaded (a miss of that group then takes a resident one's place).
+        if not to_device and not group.evictable:
+            group.evictable = True
+            for member in group.members:
+                member.host_slab = self._pin(self.slots[group.global_slot[group.slot_of(member.index)]].storage)
+        info = ExpertInfo(uid, eviction_group, len(group.members), self._pin(storage) if group.evictable else None)
         info._group = group
         group.members.append(info)
         self.registered_experts[uid] = info
@@ -158,6 +188,16 @@ class ExpertCache:
             group.add_resident(info.index, slot)
         else:
             self.n_offloaded += 1
+
+    def expert_bytes(self, uid: ExpertUID) -> torch.Tensor:
+        """The slab of a registered expert as a uint8 tensor: its pinned host copy, or (an expert that cannot be
+        evicted has none) a view of the device slot it lives in."""
+        info = self.registered_experts[uid]
+        if info.host_slab is not None:
+            return info.host_slab
+        group = self.group_infos[info.eviction_group]
+        storage = self.slots[group.global_slot[group.slot_of(info.index)]].storage
+        return torch.as_tensor(storage, dtype=torch.uint8, device=storage.device)
 
     def load_experts(self, *uids: ExpertUID, unordered: bool = False) -> Iterator[Tuple[ExpertUID, MixtralExpertWrapper]]:
         """
@@ -178,58 +218,92 @@ class ExpertCache:
         assert len(set(info.eviction_group for info in infos)) == 1, "experts must be in the same evicton group"
         group = self.group_infos[infos[0].eviction_group]
         order, local_slots, victims = group.plan([info.index for info in infos])
-        compute = torch.cuda.current_stream(self.device)
+        compute = self._compute_stream()
         miss = {idx: victim >= 0 for idx, victim in zip(order, victims)}
         local_of = dict(zip(order, local_slots))
+        sequence = order if unordered else [info.index for info in infos]
+        rank = {idx: i for i, idx in enumerate(sequence)}
         to_load = deque(idx for idx in order if miss[idx])  # in the order the policy evicted for them
         slot_for: Dict[int, int] = {idx: group.global_slot[local_of[idx]] for idx in order if not miss[idx]}
-        waiting = set()  # device slots holding an expert of this call that has not been handed out yet
+        # Device slots whose content is an expert of this call that has not been handed out yet -- hits included: the
+        # policy marks every requested expert used and then lets later misses of the same call evict the earlier ones
+        # (a call may ask for more experts than the group has places).  Nothing is copied into such a slot.
+        holder: Dict[int, int] = {slot: idx for idx, slot in slot_for.items()}
+        copied = set()  # experts whose slot is filled by a copy of this call: the compute stream waits for it
+        again = set()   # experts whose slot had to be given up before their turn (ordered iteration only)
 
-        def issue_loads():
-            # Start as many loads as there are spare slots, on the side stream.  A spare that still holds an expert
-            # of this call (evicted again by a later miss of the same call) is not touched until that expert has
-            # been handed out; it is always ahead in the sequence, so this cannot stall.
-            while to_load and self.spare and self.spare[0] not in waiting:
-                idx = to_load.popleft()
-                dst = self.spare.popleft()
-                local = local_of[idx]
-                self.spare.append(group.global_slot[local])  # the victim's slot is the next spare
+        def copy_to(idx: int, dst: int) -> None:
+            if self._used[dst]:  # its last reader on the compute stream must be done before it is overwritten
+                self.copy_stream.wait_event(self.released[dst])
+            self._copy_in(group.members[idx], dst)
+            self.bytes_copied += self.module_size
+            slot_for[idx] = dst
+            holder[dst] = idx
+            copied.add(idx)
+
+        def give_up(candidates) -> int:
+            # every candidate holds an expert that this call still has to hand out, all of them later in the sequence
+            # (ordered iteration asked for a miss before hits that the policy evicted for it): the one needed last
+            # loses its place and is copied in again from its host slab when its turn comes
+            dst = max(candidates, key=lambda s: rank[holder[s]])
+            bumped = holder.pop(dst)
+            del slot_for[bumped]
+            again.add(bumped)
+            return dst
+
+        def start_load(idx: int, force: bool) -> bool:
+            # A miss goes into a spare slot and its victim's slot becomes the next spare (so the copy never waits for
+            # the victim's last use), or, with no spare free, into the victim's own slot.
+            local = local_of[idx]
+            home = group.global_slot[local]
+            dst = next((s for s in self.spare if s not in holder), None)
+            if dst is None and home not in holder:
+                dst = home
+            if dst is None:
+                if not force:
+                    return False
+                dst = give_up([home] + list(self.spare))
+            if dst != home:
+                self.spare.remove(dst)
+                self.spare.append(home)
                 group.global_slot[local] = dst
-                if self._used[dst]:  # its last reader on the compute stream must be done before it is overwritten
-                    self.copy_stream.wait_event(self.released[dst])
-                self._copy_in(group.members[idx], dst)
-                slot_for[idx] = dst
-                waiting.add(dst)
+            copy_to(idx, dst)
+            return True
+
+        def issue_loads() -> None:
+            while to_load and start_load(to_load[0], force=False):
+                to_load.popleft()
 
         try:
             self.active = True
-            if to_load and not self.spare:
-                raise ValueError("No free device buffer: buffer_size must be at least 1")
             issue_loads()
-            sequence = order if unordered else [info.index for info in infos]
             for idx in sequence:
                 if idx not in slot_for:
                     issue_loads()
-                    if idx not in slot_for:
+                if idx not in slot_for and idx in again:
+                    # evicted by the policy within this call: it only passes through a spare slot
+                    if not self.spare:
                         raise RuntimeError("internal error: caching algorithm failed")
+                    dst = next((s for s in self.spare if s not in holder), None)
+                    copy_to(idx, dst if dst is not None else give_up(list(self.spare)))
+                elif idx not in slot_for:
+                    if not to_load or to_load[0] != idx:
+                        raise RuntimeError("internal error: caching algorithm failed")
+                    start_load(to_load.popleft(), force=True)
                 slot = slot_for[idx]
-                if miss[idx]:
+                if idx in copied:
                     compute.wait_event(self.ready[slot])
                 yield (group.members[idx].uid, self.slots[slot])
                 self.released[slot].record(compute)
                 self._used[slot] = True
-                waiting.discard(slot)
+                del holder[slot]
                 issue_loads()
         finally:
+            # a caller that leaves the loop early: the policy already counts the remaining misses as resident
+            holder.clear()
+            while to_load:
+                start_load(to_load.popleft(), force=True)
             self.active = False
-
-    def _copy_in(self, info: ExpertInfo, slot: int) -> None:
-        dst = self.slots[slot].storage
-        with torch.cuda.device(self.device):
-            _lib.check(_lib.lib.hqq_slab_h2d_async(dst.data_ptr(), info.host_slab.data_ptr(), self.module_size,
-                                                   self.copy_stream.cuda_stream, None), "hqq_slab_h2d_async")
-            self.ready[slot].record(self.copy_stream)
-        self.bytes_copied += self.module_size
 
     def resident_group(self, eviction_group: int) -> Optional[List[MixtralExpertWrapper]]:
         """The device modules of every expert of a group, in expert order, when all of them are resident and none

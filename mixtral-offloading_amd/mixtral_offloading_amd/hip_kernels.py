@@ -433,6 +433,8 @@ def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: tor
     assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous() and cache_k.is_contiguous() and cache_v.is_contiguous()
     assert pos.dtype == torch.int64 and pos.is_cuda and cos.shape[-1] == hd and cos.is_contiguous() and sin.is_contiguous()
     assert out.numel() == n_heads * hd and k.numel() == n_kv * hd == v.numel()
+    # the kernel bounds the device-side position by the cache length only: the rope tables must cover the cache
+    assert cos.shape[0] >= max_len and sin.shape[0] >= max_len, "rope tables shorter than the KV cache"
     with _on(q.device):
         _lib.check(_lib.lib.hqq_attention_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), cos.data_ptr(), sin.data_ptr(),
                                                  pos.data_ptr(), cache_k.data_ptr(), cache_v.data_ptr(), max_len, n_heads,

@@ -131,6 +131,10 @@ class DecodeGraph:
 
         self.model, self.max_len = model, max_len
         cfg, dev = model.config, model.device
+        # the attention kernel reads the rope tables at the device-side position, which only the cache length bounds
+        if max_len > model.rotary.cos.shape[0]:
+            raise ValueError(f"a cache of {max_len} positions exceeds the rope tables ({model.rotary.cos.shape[0]} "
+                             "positions): build the model with a larger max_positions")
         self.tables = []
         for layer_id, layer in enumerate(model.model.layers):
             mods = layer.block_sparse_moe.experts.resident_group(layer_id)
@@ -260,6 +264,8 @@ class MixtralForCausalLM(nn.Module):
         cfg = self.config
         hd = cfg.hidden_size // cfg.num_attention_heads
         L = max_len or self.max_positions
+        if L > self.rotary.cos.shape[0]:
+            raise ValueError(f"a cache of {L} positions exceeds the rope tables ({self.rotary.cos.shape[0]} positions)")
         mk = dict(dtype=torch.float16, device=self.device)
         return [(torch.zeros((cfg.num_key_value_heads, L, hd), **mk), torch.zeros((cfg.num_key_value_heads, L, hd), **mk))
                 for _ in range(cfg.num_hidden_layers)]

@@ -299,6 +299,10 @@ def test_graph_decode_guards_its_cache_capacity():
     off = bm.OffloadConfig(main_size=8, offload_size=0, buffer_size=1, offload_per_layer=0)
     model = bm.build_model(torch.device("cuda:0"), bm.default_quant_config(), off, model_config=cfg, seed=5,
                            max_positions=64)
+    with pytest.raises(ValueError):
+        DecodeGraph(model, 65)  # a cache longer than the rope tables: the device-side position could run past them
+    with pytest.raises(ValueError):
+        model.new_cache(65)
     dec = DecodeGraph(model, 12)
     with pytest.raises(ValueError):
         dec.prefill(torch.zeros(12, dtype=torch.int64, device="cuda"))

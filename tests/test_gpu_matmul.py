@@ -235,3 +235,51 @@ def test_other_model_shapes_against_dequantize_then_matmul(nbits, n, k, gs, m):
         err = (y.float() - ref).abs()
         bound = 1e-2 * ref.abs() + atol + ref.abs() * 2.0 ** -11
         assert bool((err <= bound).all()), float((err / bound).max())
+
+
+def _signed_layer(nbits, n, k, gs, seed):
+    """A layer whose weights are +-(2q + 1 - 2^nbits) * step / 2 (zero = (2^nbits - 1) / 2 everywhere, one scale), with
+    the codes of row G the complement of row 0's, so that row G is minus row 0."""
+    from mixtral_offloading_amd import hip_kernels, packing
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    s_cnt = n * k // gs
+    top = 2 ** nbits - 1
+    q = torch.randint(0, top + 1, (n, k), dtype=torch.uint8, device="cuda", generator=g)
+    q[n // gs] = top - q[0]
+    pack = {4: packing.pack_4bit_u8_common, 2: packing.pack_2bit_u8_common, 3: packing.pack_3bit_i32_common}[nbits]
+    meta = {"nbits": nbits, "group_size": gs, "shape": (n, k), "quant_scale": True, "quant_zero": True,
+            "scale_q": torch.full((128, s_cnt // 128), 200, dtype=torch.uint8, device="cuda"),
+            "meta_scale": {"scale": torch.full((1, s_cnt // 128), 1e-4, device="cuda").half(),
+                           "zero": torch.zeros((1, s_cnt // 128), device="cuda").half()},
+            "zero_q": torch.full((1, s_cnt), top, dtype=torch.uint8, device="cuda"),
+            "meta_zero": {"scale": torch.tensor([0.5], device="cuda").half(), "zero": torch.tensor([0.0], device="cuda").half()}}
+    return hip_kernels.LinearDesc(pack(q), meta)
+
+
+@pytest.mark.parametrize("nbits,n,k,gs", [(2, 4096, 14336, 16), (3, 4096, 14336, 64), (4, 1024, 8192, 64)])
+def test_split_k_keeps_nan_and_infinity(nbits, n, k, gs):
+    """Where K is split over blocks the partial sums meet in fixed-point slots: a NaN or an overflowing partial sum
+    must still come out as NaN / +-inf, as the reference's fp32 accumulation followed by the fp16 cast gives
+    (src/triton_kernels.py:103-131), not as a finite number."""
+    from mixtral_offloading_amd import hip_kernels
+    desc = _signed_layer(nbits, n, k, gs, seed=nbits)
+    w = hip_kernels.dequantize(desc).float()
+    G = n // gs
+    assert torch.equal(w[G], -w[0])
+    # every term of row 0 positive and huge: +inf there, -inf in row G
+    x = (torch.sign(w[0]) * 65504.0).half().view(1, k).contiguous()
+    ref = (x.float() @ w.t()).half()
+    assert bool(torch.isposinf(ref[0, 0])) and bool(torch.isneginf(ref[0, G]))
+    y = hip_kernels.matmul(desc, x)
+    assert bool(torch.isposinf(y[0, 0])) and bool(torch.isneginf(y[0, G]))
+    # a NaN activation reaches every output
+    x = torch.randn((1, k), device="cuda").half()
+    x[0, k // 2 + 3] = float("nan")
+    for rep in range(2):  # and leaves the slots clean for the next call
+        y = hip_kernels.matmul(desc, x)
+        assert bool(torch.isnan(y).all())
+    x[0, k // 2 + 3] = 1.0
+    y = hip_kernels.matmul(desc, x)
+    ref = x.float() @ w.t()
+    assert bool(torch.isfinite(y).all())
+    assert float((y.float() - ref).abs().max()) <= 1e-2 * float(ref.abs().max()) + 1e-3 * float(x.float().norm() * w.norm(dim=1).max())
