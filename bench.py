@@ -71,28 +71,85 @@ def make_expert(seed, device):
     return layers
 
 
-def cpu_baseline(budget_s=15.0):
+def make_attention(device):
+    """The four 4-bit g64 projections of one decoder layer (q, k, v, o), random-init, for the CPU decode figure."""
+    import torch
+    from torch import nn
+
+    from mixtral_offloading_amd.custom_layers import HQQLinearTritonSavable
+    from mixtral_offloading_amd.hqq_core import BaseQuantizeConfig
+
+    cfg = BaseQuantizeConfig(nbits=4, group_size=64, quant_zero=True, quant_scale=True)
+    cfg["weight_quant_params"]["optimize"] = False
+    g = torch.Generator(device=device).manual_seed(77)
+    layers = []
+    for n in (HIDDEN, 1024, 1024, HIDDEN):
+        lin = nn.Linear(HIDDEN, n, bias=False, device=device, dtype=torch.float16)
+        lin.weight.data = (torch.randn((n, HIDDEN), device=device, generator=g) * 0.02).half()
+        layers.append(HQQLinearTritonSavable(lin, cfg))
+    return layers
+
+
+def _cpu_layer(lin):
+    """A quantised layer of the GPU leg as the CPU path's layer dict (the same tensors, copied to the host)."""
+    import torch
+
+    meta = lin.meta
+    out = {"nbits": int(meta["nbits"]), "group_size": int(meta["group_size"]), "shape": tuple(int(v) for v in meta["shape"]),
+           "quant_scale": bool(meta.get("quant_scale")), "quant_zero": bool(meta.get("quant_zero")),
+           "W_q": torch.Tensor.as_subclass(lin.W_q, torch.Tensor).cpu()}
+    for q, m in (("scale_q", "meta_scale"), ("zero_q", "meta_zero")):
+        if q in meta:
+            out[q] = meta[q].cpu()
+            out[m] = {"scale": meta[m]["scale"].cpu().half(), "zero": meta[m]["zero"].cpu().half()}
+    for key in ("scale", "zero"):
+        if key in meta and key + "_q" not in meta:
+            out[key] = meta[key].cpu()
+    return out
+
+
+def cpu_baseline(expert, x, attention=None, budget_s=12.0):
+    """The reference's PyTorch path (meta expansion + dequantize + matmul per call, src/custom_layers.py:95-116) on the
+    host cores, on the tensors the GPU leg runs on: expert 0 and the same x.  With `attention` (the four 4-bit
+    projections of one decoder layer) it also times one decoder layer's quantised linears, from which a CPU decode
+    rate follows: a token is 32 layers of 4 attention projections and 2 expert FFNs (the fp16 head, the norms, the
+    router and the attention itself are left out, which flatters the CPU)."""
     import torch
 
     from oracle import torch_path as tp
 
-    gen = torch.Generator().manual_seed(0)
-    w1 = tp.random_layer(gen, FFN, HIDDEN, NBITS, GROUP, META_GROUP)
-    w2 = tp.random_layer(gen, HIDDEN, FFN, NBITS, GROUP, META_GROUP)
-    w3 = tp.random_layer(gen, FFN, HIDDEN, NBITS, GROUP, META_GROUP)
-    x = torch.randn((1, HIDDEN), generator=gen).half()
+    w1, w2, w3 = (_cpu_layer(l) for l in expert)
+    xc = x.cpu()
     with torch.inference_mode():
-        tp.expert_ffn(x, w1, w2, w3)  # warm up
+        tp.expert_ffn(xc, w1, w2, w3)  # warm up
         t0 = time.perf_counter()
         n = 0
         while n < 3 or (time.perf_counter() - t0 < budget_s and n < 200):
-            tp.expert_ffn(x, w1, w2, w3)
+            tp.expert_ffn(xc, w1, w2, w3)
             n += 1
         dt = (time.perf_counter() - t0) / n
-    return {"value": round(ffn_step_bytes(1) / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
-            "kind": "port", "ms_per_step": round(dt * 1e3, 2),
-            "sample": f"{n} steps of the same batch-1 2-bit expert FFN (one expert, host-resident), torch CPU half ops, "
-                      f"meta expansion + dequantize + matmul per call as the reference does"}
+        out = {"value": round(ffn_step_bytes(xc.shape[0]) / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+               "os_cpu_count": os.cpu_count(), "kind": "port", "ms_per_step": round(dt * 1e3, 2),
+               "sample": f"{n} steps of the same batch-{xc.shape[0]} 2-bit expert FFN on the GPU leg's own tensors (expert 0 "
+                         f"and x copied to the host), torch CPU half ops, meta expansion + dequantize + matmul per call "
+                         f"as the reference does"}
+        if attention is not None:
+            att = [_cpu_layer(l) for l in attention]
+            xa = torch.randn((1, HIDDEN), generator=torch.Generator().manual_seed(5)).half()
+            for l in att:
+                tp.forward(xa, l)
+            t0 = time.perf_counter()
+            reps = 3
+            for _ in range(reps):
+                for l in att:
+                    tp.forward(xa, l)
+            dt_att = (time.perf_counter() - t0) / reps
+            layer_ms = (dt_att + 2 * dt) * 1e3
+            out["decode_layer_ms"] = round(layer_ms, 1)
+            out["decode_tok_s"] = round(1e3 / (32 * layer_ms), 4)
+            out["decode_sample"] = (f"one decoder layer's quantised linears at batch 1 (q, k, v, o 4-bit g64: {dt_att * 1e3:.1f} ms, "
+                                    f"measured {reps} times; 2 expert FFNs at the rate above) x 32 layers")
+    return out
 
 
 def random_desc(nbits, n, k, gs, seed, dev):
@@ -115,6 +172,23 @@ def random_desc(nbits, n, k, gs, seed, dev):
             "meta_zero": {"scale": torch.tensor([(2 ** nbits - 1) / 255.0], device=dev).half(),
                           "zero": torch.tensor([0.0], device=dev).half()}}
     return hip_kernels.LinearDesc(pack(q), meta), q
+
+
+PROFILE = os.path.join(ROOT, "profiles", "gemv_strip_kernel_ffn_2bit_g16_m1.txt")
+
+
+def profiled_traffic():
+    """HBM bytes per launch of the dominant kernel as the tracked counter profile records them (a line
+    `traffic_bytes_per_launch: <int>`, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this command scaled by a copy of
+    known size); None when the profile has no such line."""
+    try:
+        with open(PROFILE) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return int(line.split(":")[1].split()[0].replace(",", ""))
+    except OSError:
+        pass
+    return None
 
 
 def survey_section(dev):
@@ -189,7 +263,7 @@ def survey_section(dev):
     return rows
 
 
-def decode_section(dev, tokens_resident=256, tokens_offload=48):
+def decode_section(dev, tokens_resident=256, tokens_offload=256):
     """Tokens per second of the whole model; every figure is measured between synchronisations
     around the decode loop, prompt processing excluded."""
     import gc
@@ -382,14 +456,14 @@ def main():
                    "bytes_per_step": ffn_step_bytes(m), "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this command, scaled by a
-                     # 256 MiB copy (profiles/gemv_strip_kernel_ffn_2bit_g16_m1.txt); measured at batch 1 only
-                     "traffic": 46320457 if m == 1 else None,
+                     # read from the tracked counter profile (measured at batch 1 only)
+                     "traffic": profiled_traffic() if m == 1 else None,
+                     "traffic_source": "profiles/gemv_strip_kernel_ffn_2bit_g16_m1.txt",
                      "kernel": "gemv_strip_kernel<2,1,4,2,8,1,2,1,false,0> as launched by hqq_gate_up (w1 and w3 in one grid, one launch)",
                      "bytes_per_launch": gate_up_bytes(m), "us_per_launch": round(ms_gate * 1e3, 3)},
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline()
+        out["cpu_baseline"] = cpu_baseline(experts[0], x, attention=make_attention(dev))
     if args.survey:
         out["kernels"] = survey_section(dev)
     if not args.no_decode:

@@ -714,14 +714,12 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl, int nl = 1)
     pl.BM = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
     if (M > 128 && pl.kinds != 0 && ((M + 127) / 128) * (760 + 8 * 128) <= ((M + 63) / 64) * (760 + 8 * 64))
         pl.BM = 128;
-    if (tuning_overrides())
-        if (const char *e = std::getenv("HQQ_TILE_BM"))
-            pl.BM = std::atoi(e);
+    pl.BM = tuning_int("HQQ_TILE_BM", pl.BM);
     const int64_t mtiles = (M + pl.BM - 1) / pl.BM;
     if (mtiles > 65535)
         return false;
     pl.JW = kWaves, pl.KW = 1;
-    if (pl.BM <= 32 && pl.kinds != 0 && !(tuning_overrides() && std::getenv("HQQ_TILE_KW1"))) {
+    if (pl.BM <= 32 && pl.kinds != 0 && !tuning_flag("HQQ_TILE_KW1")) {
         // the narrowest batch tile: a block is one packed row, its eight waves split the block's K range.  Blocks
         // along K only until the chip is covered, with at least four steps (256 columns) per wave.
         pl.JW = nl == 2 ? 2 : 1, pl.KW = 8; // a gate: both projections of a packed row in one block of sixteen waves
@@ -733,9 +731,7 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl, int nl = 1)
             kb = pl.KT / (4 * pl.KW);
         if (kb < 1)
             kb = 1;
-        if (tuning_overrides())
-            if (const char *e = std::getenv("HQQ_TILE_KSP"))
-                kb = std::atoi(e);
+        kb = tuning_int("HQQ_TILE_KSP", (int)kb);
         pl.KTS = (int)((pl.KT + kb * pl.KW - 1) / (kb * pl.KW));
         pl.KSP = (pl.KT + pl.KTS * pl.KW - 1) / (pl.KTS * pl.KW);
         return (int64_t)pl.GP * pl.KSP <= 0x7fffffff;
@@ -752,9 +748,7 @@ bool make_plan(const hqq_linear *l, int64_t M, TilePlan &pl, int nl = 1)
         ksp = pl.KT / 8;
     if (ksp < 1)
         ksp = 1;
-    if (tuning_overrides())
-        if (const char *e = std::getenv("HQQ_TILE_KSP"))
-            ksp = std::atoi(e);
+    ksp = tuning_int("HQQ_TILE_KSP", (int)ksp);
     pl.KTS = (int)((pl.KT + ksp - 1) / ksp);
     pl.KSP = (pl.KT + pl.KTS - 1) / pl.KTS;
     if ((int64_t)(pl.GP / kWaves) * pl.KSP * nl > 0x7fffffff)

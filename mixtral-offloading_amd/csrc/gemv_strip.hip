@@ -720,12 +720,6 @@ __global__ void zero_words_kernel(uint32_t *p, size_t n)
         p[i] = 0;
 }
 
-int env_int(const char *name, int dflt)
-{
-    const char *v = std::getenv(name);
-    return v ? std::atoi(v) : dflt;
-}
-
 struct StripPlan {
     int F, GP, RB, NS, MT, S, D, WAVES, KS, BK, SKIND, ZKIND;
 };
@@ -795,10 +789,10 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl, int64_t ti
             KS = ((pl.NS + S - 1) / S + BK - 1) / BK;
         }
     }
-    if (tuning_overrides() && env_int("HQQ_STRIP_K", (int)l->K) == (int)l->K && env_int("HQQ_STRIP_NL", NL) == NL) {
-        S = env_int("HQQ_STRIP_S", S);
-        KS = env_int("HQQ_STRIP_KS", KS);
-        BK = env_int("HQQ_STRIP_BK", BK);
+    if (tuning_int("HQQ_STRIP_K", (int)l->K) == (int)l->K && tuning_int("HQQ_STRIP_NL", NL) == NL) {
+        S = tuning_int("HQQ_STRIP_S", S);
+        KS = tuning_int("HQQ_STRIP_KS", KS);
+        BK = tuning_int("HQQ_STRIP_BK", BK);
     }
     if (S != 1 && S != 2 && !(S == 4 && pl.MT <= 2))
         return false;
@@ -946,7 +940,7 @@ int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t
     // A gate of three or four rows whose blocks hold all of K runs as two passes of the two-row kernel in one launch.
     int passes = 1;
     if ((M == 3 || M == 4) && j.EPI == 1 && j.NL == 2 && j.NG == 1 && !j.norm_weight &&
-        !(tuning_overrides() && std::getenv("HQQ_STRIP_NOPASS")) && plan_job(j, 2, pl, per_group, part_bytes) &&
+        !tuning_flag("HQQ_STRIP_NOPASS") && plan_job(j, 2, pl, per_group, part_bytes) &&
         pl.BK == 1 && 2 * per_group[0].GP <= 65535)
         passes = 2;
     if (passes == 1 && !plan_job(j, M, pl, per_group, part_bytes))

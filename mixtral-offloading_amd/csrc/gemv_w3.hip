@@ -437,16 +437,16 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, W3Plan &pl)
     int BK = (pl.NS + kW3Waves * kW3S - 1) / (kW3Waves * kW3S);
     while ((int64_t)pl.P * pl.RB * NL * BK < 200 && BK < pl.NS)
         ++BK;
-    const bool tune = tuning_overrides() && (!std::getenv("HQQ_W3_K") || std::atoi(std::getenv("HQQ_W3_K")) == (int)l->K);
-    if (tune && std::getenv("HQQ_W3_BK"))
-        BK = std::atoi(std::getenv("HQQ_W3_BK"));
+    const bool tune = tuning_int("HQQ_W3_K", (int)l->K) == (int)l->K;
+    if (tune)
+        BK = tuning_int("HQQ_W3_BK", BK);
     if (BK < 1 || BK > pl.NS || (pl.NS + BK - 1) / BK > kW3Waves * kW3S)
         return false;
     pl.SB = (pl.NS + BK - 1) / BK;
     pl.BK = (pl.NS + pl.SB - 1) / pl.SB;
     pl.S = pl.SB > kW3Waves ? kW3S : 1;
-    if (tune && std::getenv("HQQ_W3_S"))
-        pl.S = std::atoi(std::getenv("HQQ_W3_S")) == 2 ? 2 : pl.S;
+    if (tune)
+        pl.S = tuning_int("HQQ_W3_S", pl.S) == 2 ? 2 : pl.S;
     pl.KS = (pl.SB + pl.S - 1) / pl.S;
     if ((int64_t)pl.P * NL > 65535 || pl.RB > 65535 || (int64_t)pl.P * pl.RB * NL * sizeof(int) > kCounterBytes)
         return false;

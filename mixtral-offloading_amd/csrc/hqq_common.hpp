@@ -78,13 +78,20 @@ __device__ __forceinline__ float wave_sum(float v)
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Launch shapes can be overridden through HQQ_* environment variables for experiments, but only in a process that
-// has HQQ_TUNING set when the library is first used: a normal call never reads the environment.
-inline bool tuning_overrides()
+// The library never reads the environment.  A tuning build (make TUNING=1, -DHQQ_TUNING_BUILD, a separate .so that
+// experiments select through HQQ_MI355X_LIB) lets HQQ_* variables override launch shapes; in the normal build these
+// helpers are constants and the override code folds away.
+#ifdef HQQ_TUNING_BUILD
+inline int tuning_int(const char *name, int dflt)
 {
-    static const bool on = std::getenv("HQQ_TUNING") != nullptr;
-    return on;
+    const char *v = std::getenv(name);
+    return v ? std::atoi(v) : dflt;
 }
+inline bool tuning_flag(const char *name) { return std::getenv(name) != nullptr; }
+#else
+constexpr int tuning_int(const char *, int dflt) { return dflt; }
+constexpr bool tuning_flag(const char *) { return false; }
+#endif
 
 // launch-status helper: kernels are launched with <<<>>> and checked once
 inline int launch_status()

@@ -361,12 +361,6 @@ __global__ __launch_bounds__(64) void smallbatch_finish_kernel(const float *__re
     }
 }
 
-int env_int(const char *name, int dflt)
-{
-    const char *v = std::getenv(name);
-    return v ? std::atoi(v) : dflt;
-}
-
 struct SBPlan {
     int F, GP, RB, WR, WS, KT, NS, NSG, MT, WAVES, SK, TMODE;
 };
@@ -405,7 +399,7 @@ bool make_plan(const hqq_linear *l, int64_t M, SBPlan &pl)
     pl.MT = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : (M <= 8 ? 8 : 16)));
     pl.WAVES = pl.MT <= 4 ? 16 : (pl.MT == 8 ? 8 : 4);
     {
-        const int forced = tuning_overrides() ? env_int("HQQ_SB_BLOCK_WAVES", 0) : 0;
+        const int forced = tuning_int("HQQ_SB_BLOCK_WAVES", 0);
         if ((forced == 4 || forced == 8 || forced == 16) && forced <= pl.WAVES)
             pl.WAVES = forced;
     }
@@ -526,7 +520,7 @@ int launch_smallbatch_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *
     fill_params(p, pl, l, 0, reinterpret_cast<float *>(static_cast<char *>(ws) + workspace_head_bytes()));
     p.layer[1] = p.layer[0];
     p.x = x, p.M = (int)M;
-    p.probe = tuning_overrides() ? env_int("HQQ_SB_PROBE", 0) : 0;
+    p.probe = tuning_int("HQQ_SB_PROBE", 0);
     SBEpilogue e = {y, static_cast<const f16 *>(l->bias), ep.row_scale, ep.accumulate};
     const dim3 grid((unsigned)pl.NSG, (unsigned)(pl.RB / pl.WR), (unsigned)pl.GP);
     if (l->nbits == 2)

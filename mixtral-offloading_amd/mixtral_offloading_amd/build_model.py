@@ -120,6 +120,21 @@ def make_random_expert(model_config, quant_config: QuantConfig, gen: torch.Gener
     return expert
 
 
+def checkpoint_layout(index: dict) -> str:
+    """Code layout of a checkpoint directory, from its index: the reference's files carry no such entry and hold
+    hqq's step layout; save_quantized_checkpoint records what it wrote."""
+    layout = (index.get("metadata") or {}).get("layout", "hqq")
+    if layout not in ("hqq", "kernel"):
+        raise ValueError(f"unknown code layout {layout!r} in model.safetensors.index.json")
+    return layout
+
+
+def set_checkpoint_layout(module, layout: str) -> None:
+    for sub in module.modules():
+        if isinstance(sub, HQQLinearTritonSavable):
+            sub.checkpoint_layout = layout
+
+
 def make_and_load_expert_wrapper(config, quant_config: QuantConfig, states_dir: str, expert_uid: tuple,
                                  device: torch.device) -> MixtralExpertWrapper:
     """Reads one expert from the reference's safetensors shards (src/build_model.py:137-155)."""
@@ -128,9 +143,11 @@ def make_and_load_expert_wrapper(config, quant_config: QuantConfig, states_dir: 
     layer_idx, expert_idx = expert_uid
     with open(os.path.join(states_dir, "model.safetensors.index.json")) as f:
         module_idx = f"model.layers.{layer_idx}.block_sparse_moe.experts.{expert_idx}"
-        state_fpath = json.load(f)["weight_map"][f"{module_idx}.w1.W_q"]
+        index = json.load(f)
+        state_fpath = index["weight_map"][f"{module_idx}.w1.W_q"]
     state_dict = load_file(os.path.join(states_dir, state_fpath), device=str(device))
     expert = make_empty_expert(config, quant_config)
+    set_checkpoint_layout(expert, checkpoint_layout(index))
     expert.load_state_dict(state_dict, strict=True)
     return MixtralExpertWrapper(expert, device)
 
@@ -168,7 +185,8 @@ def save_quantized_checkpoint(model, state_path: str, layout: str = "hqq") -> No
 
     ``layout="hqq"`` stores the codes as the reference's checkpoints do (quantise-time shape, step layout), so the
     reference can read the directory as well; ``layout="kernel"`` stores them as they sit in memory, ``(N/f, K)``
-    interleaved, which only this package reads (it tells the two apart by the shape of ``W_q``)."""
+    interleaved, which only this package reads (the index records the layout under ``metadata.layout``; a directory without that
+    entry, like the reference's, is read as hqq's)."""
     from safetensors.torch import save_file
 
     assert layout in ("hqq", "kernel")
@@ -223,7 +241,9 @@ def build_model(device: torch.device, quant_config: QuantConfig, offload_config:
         from safetensors.torch import load_file
 
         with open(os.path.join(state_path, "model.safetensors.index.json")) as f:
-            weight_map = json.load(f)["weight_map"]
+            index = json.load(f)
+        weight_map = index["weight_map"]
+        set_checkpoint_layout(model, checkpoint_layout(index))
         trunk = load_file(os.path.join(state_path, weight_map["model.embed_tokens.weight"]), device=str(device))
         model.load_state_dict(trunk, strict=True)
     else:

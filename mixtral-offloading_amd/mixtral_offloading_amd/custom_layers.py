@@ -52,19 +52,29 @@ class HQQLinearTritonSavable(HQQLinear):
         super().quantize(*args, **kwargs)
         self.repack()
 
+    # Layout of the codes a state dict brings in: "hqq" (the quantiser's (gs/f, N*K/gs) step layout, what the
+    # reference's checkpoints hold and what the reference assumes of every untagged tensor, src/packing.py:29-33) or
+    # "kernel" ((N/f, K) interleaved, written by save_quantized_checkpoint(layout="kernel")).  The two shapes can
+    # coincide (N == group_size), so the layout is never guessed from the shape: the loader sets this from the
+    # checkpoint's index.
+    checkpoint_layout = "hqq"
+
     def in_kernel_layout(self) -> bool:
-        return self.W_q is not None and tuple(self.W_q.shape) == _codes_shape(self.meta)
+        """Codes are in the kernel layout when they carry the interleaved packers' tag and have the (N/f, K) shape.
+        (Tagged codes of that shape cannot be anything else: the quantiser's view (gs, N*K/gs) has it only when
+        gs == N, where the two layouts are the same array.)  Untagged codes never are: they hold hqq's step layout."""
+        return isinstance(self.W_q, PackedTensor) and tuple(self.W_q.shape) == _codes_shape(self.meta)
 
     def repack(self):
         """Quantise-time layout (gs/f, N*K/gs) -> kernel layout (N/f, K)
-        (reference src/custom_layers.py:41-47)."""
+        (reference src/custom_layers.py:41-47).  Untagged codes are in hqq's step layout, as in the reference; tagged
+        ones were packed by the interleaved packers (the patched registry) in the quantiser's shape."""
         if not self.in_kernel_layout():
             sh = tuple(int(v) for v in self.meta["shape"])
             codes = Quantizer.unpack[self.meta["packing"]](self.W_q)
             codes = codes.reshape((-1,) + sh[1:])[: sh[0], ...]
             self.W_q = Quantizer.pack[self.meta["packing"]](codes.contiguous())
-        elif not isinstance(self.W_q, PackedTensor):
-            self.W_q = PackedTensor(self.W_q)
+        assert tuple(self.W_q.shape) == _codes_shape(self.meta), "codes do not have the kernel layout's shape"
         self._desc_cache = None
 
     # --------------------------------------------------------------- compute
@@ -143,6 +153,11 @@ class HQQLinearTritonSavable(HQQLinear):
             return state_dict.pop(prefix + name)
 
         self.W_q = take("W_q")
+        if self.checkpoint_layout == "kernel":
+            assert tuple(self.W_q.shape) == _codes_shape(self.meta), "a kernel-layout checkpoint holds (N/f, K) codes"
+            self.W_q = PackedTensor(torch.Tensor.as_subclass(self.W_q, torch.Tensor))
+        else:
+            self.W_q = torch.Tensor.as_subclass(self.W_q, torch.Tensor)  # untagged: hqq's step layout
         self.bias = take("bias") if (prefix + "bias") in state_dict else None
         if not hasattr(self, "meta"):
             self.meta = {}
