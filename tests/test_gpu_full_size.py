@@ -1,0 +1,232 @@
+"""GPU tests at the full sizes of the benchmark configurations.
+
+* One Mixtral-8x7B decoder layer (hidden 4096, 32 query / 8 KV heads of 128, rope theta 1e6, 4-bit g64 attention,
+  8 experts of 2-bit g16 FFN 4096 -> 14336, top-2 router, RMSNorm eps 1e-5): a 128-token prefill, and a batch-1 decode
+  step on a 512-token KV cache, against a reference composed from the library's bit-exact de-quantiser
+  (hqq_dequantize, itself checked against the oracle elsewhere) and fp32 torch ops -- the reference's PyTorch path
+  (src/custom_layers.py:95-116 for the linears, :253-256 for the FFN, :276-312 for the MoE block).
+* The 32-layer model with per-layer expert caches of 2 and 4: 256 greedy tokens from a 64-token prompt must equal
+  the tokens of the same model with every expert resident, and the cache's hit / miss counts must follow the LRU
+  model of src/expert_cache.py on the requests the run made."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import hqq_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+
+# ------------------------------------------------------------------------------------------- one decoder layer
+@pytest.fixture(scope="module")
+def one_layer():
+    from mixtral_offloading_amd import build_model as bm
+    cfg = bm.mixtral_config(num_hidden_layers=1, vocab_size=2048)
+    off = bm.OffloadConfig(main_size=8, offload_size=0, buffer_size=1, offload_per_layer=0)
+    model = bm.build_model(torch.device("cuda:0"), bm.default_quant_config(), off, model_config=cfg, seed=11,
+                           max_positions=1024)
+    # a residual stream of unit scale going into the layer, as inside a real model (the random-init embedding is
+    # 0.02 wide, which would make the layer's own output the whole hidden state)
+    model.model.embed_tokens.weight.data.normal_(0.0, 1.0, generator=torch.Generator(device="cuda").manual_seed(12))
+    layer = model.model.layers[0]
+    from mixtral_offloading_amd import hip_kernels
+    att = layer.self_attn
+    w = {name: hip_kernels.dequantize(getattr(att, name)._desc()).float() for name in ("q_proj", "k_proj", "v_proj", "o_proj")}
+    experts = []
+    for m in model.expert_cache.resident_group(0):
+        e = m._expert[0]
+        experts.append(tuple(hip_kernels.dequantize(l._desc()).float() for l in (e.w1, e.w2, e.w3)))
+    yield model, cfg, w, experts
+    del model
+
+
+def _r16(t):
+    """Round to fp16 where the reference's fp16 model holds a tensor (every op of it returns fp16)."""
+    return t.half().float()
+
+
+def _rms(x, weight, eps):
+    return weight.float() * _r16(x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps))
+
+
+def _reference_layer(model, cfg, w, experts, x, past_k, past_v, start, choice=None):
+    """Forward of the decoder layer on hidden states x (T, hidden) with exact (fp32) sums and the fp16 roundings of
+    the reference's fp16 model between ops; past_k / past_v (kv, start, hd).  Returns (hidden out, router logits,
+    keys, values).  `choice` (T, 2) overrides the router's top-2 where given."""
+    layer, rot = model.model.layers[0], model.rotary
+    H, KV = cfg.num_attention_heads, cfg.num_key_value_heads
+    hd = cfg.hidden_size // H
+    T = x.shape[0]
+    h = _r16(_rms(x, layer.input_layernorm.weight, cfg.rms_norm_eps))
+    q = _r16(h @ w["q_proj"].t()).view(T, H, hd)
+    k = _r16(h @ w["k_proj"].t()).view(T, KV, hd)
+    v = _r16(h @ w["v_proj"].t()).view(T, KV, hd)
+    pos = torch.arange(start, start + T, device=x.device)
+    cos, sin = rot.cos[pos].float()[:, None, :], rot.sin[pos].float()[:, None, :]
+    rh = lambda t: torch.cat((-t[..., hd // 2:], t[..., :hd // 2]), dim=-1)  # noqa: E731
+    q, k = _r16(_r16(q * cos) + _r16(rh(q) * sin)), _r16(_r16(k * cos) + _r16(rh(k) * sin))
+    keys = torch.cat([past_k, k.transpose(0, 1)], dim=1)  # (KV, L, hd)
+    vals = torch.cat([past_v, v.transpose(0, 1)], dim=1)
+    g = H // KV
+    qh = q.view(T, KV, g, hd).permute(1, 2, 0, 3)  # (KV, g, T, hd)
+    scores = _r16(torch.einsum("kgtd,kld->kgtl", qh, keys)) / math.sqrt(hd)
+    L = keys.shape[1]
+    allowed = torch.arange(L, device=x.device)[None, :] <= (start + torch.arange(T, device=x.device))[:, None]
+    scores = scores.masked_fill(~allowed[None, None], float("-inf"))
+    out = _r16(torch.einsum("kgtl,kld->kgtd", _r16(torch.softmax(scores, dim=-1)), vals))  # (KV, g, T, hd)
+    out = out.permute(2, 0, 1, 3).reshape(T, H * hd)
+    x = _r16(x + _r16(out @ w["o_proj"].t()))
+    h2 = _r16(_rms(x, layer.post_attention_layernorm.weight, cfg.rms_norm_eps))
+    logits = _r16(h2 @ layer.block_sparse_moe.gate.weight.float().t())
+    probs = torch.softmax(logits, dim=-1)
+    top_w, top_e = torch.topk(probs, 2, dim=-1)
+    if choice is not None:
+        top_e = choice
+        top_w = torch.gather(probs, 1, choice)
+    top_w = _r16(top_w / top_w.sum(-1, keepdim=True))
+    moe = torch.zeros_like(x)
+    for e, (w1, w2, w3) in enumerate(experts):
+        for slot in range(2):
+            rows = (top_e[:, slot] == e).nonzero().flatten()
+            if rows.numel():
+                hh = h2[rows]
+                mid = _r16(_r16(torch.nn.functional.silu(_r16(hh @ w1.t()))) * _r16(hh @ w3.t()))
+                moe[rows] = _r16(moe[rows] + _r16(_r16(mid @ w2.t()) * top_w[rows, slot:slot + 1]))
+    return _r16(x + moe), logits, keys, vals
+
+
+def _device_choice(logits_dev, logits_ref):
+    """The device's top-2 per token, and which tokens have a clear top-2 in the reference (no near-tie: there the
+    two must agree on their own)."""
+    top_dev = torch.topk(logits_dev.float(), 2, dim=-1).indices
+    srt = torch.sort(logits_ref, dim=-1, descending=True).values
+    clear = (srt[:, 1] - srt[:, 2] > 0.05) & (srt[:, 0] - srt[:, 1] > 0.05)
+    top_ref = torch.topk(logits_ref, 2, dim=-1).indices
+    assert torch.equal(top_dev[clear], top_ref[clear])
+    return top_dev
+
+
+def _check(got, ref, what, headroom):
+    """|got - ref| <= 1e-2 |ref| + 1e-2 rms(ref), the path's matmul tolerance carried through a layer's residual
+    stream; the worst err / bound is printed and must stay below `headroom`, so that a loss of precision inside the
+    tolerance is seen."""
+    err = (got.float() - ref).abs()
+    bound = 1e-2 * ref.abs() + 1e-2 * ref.pow(2).mean().sqrt()
+    worst = float((err / bound).max())
+    print(f"{what}: worst err/bound {worst:.3f} (max |ref| {float(ref.abs().max()):.3f})")
+    assert worst <= headroom, (what, worst)
+    return worst
+
+
+@torch.inference_mode()
+def test_decoder_layer_prefill_128_tokens(one_layer):
+    model, cfg, w, experts = one_layer
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn((128, cfg.hidden_size), device="cuda", generator=g).half()
+    ck, cv = model.new_cache(130)[0]
+    layer = model.model.layers[0]
+    got = layer(x, model.rotary, ck, cv, 0)
+    _, logits_dev = layer.block_sparse_moe(layer.post_attention_layernorm(
+        x + layer.self_attn(layer.input_layernorm(x), model.rotary, ck.clone(), cv.clone(), 0))[None])
+    empty = torch.zeros((cfg.num_key_value_heads, 0, cfg.hidden_size // cfg.num_attention_heads), device="cuda")
+    _, logits_ref, _, _ = _reference_layer(model, cfg, w, experts, x.float(), empty, empty, 0)
+    choice = _device_choice(logits_dev, logits_ref)
+    ref, _, keys, vals = _reference_layer(model, cfg, w, experts, x.float(), empty, empty, 0, choice=choice)
+    assert float((logits_dev.float() - logits_ref).abs().max()) <= 2e-2 * float(logits_ref.abs().max()) + 2e-2
+    _check(ck[:, :128], keys, "prefill keys", 0.5)
+    _check(cv[:, :128], vals, "prefill values", 0.5)
+    # the residual stream is fp16, as in the reference's model: a few roundings of values near 4 are part of the error
+    _check(got, ref, "prefill hidden", 0.75)
+
+
+@torch.inference_mode()
+def test_decoder_layer_decode_step_on_a_512_token_cache(one_layer):
+    """The single-token step (grouped q/k/v with the norm folded in, the attention kernel, norm + router, the fused
+    expert FFNs) at position 512, through the whole one-layer model so that the launches are the decode path's."""
+    model, cfg, w, experts = one_layer
+    g = torch.Generator(device="cuda").manual_seed(4)
+    hd = cfg.hidden_size // cfg.num_attention_heads
+    cache = model.new_cache(520)
+    ck, cv = cache[0]
+    ck[:, :512] = torch.randn((cfg.num_key_value_heads, 512, hd), device="cuda", generator=g).half()
+    cv[:, :512] = torch.randn((cfg.num_key_value_heads, 512, hd), device="cuda", generator=g).half()
+    past_k, past_v = ck[:, :512].float().clone(), cv[:, :512].float().clone()
+    for trial in range(3):
+        tok = torch.randint(0, cfg.vocab_size, (1,), device="cuda", generator=g)
+        logits = model.forward_token(tok, cache, 512)  # (1, vocab)
+        st = model._token_state()
+        x0 = model.model.embed_tokens(tok).float()
+        # the device's router choice (sel) is what the step ran with
+        sel = st["sel"].to(torch.int64).view(1, 2)
+        hidden_ref, logits_ref, keys, vals = _reference_layer(model, cfg, w, experts, x0, past_k, past_v, 512, choice=sel)
+        srt = torch.sort(logits_ref[0], descending=True)
+        if float(srt.values[1] - srt.values[2]) > 0.05 and float(srt.values[0] - srt.values[1]) > 0.05:
+            assert sel[0].tolist() == srt.indices[:2].tolist()
+        _check(ck[:, 512:513], keys[:, 512:513], "decode key", 0.5)
+        normed_ref = _rms(hidden_ref, model.model.norm.weight, cfg.rms_norm_eps)
+        _check(st["xn"], normed_ref, "decode hidden after the final norm", 0.75)
+        # the fp16 head on top (a torch linear, not part of the path): within the bound itself
+        _check(logits, normed_ref @ model.lm_head.weight.float().t(), "decode logits", 1.0)
+
+
+# ------------------------------------------------------------------------------------------- the 32-layer model
+PROMPT, NEW_TOKENS = 64, 256
+
+
+def _build(per_layer):
+    from mixtral_offloading_amd import build_model as bm
+    cfg = bm.mixtral_config()
+    off = bm.OffloadConfig(main_size=32 * per_layer, offload_size=32 * (8 - per_layer), buffer_size=4,
+                           offload_per_layer=8 - per_layer)
+    return bm.build_model(torch.device("cuda:0"), bm.default_quant_config(), off, model_config=cfg, seed=0,
+                          max_positions=512), cfg
+
+
+@pytest.fixture(scope="module")
+def resident_tokens():
+    model, cfg = _build(8)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    prompt = torch.randint(0, cfg.vocab_size, (PROMPT,), device="cuda", generator=g)
+    tokens = model.generate(prompt, NEW_TOKENS)
+    torch.cuda.synchronize()
+    assert all(i.host_slab is None for i in model.expert_cache.registered_experts.values())  # nothing to evict: nothing pinned
+    del model
+    torch.cuda.empty_cache()
+    return prompt, tokens
+
+
+@pytest.mark.parametrize("per_layer", [2, 4])
+def test_32_layer_model_with_expert_cache_equals_resident_model(per_layer, resident_tokens):
+    prompt, want = resident_tokens
+    model, cfg = _build(per_layer)
+    cache = model.expert_cache
+    requests = []
+    inner = cache.load_experts
+
+    def recording(*uids, unordered=False):
+        requests.append(list(uids))
+        return inner(*uids, unordered=unordered)
+
+    cache.load_experts = recording
+    got = model.generate(prompt, NEW_TOKENS)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want), int((got != want).nonzero()[0]) if (got != want).any() else None
+    # the LRU model of the reference on the same requests, one eviction group per layer
+    lru = {l: o.LruModel(resident=list(range(8 - per_layer, 8)), offloaded=list(range(8 - per_layer))) for l in range(32)}
+    for req in requests:
+        layer = req[0][0]
+        assert all(u[0] == layer for u in req)
+        lru[layer].load([u[1] for u in req])
+    st = cache.stats()
+    assert st["hits"] == sum(m.hits for m in lru.values())
+    assert st["misses"] == sum(m.misses for m in lru.values())
+    assert st["bytes_copied"] == st["misses"] * cache.module_size
+    for l in range(32):
+        g = cache.group_infos[l]
+        assert sorted(i.index for i in g.members if not i.offloaded) == sorted(lru[l].main)
+    # the prompt asked for more experts of a layer than it has places: the case where a call evicts its own hits
+    assert max(len(r) for r in requests) > per_layer
+    del model
+    torch.cuda.empty_cache()

@@ -167,7 +167,12 @@ def test_full_size_against_dequantize_then_matmul(nbits, n, k, gs, m):
     atol = 1e-3 * x.float().norm(dim=1)[:, None] * w.norm(dim=1)[None, :]
     err = (y.float() - ref).abs()
     bound = 1e-2 * ref.abs() + atol + ref.abs() * 2.0 ** -11  # + fp16 rounding of the reference itself
-    assert bool((err <= bound).all()), float((err / bound).max())
+    worst = float((err / bound).max())
+    print(f"w{nbits} {n}x{k} M={m}: worst err/bound {worst:.4f}")
+    assert bool((err <= bound).all()), worst
+    # headroom: measured 0.01-0.03 at these shapes (a correctly rounded fp16 result gives about 0.012); a kernel
+    # that loses precision inside the tolerance (activations folded with the scale are held in fp16) shows up here
+    assert worst <= 0.1, worst
     # linearity: doubling x doubles y (exactly for kernels whose intermediates stay in normal range; the kernels
     # that hold scale*x in fp16 may differ by an fp16 rounding of a few tiny terms)
     y2 = hip_kernels.matmul(desc, (x * 2).contiguous())
