@@ -215,13 +215,39 @@ def survey_section(dev):
             stream.synchronize()
         return e0.elapsed_time(e1) * 1e3 / iters
 
-    def add(name, us, nbytes, flops=None):
+    # the ceiling of a launch of a given size: a plain 128-bit streaming read of that many bytes, timed the same way
+    # (rotating over more than 256 MB), cached per size
+    pool = torch.empty(768 << 20, dtype=torch.uint8, device=dev).fill_(3)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    ceilings = {}
+
+    def stream_us(nbytes):
+        key = (int(nbytes) + (1 << 20) - 1) >> 20  # per MiB
+        if key not in ceilings:
+            span = (int(nbytes) + 4095) // 4096 * 4096
+            slots = max(1, pool.numel() // span)
+
+            def f(i):
+                rc = lib.hqq_probe_stream_read(pool.data_ptr() + (i % slots) * span, int(nbytes), sink.data_ptr(), stream.cuda_stream)
+                if rc != 0:
+                    raise _lib.HqqError(rc, "hqq_probe_stream_read")
+
+            ceilings[key] = timed(f, 48)
+        return ceilings[key]
+
+    def add(name, us, nbytes, flops=None, ceiling=False):
         r = {"kernel": name, "us": round(us, 2), "GB_s": round(nbytes / us / 1e3, 0), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)}
+        if ceiling:
+            c = stream_us(nbytes)
+            r["stream_read_same_bytes_us"] = round(c, 2)
+            r["frac_of_stream_read"] = round(c / us, 3)
         if flops:
             r["TFLOP_s"] = round(flops / us / 1e6, 1)
             r["frac_mfma_f16"] = round(flops / us / 1e6 / 2500.0, 3)
         rows.append(r)
-        print(f"{name:58s} {us:9.2f} us {r['GB_s']:8.0f} GB/s" + (f" {r['TFLOP_s']:8.1f} TFLOP/s" if flops else ""), file=sys.stderr, flush=True)
+        print(f"{name:58s} {us:9.2f} us {r['GB_s']:8.0f} GB/s" + (f" {r['TFLOP_s']:8.1f} TFLOP/s" if flops else "")
+              + (f"  stream read of the same bytes {r['stream_read_same_bytes_us']:.2f} us ({r['frac_of_stream_read']:.2f})" if ceiling else ""),
+              file=sys.stderr, flush=True)
 
     shapes = [(4, 4096, 4096, 64, (1, 4, 16, 128, 512)), (4, 1024, 4096, 64, (1,)), (2, 14336, 4096, 16, (1, 4, 16, 128, 512)),
               (2, 4096, 14336, 16, (1, 4, 16, 128, 512)), (3, 14336, 4096, 64, (1, 8, 128)), (3, 4096, 14336, 64, (1, 8, 128))]
@@ -257,7 +283,8 @@ def survey_section(dev):
                     raise _lib.HqqError(rc, "hqq_matmul_transpose")
 
             fam = lib.hqq_matmul_kernel_family(layers[0].ref, m)
-            add(f"matmul {tag} M={m} (family {fam})", timed(f, 48 if m <= 16 else 16), wbytes + 2 * m * (n + k), 2.0 * m * n * k)
+            add(f"matmul {tag} M={m} (family {fam})", timed(f, 48 if m <= 16 else 16), wbytes + 2 * m * (n + k), 2.0 * m * n * k,
+                ceiling=m <= 16)
         del layers
         torch.cuda.empty_cache()
     return rows
@@ -339,6 +366,19 @@ def decode_section(dev, tokens_resident=256, tokens_offload=256):
             out[f"expert_cache_{per_layer}_per_layer_detail"] = {
                 "tokens": tokens_offload, "hits": st["hits"] - before["hits"], "misses": st["misses"] - before["misses"],
                 "GB_copied_host_to_device": round((st["bytes_copied"] - before["bytes_copied"]) / 1e9, 2)}
+            # the same with speculative loads: the next layer's router applied one layer early picks what to prefetch
+            model.speculate = True
+            before = model.expert_cache.stats()
+            spec_tokens = 64
+            out[f"expert_cache_{per_layer}_per_layer_speculative_tok_s"] = round(timed_eager(model, spec_tokens), 2)
+            st = model.expert_cache.stats()
+            loads = st["prefetch_loads"] - before["prefetch_loads"]
+            out[f"expert_cache_{per_layer}_per_layer_speculative_detail"] = {
+                "tokens": spec_tokens, "prefetch_loads": loads,
+                "guess_accuracy": round((st["prefetch_useful"] - before["prefetch_useful"]) / max(1, loads), 3),
+                "misses": st["misses"] - before["misses"],
+                "GB_copied_host_to_device": round((st["bytes_copied"] - before["bytes_copied"]) / 1e9, 2)}
+            model.speculate = False
         del model
         gc.collect()
         torch.cuda.empty_cache()

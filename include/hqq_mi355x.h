@@ -230,6 +230,11 @@ int hqq_attention_decode(const void *q_f16, const void *k_f16, const void *v_f16
                          const int64_t *pos, void *cache_k_f16, void *cache_v_f16, int64_t max_len, int32_t n_heads,
                          int32_t n_kv_heads, int32_t head_dim, void *out_f16, void *stream);
 
+/* ---- measurement aid, no counterpart in the reference: a plain 128-bit streaming read of `bytes` bytes (16-byte aligned)
+ *      that computes nothing; sink_u32 is one device word that is never written in practice.  Its duration is the
+ *      ceiling for any launch that must fetch the same bytes, which is what bench.py --survey prints beside each GEMV. */
+int hqq_probe_stream_read(const void *src, size_t bytes, void *sink_u32, void *stream);
+
 /* ---- which kernel family a call would use (for tests and profiles): 0 general, 1 MFMA small-batch, 2 MFMA tile,
  *      3 three-bit vector kernel.                                                                                     */
 int hqq_matmul_kernel_family(const hqq_linear *l, int64_t M);

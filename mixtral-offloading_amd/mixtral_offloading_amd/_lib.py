@@ -77,6 +77,7 @@ _SIGNATURES = {
                                        c_void_p, c_void_p, c_void_p, c_void_p]),
     "hqq_attention_decode": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
+    "hqq_probe_stream_read": (c_int, [c_void_p, c_size_t, c_void_p, c_void_p]),
     "hqq_slab_h2d_async": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
     "hqq_stream_wait_event": (c_int, [c_void_p, c_void_p]),
     "hqq_lru_create": (c_void_p, [c_int32, c_int32]),

@@ -251,11 +251,13 @@ class SparseMoeWrapper(nn.Module):
 
     @torch.inference_mode()
     def forward_routed(self, hidden_states: torch.Tensor, selected: torch.Tensor, weights: torch.Tensor,
-                       out: torch.Tensor) -> torch.Tensor:
+                       out: torch.Tensor, chosen=None) -> torch.Tensor:
         """One token whose router has already run on the device (``hip_kernels.add_rmsnorm_router``): ``selected``
         int32[2] and ``weights`` fp16[2] are device tensors.  The host reads the choice (the one synchronisation of the
-        layer, as the cache is driven from the host), loads what is missing and runs the experts into ``out``."""
-        chosen = selected.cpu().tolist()
+        layer, as the cache is driven from the host; ``chosen`` hands it in when the caller has read it already),
+        loads what is missing and runs the experts into ``out``."""
+        if chosen is None:
+            chosen = selected.cpu().tolist()
         first = True
         for (_layer_index, expert_idx), expert_layer in self.experts.load_experts(
                 *((self.layer_id, expert_idx) for expert_idx in sorted(set(chosen))), unordered=True):

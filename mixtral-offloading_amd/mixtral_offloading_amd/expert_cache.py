@@ -59,6 +59,9 @@ class EvictionGroup:
         self.members: List[ExpertInfo] = []
         self.global_slot: List[int] = []  # local slot -> global device slot
         self.evictable = False  # true once an expert of the group is offloaded: residents can then be evicted
+        # requests made by speculative prefetches, kept apart so that hits / misses count real requests only
+        self.spec_hits = 0
+        self.spec_misses = 0
 
     def __del__(self):
         if getattr(self, "_lru", None):
@@ -67,11 +70,11 @@ class EvictionGroup:
 
     @property
     def hits(self) -> int:
-        return _lib.lib.hqq_lru_hits(self._lru)
+        return _lib.lib.hqq_lru_hits(self._lru) - self.spec_hits
 
     @property
     def misses(self) -> int:
-        return _lib.lib.hqq_lru_misses(self._lru)
+        return _lib.lib.hqq_lru_misses(self._lru) - self.spec_misses
 
     def slot_of(self, index: int) -> int:
         return _lib.lib.hqq_lru_slot_of(self._lru, index)
@@ -112,6 +115,13 @@ class ExpertCache:
         self._init_device_side()
         self._used = [False] * len(self.slots)
         self.bytes_copied = 0
+        self._copy_pending = set()  # slots filled by a copy that the compute stream has not been made to wait for yet
+        # speculative prefetches: experts loaded on a guess and not asked for yet, and how the guesses turned out
+        self._speculative = set()
+        self.prefetch_loads = 0   # copies started on a guess
+        self.prefetch_useful = 0  # of those, experts that a real request then found on the device
+        self.copy_trace = None    # a list: (uid, start event, end event, kind) of every copy, for tests that look at overlap
+        self._copy_kind = "demand"
 
     # ---- the device side, kept apart so that the scheduling above it can be driven on a machine without a GPU
     def _init_device_side(self) -> None:
@@ -129,9 +139,15 @@ class ExpertCache:
     def _copy_in(self, info: ExpertInfo, slot: int) -> None:
         dst = self.slots[slot].storage
         with torch.cuda.device(self.device):
+            if self.copy_trace is not None:
+                t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                t0.record(self.copy_stream)
             _lib.check(_lib.lib.hqq_slab_h2d_async(dst.data_ptr(), info.host_slab.data_ptr(), self.module_size,
                                                    self.copy_stream.cuda_stream, None), "hqq_slab_h2d_async")
             self.ready[slot].record(self.copy_stream)
+            if self.copy_trace is not None:
+                t1.record(self.copy_stream)
+                self.copy_trace.append((info.uid, t0, t1, self._copy_kind))
 
     def _check_module(self, module: MixtralExpertWrapper):
         assert isinstance(module.storage, torch.UntypedStorage)
@@ -220,6 +236,7 @@ class ExpertCache:
         order, local_slots, victims = group.plan([info.index for info in infos])
         compute = self._compute_stream()
         miss = {idx: victim >= 0 for idx, victim in zip(order, victims)}
+        self._settle_speculation(group, order, victims, real=True)
         local_of = dict(zip(order, local_slots))
         sequence = order if unordered else [info.index for info in infos]
         rank = {idx: i for i, idx in enumerate(sequence)}
@@ -237,6 +254,7 @@ class ExpertCache:
                 self.copy_stream.wait_event(self.released[dst])
             self._copy_in(group.members[idx], dst)
             self.bytes_copied += self.module_size
+            self._copy_pending.add(dst)
             slot_for[idx] = dst
             holder[dst] = idx
             copied.add(idx)
@@ -291,8 +309,9 @@ class ExpertCache:
                         raise RuntimeError("internal error: caching algorithm failed")
                     start_load(to_load.popleft(), force=True)
                 slot = slot_for[idx]
-                if idx in copied:
+                if slot in self._copy_pending:  # filled by this call, or by a prefetch nobody has waited for yet
                     compute.wait_event(self.ready[slot])
+                    self._copy_pending.discard(slot)
                 yield (group.members[idx].uid, self.slots[slot])
                 self.released[slot].record(compute)
                 self._used[slot] = True
@@ -304,6 +323,60 @@ class ExpertCache:
             while to_load:
                 start_load(to_load.popleft(), force=True)
             self.active = False
+
+    def _settle_speculation(self, group: EvictionGroup, order, victims, real: bool) -> None:
+        """Book-keeping of guesses after a plan: a real request that finds a speculatively loaded expert makes that
+        guess useful; an expert evicted before anyone asked for it was a wasted one."""
+        gid = id(group)
+        for idx, victim in zip(order, victims):
+            if victim >= 0:
+                self._speculative.discard((gid, victim))
+            if real and (gid, idx) in self._speculative:
+                self._speculative.discard((gid, idx))
+                if victim < 0:
+                    self.prefetch_useful += 1
+
+    def prefetch(self, *uids: ExpertUID) -> int:
+        """Start loading the given experts of one eviction group on a guess (the reference lists speculative loading
+        as not yet available, README.md:24-26).  It is a request like any other to the LRU policy -- the experts become
+        most recently used, misses evict the least recently used residents -- except that nothing is handed out and
+        hits / misses are not counted: the copies run on the side stream and whoever asks for the expert later finds
+        it on the device.  Returns the number of copies started."""
+        assert not self.active, "already loading experts; buffers are busy"
+        infos = [self.registered_experts[uid] for uid in dict.fromkeys(uids)]
+        if not infos:
+            return 0
+        assert len(set(info.eviction_group for info in infos)) == 1, "experts must be in the same evicton group"
+        group = self.group_infos[infos[0].eviction_group]
+        before = (_lib.lib.hqq_lru_hits(group._lru), _lib.lib.hqq_lru_misses(group._lru))
+        order, local_slots, victims = group.plan([info.index for info in infos])
+        group.spec_hits += _lib.lib.hqq_lru_hits(group._lru) - before[0]
+        group.spec_misses += _lib.lib.hqq_lru_misses(group._lru) - before[1]
+        self._settle_speculation(group, order, victims, real=False)
+        started = 0
+        for idx, local, victim in zip(order, local_slots, victims):
+            if victim < 0:
+                continue
+            home = group.global_slot[local]
+            if self.spare:
+                dst = self.spare.popleft()
+                self.spare.append(home)
+                group.global_slot[local] = dst
+            else:
+                dst = home
+            if self._used[dst]:
+                self.copy_stream.wait_event(self.released[dst])
+            self._copy_kind = "prefetch"
+            try:
+                self._copy_in(group.members[idx], dst)
+            finally:
+                self._copy_kind = "demand"
+            self.bytes_copied += self.module_size
+            self._copy_pending.add(dst)
+            self._speculative.add((id(group), idx))
+            started += 1
+        self.prefetch_loads += started
+        return started
 
     def resident_group(self, eviction_group: int) -> Optional[List[MixtralExpertWrapper]]:
         """The device modules of every expert of a group, in expert order, when all of them are resident and none
@@ -322,4 +395,5 @@ class ExpertCache:
     # convenience counters (the reference keeps hits / misses per EvictionGroupInfo)
     def stats(self) -> Dict[str, int]:
         return {"hits": sum(g.hits for g in self.group_infos.values()),
-                "misses": sum(g.misses for g in self.group_infos.values()), "bytes_copied": self.bytes_copied}
+                "misses": sum(g.misses for g in self.group_infos.values()), "bytes_copied": self.bytes_copied,
+                "prefetch_loads": self.prefetch_loads, "prefetch_useful": self.prefetch_useful}

@@ -279,10 +279,12 @@ class MixtralForCausalLM(nn.Module):
             cfg, mk = self.config, dict(device=self.device)
             row = lambda n: torch.zeros((1, n), dtype=torch.float16, **mk)  # noqa: E731
             st = dict(x=row(cfg.hidden_size), x2=row(cfg.hidden_size), xn=row(cfg.hidden_size), moe=row(cfg.hidden_size),
-                      att=row(cfg.hidden_size), sel=torch.zeros(2, dtype=torch.int32, **mk),
+                      att=row(cfg.hidden_size), sel4=torch.zeros(4, dtype=torch.int32, **mk),
+                      guess_w=torch.zeros(2, dtype=torch.float16, **mk),
                       rw=torch.zeros(2, dtype=torch.float16, **mk), pos=torch.zeros(1, dtype=torch.int64, **mk),
                       qkv=[hip_kernels.LinearGroup([p._desc() for p in (l.self_attn.q_proj, l.self_attn.k_proj, l.self_attn.v_proj)])
                            for l in self.model.layers])
+            st["sel"], st["guess"] = st["sel4"][0:2], st["sel4"][2:4]  # one copy to the host brings both
             self._token_bufs = st
         return st
 
@@ -298,6 +300,9 @@ class MixtralForCausalLM(nn.Module):
             raise ValueError("the single-token step takes top-2 routing and a position inside the cache")
         eps = cfg.rms_norm_eps
         x, spare, xn, moe = st["x"], st["x2"], st["xn"], st["moe"]
+        # speculative expert loads (self.speculate, off by default): the next layer's experts are guessed one layer ahead
+        speculate = bool(getattr(self, "speculate", False))
+        trace = getattr(self, "attention_trace", None)  # a list: (layer, start event, end event) around each attention
         st["pos"].fill_(start)
         x.copy_(self.model.embed_tokens(token.view(1)))
         delta = None
@@ -312,10 +317,25 @@ class MixtralForCausalLM(nn.Module):
             else:
                 hip_kernels.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps, xn)
                 q, k, v = attn.q_proj(xn), attn.k_proj(xn), attn.v_proj(xn)
+            if trace is not None:
+                trace.append((i, torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)))
+                trace[-1][1].record()
             out = hip_kernels.attention_decode(q, k, v, self.rotary.cos, self.rotary.sin, st["pos"], ck, cv, st["att"])
+            if trace is not None:
+                trace[-1][2].record()
+            moe_block = layer.block_sparse_moe
             hip_kernels.add_rmsnorm_router(x, attn.o_proj(out), layer.post_attention_layernorm.weight, eps, xn,
-                                           layer.block_sparse_moe.gate.weight, st["sel"], st["rw"])
-            layer.block_sparse_moe.forward_routed(xn, st["sel"], st["rw"], moe)
+                                           moe_block.gate.weight, st["sel"], st["rw"])
+            nxt = self.model.layers[i + 1].block_sparse_moe if speculate and i + 1 < len(self.model.layers) else None
+            if nxt is not None:
+                # the guess for the next layer: its router applied to this layer's post-attention state
+                hip_kernels.router_top2(xn, nxt.gate.weight, st["guess"], st["guess_w"])
+                both = st["sel4"].cpu().tolist()  # the layer's one synchronisation
+                moe_block.forward_routed(xn, st["sel"], st["rw"], moe, chosen=both[:2])
+                # started now, before the host goes on to the next layer's attention: the copies overlap it
+                nxt.experts.prefetch(*((nxt.layer_id, e) for e in sorted(set(both[2:]))))
+            else:
+                moe_block.forward_routed(xn, st["sel"], st["rw"], moe)
             delta = moe
         hip_kernels.add_rmsnorm(x, delta, self.model.norm.weight, eps, xn)
         return self.lm_head(xn)

@@ -9,11 +9,11 @@ pytestmark = pytest.mark.gpu
 
 
 def _small_setup(layers=2, hidden=256, ffn=512, experts=8, vocab=128, offload_per_layer=6, main_per_layer=2,
-                 buffers=2, seed=0, ffn_bits=2):
+                 buffers=2, seed=0, ffn_bits=2, heads=4, kv_heads=2):
     from mixtral_offloading_amd import build_model as bm
     from mixtral_offloading_amd.hqq_core import BaseQuantizeConfig
-    cfg = bm.mixtral_config(hidden_size=hidden, intermediate_size=ffn, num_hidden_layers=layers, num_attention_heads=4,
-                            num_key_value_heads=2, vocab_size=vocab, num_local_experts=experts)
+    cfg = bm.mixtral_config(hidden_size=hidden, intermediate_size=ffn, num_hidden_layers=layers, num_attention_heads=heads,
+                            num_key_value_heads=kv_heads, vocab_size=vocab, num_local_experts=experts)
     off = bm.OffloadConfig(main_size=layers * main_per_layer, offload_size=layers * offload_per_layer,
                            buffer_size=buffers, offload_per_layer=offload_per_layer)
     qc = bm.default_quant_config()
@@ -238,3 +238,47 @@ def test_single_token_step_equals_the_layerwise_forward(offload_per_layer):
         assert float((ka.float() - kb.float()).abs().max()) <= 2e-2 and float((va.float() - vb.float()).abs().max()) <= 2e-2
     with pytest.raises(ValueError):
         model.forward_token(tok, cache_a, 32)  # past the cache
+
+
+def test_speculative_prefetch_overlaps_attention_and_keeps_the_tokens():
+    """Speculative expert loads (the reference lists them as not yet available, README.md:24-26): the next layer's
+    router is applied to this layer's post-attention state and the guessed experts start loading before the next
+    layer's attention is launched.  The router is made predictable by construction -- a residual stream so large that
+    a layer barely changes it, so consecutive layers see nearly the same normed state -- and the test checks that the
+    guesses are mostly right, that the guessed copies run while the next layer's attention does, and that the tokens
+    are those of the run without speculation."""
+    def run(speculate):
+        # experts of 19 MB: a copy takes a few hundred microseconds, longer than the host needs to launch the next
+        # layer's attention
+        model, cfg = _small_setup(layers=4, hidden=2048, ffn=8192, offload_per_layer=6, main_per_layer=2, buffers=4, seed=21,
+                                  heads=16, kv_heads=4)
+        model.model.embed_tokens.weight.data.mul_(2000.0)  # hidden states of size 40 against layer outputs of size 1
+        model.speculate = speculate
+        cache = model.expert_cache
+        cache.copy_trace, model.attention_trace = [], []
+        base = torch.cuda.Event(enable_timing=True)
+        base.record()
+        prompt = torch.randint(0, cfg.vocab_size, (5,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(3))
+        tokens = model.generate(prompt, 16)
+        torch.cuda.synchronize()
+        return model, tokens, base
+
+    plain, want, _ = run(False)
+    assert plain.expert_cache.stats()["prefetch_loads"] == 0
+    spec, got, base = run(True)
+    assert torch.equal(got, want)
+    st, st_plain = spec.expert_cache.stats(), plain.expert_cache.stats()
+    assert st["prefetch_loads"] > 10
+    # predictable by construction: most guesses are asked for next
+    assert st["prefetch_useful"] >= 0.7 * st["prefetch_loads"], st
+    # experts that arrived on a guess are hits of the real requests: fewer real misses than without speculation
+    assert st["misses"] < st_plain["misses"] and st["hits"] + st["misses"] == st_plain["hits"] + st_plain["misses"]
+    assert st["bytes_copied"] == (st["misses"] + st["prefetch_loads"]) * spec.expert_cache.module_size
+    # overlap: a copy started on a guess for layer L+1 is in flight while layer L+1's attention runs
+    att = [(layer, base.elapsed_time(a), base.elapsed_time(b)) for layer, a, b in spec.attention_trace]
+    copies = [(uid, base.elapsed_time(a), base.elapsed_time(b)) for uid, a, b, kind in spec.expert_cache.copy_trace if kind == "prefetch"]
+    assert copies
+    overlapping = 0
+    for (layer, e), c0, c1 in copies:
+        overlapping += any(l == layer and a0 < c1 and c0 < a1 for l, a0, a1 in att)
+    assert overlapping >= 0.5 * len(copies), (overlapping, len(copies))
