@@ -103,7 +103,7 @@ int hqq_dequantize(const hqq_linear *l, void *w_out_f16, void *stream);
 size_t hqq_matmul_workspace_bytes(const hqq_linear *l, int64_t M);
 /* zero the head (counters and slots) of a workspace with a small fill kernel (safe under stream capture)            */
 int hqq_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
-/* same, with the kernel family forced (-1 = automatic choice, else 0..3 as hqq_matmul_kernel_family reports):
+/* same, with the kernel family forced (-1 = automatic choice, else 0..4 as hqq_matmul_kernel_family reports):
  * HQQ_E_UNSUPPORTED when that family does not take the configuration.  For tests and profiling.                    */
 int hqq_matmul_transpose_ex(const hqq_linear *l, const void *x_f16, int64_t M, void *y_f16, void *workspace,
                             size_t workspace_bytes, int family, void *stream);
@@ -236,7 +236,8 @@ int hqq_attention_decode(const void *q_f16, const void *k_f16, const void *v_f16
 int hqq_probe_stream_read(const void *src, size_t bytes, void *sink_u32, void *stream);
 
 /* ---- which kernel family a call would use (for tests and profiles): 0 general, 1 MFMA small-batch, 2 MFMA tile,
- *      3 three-bit vector kernel.                                                                                     */
+ *      3 three-bit vector kernel, 4 MFMA kernel with weights dequantised into shared memory (reads 3-bit words as
+ *      they are stored).                                                                                              */
 int hqq_matmul_kernel_family(const hqq_linear *l, int64_t M);
 
 /* ---- expert offload: replaces the two copies of ExpertCache._swap (src/expert_cache.py:186-189).

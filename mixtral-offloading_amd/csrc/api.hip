@@ -41,7 +41,7 @@ int validate_linear(const hqq_linear *l)
 
 static inline size_t align256(size_t v) { return (v + 255u) & ~(size_t)255u; }
 
-enum { FAM_GENERAL = 0, FAM_SMALLBATCH = 1, FAM_TILE = 2, FAM_VEC3 = 3 };
+enum { FAM_GENERAL = 0, FAM_SMALLBATCH = 1, FAM_TILE = 2, FAM_VEC3 = 3, FAM_LDS = 4 };
 constexpr int64_t kSmallBatchMax = 16;
 
 // a batch wider than the small-batch kernels take, run as slices of 16 rows (the weights of the later slices come
@@ -52,7 +52,9 @@ static int pick_family(const hqq_linear *l, int64_t M)
 {
     if (strip_supported(l, M)) // decode batches: part of the small-batch family
         return FAM_SMALLBATCH;
-    if (l->nbits == 3 && tile_supported(l, M)) // five rows and more: 3-bit codes rewritten as 4-bit ones, then the tile kernel
+    if (l->nbits == 3 && M >= 5 && M <= kSmallBatchMax && ldsgemm_supported(l, M)) // 3-bit words read as they are stored
+        return FAM_LDS;
+    if (l->nbits == 3 && tile_supported(l, M)) // wider batches: 3-bit codes rewritten as 4-bit ones, then the tile kernel
         return FAM_TILE;
     if (vec3_supported(l, M))
         return FAM_VEC3;
@@ -62,6 +64,8 @@ static int pick_family(const hqq_linear *l, int64_t M)
         return FAM_SMALLBATCH;
     if (sliced_supported(l, M))
         return FAM_SMALLBATCH;
+    if (M >= 5 && ldsgemm_supported(l, M)) // e.g. 3-bit layers whose group count the tile kernel does not take
+        return FAM_LDS;
     return FAM_GENERAL;
 }
 
@@ -73,6 +77,8 @@ static size_t family_workspace(const hqq_linear *l, int64_t M, int fam)
         return vec3_workspace_bytes(l, M);
     if (fam == FAM_TILE)
         return tile_workspace_bytes(l, M);
+    if (fam == FAM_LDS)
+        return ldsgemm_workspace_bytes(l, M);
     return 0;
 }
 
@@ -97,6 +103,8 @@ static int run_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void
         return launch_vec3_matmul(l, x, M, y, ws, ws_bytes, s);
     case FAM_TILE:
         return launch_tile_matmul(l, x, M, y, ws, ws_bytes, s);
+    case FAM_LDS:
+        return launch_ldsgemm_matmul(l, x, M, y, ws, ws_bytes, s);
     default:
         return launch_general_matmul(l, x, M, y, s);
     }
@@ -147,6 +155,9 @@ size_t hqq_matmul_workspace_bytes(const hqq_linear *l, int64_t M)
     const size_t c = tile_supported(l, M) ? tile_workspace_bytes(l, M) : 0;
     if (c > b)
         b = c;
+    const size_t d = ldsgemm_supported(l, M) ? ldsgemm_workspace_bytes(l, M) : 0;
+    if (d > b)
+        b = d;
     return align256(a > b ? a : b);
 }
 
@@ -178,7 +189,9 @@ int hqq_matmul_transpose_ex(const hqq_linear *l, const void *x_f16, int64_t M, v
         return HQQ_E_UNSUPPORTED;
     if (fam == FAM_TILE && !tile_supported(l, M))
         return HQQ_E_UNSUPPORTED;
-    if (fam < 0 || fam > FAM_VEC3)
+    if (fam == FAM_LDS && !ldsgemm_supported(l, M))
+        return HQQ_E_UNSUPPORTED;
+    if (fam < 0 || fam > FAM_LDS)
         return HQQ_E_UNSUPPORTED;
     const size_t need = family_workspace(l, M, fam);
     if (need > 0 && (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)))
@@ -259,7 +272,8 @@ int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, i
     const bool alike = w1->nbits == w3->nbits && w1->group_size == w3->group_size;
     // one fused launch where a kernel family has one for the batch; the decode kernels need no more workspace than
     // they check for themselves
-    const bool prefer_tile = tile_supported(w1, M) && tile_supported(w3, M) && !strip_supported(w1, M);
+    const bool prefer_tile = tile_supported(w1, M) && tile_supported(w3, M) && !strip_supported(w1, M) &&
+                             pick_family(w1, M) != FAM_LDS && pick_family(w3, M) != FAM_LDS;
     if (alike && !prefer_tile && smallbatch_supported(w1, M) && smallbatch_supported(w3, M))
         return launch_smallbatch_gate_up(w1, w3, x, M, h, workspace, workspace_bytes, s);
     if (prefer_tile && tile_gate_supported(w1, w3, M))
@@ -321,7 +335,8 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
         return launch_vec3_down(w2, a, b, M, y, mm, mm_bytes, ep, s);
     }
     // fused gate: decode batches always; wider ones only where the tile kernel does not take the shape
-    const bool prefer_tile = tile_supported(w1, M) && tile_supported(w3, M) && !strip_supported(w1, M);
+    const bool prefer_tile = tile_supported(w1, M) && tile_supported(w3, M) && !strip_supported(w1, M) &&
+                             pick_family(w1, M) != FAM_LDS && pick_family(w3, M) != FAM_LDS;
     const bool fast13 = !prefer_tile && smallbatch_supported(w1, M) && smallbatch_supported(w3, M) && !w1->bias &&
                         !w3->bias && w1->nbits == w3->nbits && w1->group_size == w3->group_size;
     if (fast13) {
@@ -348,6 +363,12 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
     }
     if (!row_scale_f16 && !accumulate)
         return run_matmul(w2, h, M, y, mm, mm_bytes, pick_family(w2, M), s);
+    if (pick_family(w2, M) == FAM_LDS) {
+        SmallBatchEpilogue ep; // applied by the kernel's finishing pass over its partial sums
+        ep.row_scale = (const f16 *)row_scale_f16;
+        ep.accumulate = accumulate;
+        return launch_ldsgemm_matmul(w2, h, M, y, mm, mm_bytes, s, &ep);
+    }
     if (pick_family(w2, M) == FAM_TILE && tile_epilogue_supported(w2, M)) {
         SmallBatchEpilogue ep; // the routing weight and the accumulation in the matmul's own epilogue
         ep.row_scale = (const f16 *)row_scale_f16;

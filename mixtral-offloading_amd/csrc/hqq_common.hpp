@@ -185,6 +185,11 @@ bool tile_gate_supported(const hqq_linear *w1, const hqq_linear *w3, int64_t M);
 size_t tile_gate_workspace_bytes(const hqq_linear *w1, const hqq_linear *w3, int64_t M);
 int launch_tile_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
                         size_t ws_bytes, hipStream_t s);
+// MFMA with the de-quantised weights staged in LDS (2-, 3- and 4-bit codes): the kernel of wide batches
+bool ldsgemm_supported(const hqq_linear *l, int64_t M);
+size_t ldsgemm_workspace_bytes(const hqq_linear *l, int64_t M);
+int launch_ldsgemm_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s,
+                          const SmallBatchEpilogue *ep = nullptr);
 bool vec3_supported(const hqq_linear *l, int64_t M);
 size_t vec3_workspace_bytes(const hqq_linear *l, int64_t M);
 int launch_vec3_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s);

@@ -20,7 +20,7 @@ if not os.path.exists(LIB_PATH):
 lib = ctypes.CDLL(LIB_PATH)
 
 HQQ_TABLE_F16, HQQ_TABLE_U8 = 0, 1
-FAM_GENERAL, FAM_SMALLBATCH, FAM_TILE, FAM_VEC3 = 0, 1, 2, 3
+FAM_GENERAL, FAM_SMALLBATCH, FAM_TILE, FAM_VEC3, FAM_LDS = 0, 1, 2, 3, 4
 
 
 class HqqTable(ctypes.Structure):

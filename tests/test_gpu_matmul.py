@@ -51,7 +51,7 @@ def test_matmul_auto_family(shape, m):
     _check(layer, x)
 
 
-@pytest.mark.parametrize("family", [0, 1, 2, 3])
+@pytest.mark.parametrize("family", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "w%d_%dx%d_g%d" % s[:4])
 def test_matmul_forced_family(shape, family):
     """Every family that accepts a configuration must meet the same tolerance."""
@@ -95,6 +95,48 @@ def test_tile_family_edges(shape, m):
     x = rng.standard_normal((m, k)).astype(np.float16)
     bias = rng.standard_normal(n).astype(np.float16) if m % 2 else None
     _check(layer, x, family=2, bias=bias)  # a refusal (HqqError) fails the test: these shapes are the family's own
+
+
+# the shared-memory family (4) at its edges: 3-bit words read as stored (a word count that is no multiple of the window
+# period, a last word with unused fields, ten table rows and more), 2- and 4-bit tiles of eight table rows, 8-bit and
+# fp16 tables, every batch tile width, K of one to several groups of four steps so that the split over K varies
+LDS_SHAPES = [
+    (3, 1280, 256, 64, 128, True, True),
+    (3, 1296, 512, 54, 128, True, True),
+    (3, 640, 1024, 64, 128, False, False),
+    (3, 2960, 256, 37, 128, True, True),
+    (2, 1024, 256, 16, 128, True, True),
+    (2, 512, 1280, 32, 128, False, False),
+    (4, 1024, 512, 64, 128, True, True),
+    (4, 512, 2048, 16, 128, False, False),
+]
+
+
+@pytest.mark.parametrize("shape", LDS_SHAPES, ids=lambda s: "w%d_%dx%d_g%d_%s" % (s[:4] + ("q" if s[5] else "f16",)))
+@pytest.mark.parametrize("m", [5, 16, 17, 33, 64, 65, 129, 200])
+def test_shared_memory_family_edges(shape, m):
+    nbits, n, k, gs, mgs, qs, qz = shape
+    rng = np.random.default_rng(2 * n + k + m)
+    layer, _ = o.random_layer(rng, n, k, nbits, gs, qs, qz, meta_group_size=mgs)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    bias = rng.standard_normal(n).astype(np.float16) if m % 2 else None
+    _check(layer, x, family=4, bias=bias)  # a refusal (HqqError) fails the test: these shapes are the family's own
+
+
+def test_three_bit_small_batches_read_the_stored_words():
+    """Five to sixteen rows of a 3-bit layer go to the family that reads the packed words as they are, not to the one
+    that first rewrites them as 4-bit codes; wider batches and decode batches keep their kernels."""
+    from mixtral_offloading_amd import _lib
+    rng = np.random.default_rng(77)
+    layer, _ = o.random_layer(rng, 1024, 512, 3, 64, True, True)
+    desc = desc_of(layer)
+    fam = {m: _lib.lib.hqq_matmul_kernel_family(desc.ref, m) for m in (1, 4, 5, 8, 16, 17, 64)}
+    assert fam[5] == fam[8] == fam[16] == 4
+    assert fam[1] == fam[4] == 3 and fam[17] == fam[64] == 2
+    # twenty groups: the rewrite to 4-bit codes does not take them, the stored words are read at every batch from five
+    layer, _ = o.random_layer(rng, 1280, 512, 3, 64, True, True)
+    desc = desc_of(layer)
+    assert [_lib.lib.hqq_matmul_kernel_family(desc.ref, m) for m in (4, 5, 17, 300)] == [3, 4, 4, 4]
 
 
 def test_bias_leading_dims_and_empty():
