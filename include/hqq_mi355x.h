@@ -230,6 +230,25 @@ int hqq_attention_decode(const void *q_f16, const void *k_f16, const void *v_f16
                          const int64_t *pos, void *cache_k_f16, void *cache_v_f16, int64_t max_len, int32_t n_heads,
                          int32_t n_kv_heads, int32_t head_dim, void *out_f16, void *stream);
 
+/* ---- the attention part of a decoder layer at one token as ONE launch: hqq_matmul_group_norm (input norm + q, k, v
+ *      of x + delta, x + delta to x_sum), hqq_attention_decode and hqq_matmul_transpose (o_proj) into y, with the same
+ *      bits as those three calls.  The parts run as blocks of one grid in that order and hand over through the scratch
+ *      rows q/k/v/att (n_heads*head_dim, n_kv_heads*head_dim twice, n_heads*head_dim halves) and counters in the
+ *      workspace head (hqq_workspace_init once; at least hqq_attention_chain_workspace_bytes()): the output projection
+ *      has fetched its weights by the time the heads are done.  (HF transformers' Mixtral attention in the reference;
+ *      the projections are src/custom_layers.py:55-92.)  HQQ_E_UNSUPPORTED for shapes outside it (then make the three
+ *      calls): 4-bit projections without bias whose K fits one block (K <= 4096), head_dim 128, max_len <= 4096.
+ *      A wait that does not end (it cannot, by the order of the blocks) gives up after about a quarter of a second and
+ *      sets the int at hqq_attention_chain_error_offset() bytes into the workspace, which is otherwise zero.          */
+size_t hqq_attention_chain_workspace_bytes(void);
+size_t hqq_attention_chain_error_offset(void);
+int hqq_attention_chain(const hqq_linear *q, const hqq_linear *k, const hqq_linear *v, const hqq_linear *o, const void *x_f16,
+                        const void *delta_f16, const void *norm_weight_f16, float eps, void *x_sum_f16, void *q_scratch_f16,
+                        void *k_scratch_f16, void *v_scratch_f16, void *att_scratch_f16, const void *cos_f16,
+                        const void *sin_f16, const int64_t *pos, void *cache_k_f16, void *cache_v_f16, int64_t max_len,
+                        int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, void *y_f16, void *workspace,
+                        size_t workspace_bytes, void *stream);
+
 /* ---- measurement aid, no counterpart in the reference: a plain 128-bit streaming read of `bytes` bytes (16-byte aligned)
  *      that computes nothing; sink_u32 is one device word that is never written in practice.  Its duration is the
  *      ceiling for any launch that must fetch the same bytes, which is what bench.py --survey prints beside each GEMV. */

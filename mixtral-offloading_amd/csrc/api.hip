@@ -708,4 +708,39 @@ int hqq_attention_decode(const void *q_f16, const void *k_f16, const void *v_f16
                                    n_kv_heads, head_dim, (f16 *)out_f16, (hipStream_t)stream);
 }
 
+size_t hqq_attention_chain_workspace_bytes(void) { return workspace_head_bytes(); }
+
+size_t hqq_attention_chain_error_offset(void) { return attention_chain_error_offset(); }
+
+int hqq_attention_chain(const hqq_linear *q, const hqq_linear *k, const hqq_linear *v, const hqq_linear *o, const void *x_f16,
+                        const void *delta_f16, const void *norm_weight_f16, float eps, void *x_sum_f16, void *q_scratch_f16,
+                        void *k_scratch_f16, void *v_scratch_f16, void *att_scratch_f16, const void *cos_f16,
+                        const void *sin_f16, const int64_t *pos, void *cache_k_f16, void *cache_v_f16, int64_t max_len,
+                        int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, void *y_f16, void *workspace,
+                        size_t workspace_bytes, void *stream)
+{
+    int rc;
+    if ((rc = validate_linear(q)) != HQQ_OK || (rc = validate_linear(k)) != HQQ_OK || (rc = validate_linear(v)) != HQQ_OK ||
+        (rc = validate_linear(o)) != HQQ_OK)
+        return rc;
+    if (!x_f16 || !norm_weight_f16 || !x_sum_f16 || !q_scratch_f16 || !k_scratch_f16 || !v_scratch_f16 || !att_scratch_f16 ||
+        !cos_f16 || !sin_f16 || !pos || !cache_k_f16 || !cache_v_f16 || !y_f16)
+        return HQQ_E_NULL;
+    if (q->K != k->K || q->K != v->K || o->N != q->K)
+        return HQQ_E_SHAPE;
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u) || workspace_bytes < workspace_head_bytes())
+        return HQQ_E_WORKSPACE;
+    AttentionChain c = {};
+    c.q = q, c.k = k, c.v = v, c.o = o;
+    c.x = (const f16 *)x_f16, c.delta = (const f16 *)delta_f16, c.norm_weight = (const f16 *)norm_weight_f16, c.eps = eps;
+    c.x_sum = (f16 *)x_sum_f16;
+    c.q_out = (f16 *)q_scratch_f16, c.k_out = (f16 *)k_scratch_f16, c.v_out = (f16 *)v_scratch_f16;
+    c.att_out = (f16 *)att_scratch_f16;
+    c.cos_t = (const f16 *)cos_f16, c.sin_t = (const f16 *)sin_f16, c.pos = pos;
+    c.cache_k = (f16 *)cache_k_f16, c.cache_v = (f16 *)cache_v_f16, c.max_len = max_len;
+    c.n_heads = n_heads, c.n_kv_heads = n_kv_heads, c.head_dim = head_dim;
+    c.y = (f16 *)y_f16;
+    return launch_attention_chain(c, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
 } // extern "C"

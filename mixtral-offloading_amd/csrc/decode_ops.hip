@@ -1,5 +1,6 @@
 // Small decode-step kernels around the quantized linears: the router (reference src/custom_layers.py:276-282)
 // and the residual add + RMSNorm of the decoder layer.  One block each: at batch 1 they are latency, not bandwidth.
+#include "attention_parts.hpp"
 #include "hqq_common.hpp"
 #include "norm_route.hpp"
 
@@ -154,14 +155,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_router_once_kernel(f16 *__res
     norm_route_block<CH, NE>(x, delta, weight, eps, x, y, hidden, gate_w, n_experts, sel, weights, logits_out, lds);
 }
 
-// Rotary embedding, KV-cache append and attention of ONE new token (the reference takes them from HF transformers'
-// Mixtral attention): one block per query head.  Roundings follow the fp16 torch ops they replace: rope terms
-// rounded separately, scores = fp16(q . k) then / sqrt(hd) in fp32, softmax in fp32, probabilities cast to fp16,
-// output accumulated in fp32.  The current position is read from device memory, so the launch can be replayed
-// from a graph; positions 0 .. pos are attended (the new key and value are taken from registers, and also
-// written to the cache by the first head of each KV group).
-// One block of NT threads per head: 256 for caches of up to 512 positions, 1024 beyond (the block walks the head's
-// cache rows, so a long cache wants more threads and a short one fewer reduction steps).
+// One block of NT threads per head (attention_parts.hpp): 256 for caches of up to 512 positions, 1024 beyond.
 template <int HD, int NT>
 __global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restrict__ q_in, const f16 *__restrict__ k_in,
                                                                const f16 *__restrict__ v_in, const f16 *__restrict__ cos_t,
@@ -169,160 +163,8 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restr
                                                                f16 *__restrict__ cache_k, f16 *__restrict__ cache_v,
                                                                int64_t max_len, int group, f16 *__restrict__ out)
 {
-    extern __shared__ float score_lds[]; // [pos + 1]
-    __shared__ __attribute__((aligned(16))) f16 q_lds[HD];
-    __shared__ __attribute__((aligned(16))) f16 k_lds[HD];
-    constexpr int NW = NT / 64;
-    __shared__ float red_lds[2 * NW];
-    __shared__ float acc_lds[NT / (HD / 8)][HD];
-    const int h = blockIdx.x, kv = h / group;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    // the new token's q, k and v do not depend on the position: their loads go out before it is waited for
-    const int d = tid < HD ? tid : 0, dr = d < HD / 2 ? d + HD / 2 : d - HD / 2;
-    const f16 qa = q_in[h * HD + d], qb = q_in[h * HD + dr];
-    const f16 ka = k_in[kv * HD + d], kb = k_in[kv * HD + dr];
-    const f16 vnew = v_in[kv * HD + d];
-    const int64_t pos = pos_p[0];
-    if (pos < 0 || pos >= max_len) // the position lives in device memory: a step past the cache must not write past it
-        return;
-    const f16 *cs = cos_t + pos * HD, *sn = sin_t + pos * HD;
-    // the cached key rows of the first four passes only need the position: requested before the rope table arrives
-    // (the row of the new token itself is taken from LDS later)
-    constexpr int LPK = HD / 8, KROWS = NT / LPK;
-    const int ksub = tid / LPK, kc = tid % LPK;
-    f16x8 kfirst[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int64_t l = u * KROWS + ksub;
-        const int64_t lc = l <= pos ? l : pos;
-        kfirst[u] = *reinterpret_cast<const f16x8 *>(cache_k + ((int64_t)kv * max_len + lc) * HD + 8 * kc);
-    }
-    if (tid < HD) {
-        const f16 qr = d < HD / 2 ? -qb : qb, kr = d < HD / 2 ? -kb : kb;
-        const f16 qrot = (f16)(qa * cs[d]) + (f16)(qr * sn[d]);
-        const f16 krot = (f16)(ka * cs[d]) + (f16)(kr * sn[d]);
-        q_lds[d] = qrot;
-        k_lds[d] = krot;
-        if (h % group == 0) {
-            cache_k[((int64_t)kv * max_len + pos) * HD + d] = krot;
-            cache_v[((int64_t)kv * max_len + pos) * HD + d] = vnew;
-        }
-    }
-    __syncthreads();
-
-    // scores: LPK threads share a key row (16 bytes each, so a wave's load covers whole rows), four passes of
-    // KROWS rows in flight; the pieces of a dot product meet through lane exchanges
-    const float inv = 1.0f / __builtin_sqrtf((float)HD);
-    float mx = -3.0e38f;
-    {
-        const f16x8 qq = *reinterpret_cast<const f16x8 *>(q_lds + 8 * kc);
-        for (int64_t l0 = 0; l0 <= pos; l0 += 4 * KROWS) {
-            f16x8 kk[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int64_t l = l0 + u * KROWS + ksub;
-                const int64_t lc = l <= pos ? l : pos;
-                if (lc == pos)
-                    kk[u] = *reinterpret_cast<const f16x8 *>(k_lds + 8 * kc);
-                else if (l0 == 0)
-                    kk[u] = kfirst[u];
-                else
-                    kk[u] = *reinterpret_cast<const f16x8 *>(cache_k + ((int64_t)kv * max_len + lc) * HD + 8 * kc);
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                float acc = 0.f;
-#pragma unroll
-                for (int t = 0; t < 8; ++t)
-                    acc += (float)kk[u][t] * (float)qq[t];
-#pragma unroll
-                for (int off = LPK / 2; off > 0; off >>= 1)
-                    acc += __shfl_xor(acc, off, 64);
-                const int64_t l = l0 + u * KROWS + ksub;
-                if (kc == 0 && l <= pos) {
-                    const float sc = (float)(f16)acc * inv;
-                    score_lds[l] = sc;
-                    mx = fmaxf(mx, sc);
-                }
-            }
-        }
-    }
-    // the value rows of the first four passes do not depend on the scores: requested now, used after the softmax
-    constexpr int LPR = HD / 8, ROWS = NT / LPR;
-    const int rsub = tid / LPR, c8 = tid % LPR;
-    f16x8 vfirst[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int64_t l = u * ROWS + rsub;
-        const int64_t lc = l <= pos ? l : pos;
-        const f16 *vrow = lc == pos ? v_in + kv * HD : cache_v + ((int64_t)kv * max_len + lc) * HD;
-        vfirst[u] = *reinterpret_cast<const f16x8 *>(vrow + 8 * c8);
-    }
-    // block max
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1)
-        mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-    if (lane == 0)
-        red_lds[wave] = mx;
-    __syncthreads();
-    mx = red_lds[0];
-#pragma unroll
-    for (int w = 1; w < NW; ++w)
-        mx = fmaxf(mx, red_lds[w]);
-    float sum = 0.f;
-    for (int64_t l = tid; l <= pos; l += NT) {
-        const float e = __expf(score_lds[l] - mx);
-        score_lds[l] = e;
-        sum += e;
-    }
-    sum = wave_sum(sum);
-    if (lane == 0)
-        red_lds[NW + wave] = sum;
-    __syncthreads();
-    sum = 0.f;
-#pragma unroll
-    for (int w = 0; w < NW; ++w)
-        sum += red_lds[NW + w];
-    const float rs = 1.0f / sum;
-
-    // output: LPR threads share a value row (16 bytes each), the block covers ROWS rows per pass and four passes
-    // are in flight; the ROWS partial outputs meet in LDS
-    float o[8];
-#pragma unroll
-    for (int t = 0; t < 8; ++t)
-        o[t] = 0.f;
-    for (int64_t l0 = 0; l0 <= pos; l0 += 4 * ROWS) {
-        f16x8 vv[4];
-        float pr[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int64_t l = l0 + u * ROWS + rsub;
-            const int64_t lc = l <= pos ? l : pos;
-            if (l0 == 0) {
-                vv[u] = vfirst[u];
-            } else {
-                const f16 *vrow = lc == pos ? v_in + kv * HD : cache_v + ((int64_t)kv * max_len + lc) * HD;
-                vv[u] = *reinterpret_cast<const f16x8 *>(vrow + 8 * c8);
-            }
-            pr[u] = l <= pos ? (float)(f16)(score_lds[lc] * rs) : 0.f;
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-#pragma unroll
-            for (int t = 0; t < 8; ++t)
-                o[t] += pr[u] * (float)vv[u][t];
-    }
-#pragma unroll
-    for (int t = 0; t < 8; ++t)
-        acc_lds[rsub][8 * c8 + t] = o[t];
-    __syncthreads();
-    if (tid < HD) {
-        float a = 0.f;
-#pragma unroll
-        for (int r = 0; r < ROWS; ++r)
-            a += acc_lds[r][tid];
-        out[h * HD + tid] = (f16)a;
-    }
+    attention_head<HD, NT>(q_in, k_in, v_in, cos_t, sin_t, pos_p, cache_k, cache_v, max_len, group, out, (int)blockIdx.x,
+                           CHAIN_NONE, nullptr, 0);
 }
 
 } // namespace

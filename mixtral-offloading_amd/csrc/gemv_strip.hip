@@ -24,6 +24,8 @@
 // Lane roles inside a slab.  Code lanes: (rr = lane & 15, kg = lane >> 4) own packed row jp + (16*rb + rr)*GP,
 // bytes 64*s + 16*kg .. +15 for step s.  Table lanes: (ti = lane >> 4 < F, kq = lane & 15) own table row F*jp + ti,
 // columns 16*kq .. 16*kq+15, i.e. step kq >> 2, MFMA lane group kq & 3.
+#include "attention_parts.hpp"
+#include "chain_parts.hpp"
 #include "gemv_parts.hpp"
 #include "hqq_common.hpp"
 #include "norm_route.hpp"
@@ -84,6 +86,10 @@ struct StripParams {
     int n_experts;
     int *sel_out;
     f16 *rw_out;
+    // Chained launches (the work of several launches in one grid, handed over through device words, see
+    // chain_parts.hpp): the words of the chain and how many blocks of the launch have this one's role.
+    int *chain;
+    int chain_blocks;
 };
 
 template <int MT, int SKIND, int ZKIND> struct SlabRegs {
@@ -100,10 +106,19 @@ template <int MT, int SKIND, int ZKIND> struct SlabRegs {
 // EPI: 0 y = o (+ bias) (* row_scale) (+ y);  1 y = silu(o0) * o1;  2 y = (y +) o0 * row_scale[0] + o1 * row_scale[1]
 // NORM: 0 the activations are x; 1 weight * rmsnorm(x + delta), the mean of squares added up while the weights travel;
 // 2 the same with the router of the normed row in the prologue, whose choice picks the experts of the launch
-template <int NBITS, int MT, int S, int D, int WAVES, int SKIND, int ZKIND, int EPI, bool GROUPED = false, int NORM = 0>
-__global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
+// The block (bx, by, bzi) of the launch described by p.  chain (a constant at every call site): CHAIN_NONE for a launch
+// of its own; CHAIN_FIRST when later blocks of the same grid read this block's output (stored at device scope, then
+// counted); CHAIN_LAST when the activations are produced by earlier blocks of the same grid: the weights are requested
+// first, the activations read (at device scope) once the producers have been counted, and a NORM instantiation then
+// uses them as they are.
+template <int NBITS, int MT, int S, int D, int WAVES, int SKIND, int ZKIND, int EPI, bool GROUPED, int NORM>
+__device__ __forceinline__ void strip_block(const StripParams &p, const int bx, const int by, const int bzi, const int chain)
 {
     static_assert(!NORM || (MT == 1 && WAVES >= 4), "the fused norm is for single rows and blocks of four waves and more");
+    const bool origin = bx == 0 && by == 0 && bzi == 0;
+    const bool normed = NORM != 0 && chain != CHAIN_LAST; // whether the activations go through the norm
+    if (chain == CHAIN_FIRST)
+        CHAIN_STAMP(p.chain, 0);
     constexpr bool ROUTED = NORM == 2;
     constexpr int F = 8 / NBITS;
     constexpr int ENTRY = 8; // halves per B-operand entry (16 bytes)
@@ -135,11 +150,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     // the wave index as a scalar: what depends on it (the layer, its record, the K range) then lives in scalar
     // registers, and the record is picked from the kernel arguments without a memory access of its own
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int kb = blockIdx.x, rb = blockIdx.y;
+    const int kb = bx, rb = by;
     // Batches of three and four rows run as two passes of the two-row kernel inside one launch: blocks 2z and 2z + 1
     // are the two passes of tile z, so both ask for the tile's weights at about the same time and memory delivers
     // them once (how far apart the two are in launch order, 1 to 32 workgroups, made no difference when measured).
-    int bz = (int)blockIdx.z, pass = 0;
+    int bz = bzi, pass = 0;
     if constexpr (MT == 2) {
         if (p.passes == 2) {
             pass = bz & 1;
@@ -158,7 +173,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     float rnorm = 1.0f; // NORM launches: 1 / sqrt(mean(x^2) + eps), known once the block has added the row up
     if constexpr (ROUTED) {
         // every block routes for itself (the router's rows come from L2): which records to read is known only then
-        const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0;
+        const bool writer = origin;
         // the router's scratch shares the code staging buffer, which nothing touches before the first slab is worked
         // on: with an LDS array of its own the block no longer fits twice into a compute unit
         static_assert(!ROUTED || sizeof(code_lds) >= sizeof(NormRouteLds<8>), "router scratch does not fit the staging buffer");
@@ -261,13 +276,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
         if constexpr (ROUTED) {
             // the row is in LDS already
         } else if constexpr (STAGE) {
+            if (chain != CHAIN_LAST) { // (the last role reads its activations after the wait)
 #pragma unroll
-            for (int j = 0; j < (MT + 1) / 2; ++j) {
-                int m = 2 * j + (lane >> 5);
-                m = m < M ? m : 0;
-                r.xw[j] = gload<u32x4>(xl + (k0 + (uint32_t)(8 * (lane & 31)) + (uint32_t)(m * K)));
+                for (int j = 0; j < (MT + 1) / 2; ++j) {
+                    int m = 2 * j + (lane >> 5);
+                    m = m < M ? m : 0;
+                    r.xw[j] = gload<u32x4>(xl + (k0 + (uint32_t)(8 * (lane & 31)) + (uint32_t)(m * K)));
+                }
             }
-            if constexpr (NORM == 1) {
+            if (NORM == 1 && normed) {
                 r.xg = gload<u32x4>(p.norm_weight + (k0 + (uint32_t)(8 * (lane & 31))));
                 // unconditional (a launch without delta re-reads x and ignores the value): a load under a branch
                 // would make every later wait a wait for all loads
@@ -322,7 +339,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
 #pragma unroll
             for (int j = 0; j < (ROUTED ? 0 : (MT + 1) / 2); ++j) {
                 u32x4 xv = r.xw[j];
-                if constexpr (NORM == 1) { // weight * fp16(fp32(x + delta) * r): the roundings of the stand-alone norm kernel
+                if (NORM == 1 && normed) { // weight * fp16(fp32(x + delta) * r): the roundings of the stand-alone norm kernel
                     f16x8 v = __builtin_bit_cast(f16x8, xv);
                     const f16x8 vd = v + __builtin_bit_cast(f16x8, r.xd);
                     v = p.norm_delta ? vd : v;
@@ -429,7 +446,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
     // order, so these must go out before the weights for the sum to be ready while the weights still travel.
     constexpr int NPIECE = 2;
     f16x8 nv[NPIECE];
-    if constexpr (NORM == 1) {
+    if (NORM == 1 && normed) {
 #pragma unroll
         for (int c = 0; c < NPIECE; ++c) {
             const int k = ((int)threadIdx.x + c * 256) * 8;
@@ -444,12 +461,35 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
         for (int i = 0; i < D; ++i)
             issue(regs[i], slab0 + i < p.NS ? slab0 + i : last);
     }
-    if constexpr (NORM == 1) {
+    if (chain == CHAIN_LAST) {
+        // the weights are on their way; now the activations: wait for the blocks that produce them, then read the slabs'
+        // pieces at device scope (they may have been written through another XCD's L2)
+        CHAIN_STAMP(p.chain, 0);
+        chain_wait(p.chain, CHAIN_GO_MID, kChainGoMid);
+        CHAIN_STAMP(p.chain, 1);
+        if (threadIdx.x == 0)
+            chain_passed(p.chain, p.chain_blocks);
+        if constexpr (STAGE && !ROUTED) {
+            if (wave_on) {
+#pragma unroll
+                for (int i = 0; i < D; ++i) {
+                    const int slab = slab0 + i < p.NS ? slab0 + i : last;
+#pragma unroll
+                    for (int j = 0; j < (MT + 1) / 2; ++j) {
+                        int m = 2 * j + (lane >> 5);
+                        m = m < M ? m : 0;
+                        regs[i].xw[j] = chain_load16(xl + ((uint32_t)slab * kSlab + (uint32_t)(8 * (lane & 31)) + (uint32_t)(m * K)));
+                    }
+                }
+            }
+        }
+    }
+    if (NORM == 1 && normed) {
         // the sum in the order the stand-alone norm kernel adds it (256 threads, 8 elements each per pass), so that both
         // give the same bits
         float ss = 0.f;
         if (threadIdx.x < 256) {
-            const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0;
+            const bool writer = origin;
 #pragma unroll
             for (int c = 0; c < NPIECE; ++c) {
                 const int k = ((int)threadIdx.x + c * 256) * 8;
@@ -571,10 +611,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
                     val = dst[i] + val;
                 hv[i] = val;
             }
-            if constexpr (F == 4)
+            if (chain == CHAIN_FIRST) { // read by later blocks of this grid, on any XCD: stored at device scope
+                if constexpr (F == 4)
+                    chain_store(dst, (f16x4){hv[0], hv[1], hv[2], hv[3]});
+                else
+                    chain_store(dst, (f16x2){hv[0], hv[1]});
+            } else if constexpr (F == 4) {
                 *reinterpret_cast<f16x4 *>(dst) = (f16x4){hv[0], hv[1], hv[2], hv[3]};
-            else
+            } else {
                 *reinterpret_cast<f16x2 *>(dst) = (f16x2){hv[0], hv[1]};
+            }
         }
     }
 
@@ -615,6 +661,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
                     *reinterpret_cast<f16x2 *>(dst) = (f16x2){hv[0], hv[1]};
             }
         }
+        if (chain == CHAIN_FIRST) {
+            CHAIN_STAMP(p.chain, 2);
+            chain_signal(p.chain, CHAIN_FIRST_DONE, p.chain_blocks, CHAIN_GO_FIRST, kChainGoFirst);
+        }
+        if (chain != CHAIN_NONE)
+            CHAIN_STAMP(p.chain, 3);
         return;
     }
 
@@ -711,6 +763,47 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
             *reinterpret_cast<f16x4 *>(dst) = (f16x4){hv[0], hv[1], hv[2], hv[3]};
         else
             *reinterpret_cast<f16x2 *>(dst) = (f16x2){hv[0], hv[1]};
+    }
+}
+
+template <int NBITS, int MT, int S, int D, int WAVES, int SKIND, int ZKIND, int EPI, bool GROUPED = false, int NORM = 0>
+__global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
+{
+    strip_block<NBITS, MT, S, D, WAVES, SKIND, ZKIND, EPI, GROUPED, NORM>(p, (int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z, CHAIN_NONE);
+}
+
+// The attention part of a decoder layer at one token as ONE grid (chain_parts.hpp): blocks [0, nA) are the grouped
+// q/k/v projections with the residual add and the input norm in front (first role), blocks [nA, nA + heads) one
+// query head each (middle role), the rest the output projection (last role), which has its weights in registers by
+// the time the heads are done.  Every block is 16 waves; a head uses the first NT threads.
+struct ChainAttentionArgs {
+    const f16 *q, *k, *v; // written by the first role, read by the middle one
+    const f16 *cos_t, *sin_t;
+    const int64_t *pos;
+    f16 *cache_k, *cache_v;
+    int64_t max_len;
+    int group, heads;
+    f16 *out; // written by the middle role, read by the last one (as its activations)
+};
+struct ChainParams {
+    StripParams a, c;
+    ChainAttentionArgs att;
+    int nA;
+};
+
+template <int NBITS, int SKIND, int ZKIND, int HD, int NT>
+__global__ __launch_bounds__(1024) void attention_chain_kernel(ChainParams P)
+{
+    const int L = (int)blockIdx.x;
+    if (L < P.nA) {
+        strip_block<NBITS, 1, 1, 1, 16, SKIND, ZKIND, 0, true, 1>(P.a, 0, L % P.a.RB, L / P.a.RB, CHAIN_FIRST);
+    } else if (L < P.nA + P.att.heads) {
+        if ((int)threadIdx.x < NT)
+            attention_head<HD, NT>(P.att.q, P.att.k, P.att.v, P.att.cos_t, P.att.sin_t, P.att.pos, P.att.cache_k, P.att.cache_v,
+                                   P.att.max_len, P.att.group, P.att.out, L - P.nA, CHAIN_MID, P.a.chain, P.att.heads);
+    } else {
+        const int c = L - P.nA - P.att.heads;
+        strip_block<NBITS, 1, 1, 1, 16, SKIND, ZKIND, 0, true, 1>(P.c, 0, c % P.c.RB, c / P.c.RB, CHAIN_LAST);
     }
 }
 
@@ -933,9 +1026,10 @@ bool plan_job(const StripJob &j, int64_t M, StripPlan &pl, StripPlan *per_group,
     return true;
 }
 
-int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
+// the launch parameters, plan and grid of a job
+int build_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, StripParams &p, StripPlan &pl, dim3 &grid)
 {
-    StripPlan pl, per_group[kMaxGroups];
+    StripPlan per_group[kMaxGroups];
     size_t part_bytes = 0;
     // A gate of three or four rows whose blocks hold all of K runs as two passes of the two-row kernel in one launch.
     int passes = 1;
@@ -950,7 +1044,7 @@ int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t
         return HQQ_E_WORKSPACE;
     if (j.EPI == 2 && !j.row_scale)
         return HQQ_E_NULL;
-    StripParams p = {};
+    p = StripParams{};
     char *base = static_cast<char *>(ws);
     char *part = base + kHeadBytes;
     int z = 0;
@@ -1006,7 +1100,18 @@ int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t
         p.norm_delta = j.norm_delta, p.norm_weight = j.norm_weight, p.x_sum = j.x_sum, p.norm_eps = j.norm_eps;
         p.gate_w = j.gate_w, p.n_experts = j.n_experts, p.sel_out = j.sel_out, p.rw_out = j.rw_out;
     }
-    const dim3 grid((unsigned)pl.BK, (unsigned)pl.RB, (unsigned)(z * passes));
+    grid = dim3((unsigned)pl.BK, (unsigned)pl.RB, (unsigned)(z * passes));
+    return HQQ_OK;
+}
+
+int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
+{
+    StripParams p;
+    StripPlan pl;
+    dim3 grid;
+    const int rc = build_job(j, M, ws, ws_bytes, p, pl, grid);
+    if (rc != HQQ_OK)
+        return rc;
     const bool two = j.shape[0]->nbits == 2;
     if (j.NG > 1 || j.norm_weight) {
         if (j.EPI == 0 && j.NL == 1)
@@ -1123,6 +1228,90 @@ int launch_strip_group(const hqq_linear *const *layers, int count, const f16 *x,
         j.norm_delta = norm->delta, j.norm_weight = norm->weight, j.x_sum = norm->x_sum, j.norm_eps = norm->eps;
     }
     return run_job(j, 1, ws, ws_bytes, s);
+}
+
+// The attention part of a decoder layer at one token in one launch (attention_chain_kernel).  Taken for the shapes
+// the decode step has: 4-bit projections whose blocks hold all of K in 16 waves of one slab each, heads of 128.
+static int plan_attention_chain(const AttentionChain &c, void *ws, size_t ws_bytes, ChainParams &P, int &blocks, int &nt)
+{
+    if (!c.q || !c.k || !c.v || !c.o)
+        return HQQ_E_NULL;
+    // (past 4096 positions the score row no longer fits beside the projections' staging buffers)
+    if (c.head_dim != 128 || c.n_heads < 1 || c.n_kv_heads < 1 || c.n_heads % c.n_kv_heads != 0 || c.max_len < 1 ||
+        c.max_len > 4096)
+        return HQQ_E_UNSUPPORTED;
+    if (c.q->N != (int64_t)c.n_heads * c.head_dim || c.k->N != (int64_t)c.n_kv_heads * c.head_dim || c.v->N != c.k->N ||
+        c.o->K != c.q->N || c.q->nbits != 4 || !same_family(c.q, c.o))
+        return HQQ_E_UNSUPPORTED;
+    if (c.q->bias || c.k->bias || c.v->bias || c.o->bias || c.q->K % 8 != 0)
+        return HQQ_E_UNSUPPORTED;
+    StripJob ja = {};
+    ja.shape[0] = c.q, ja.shape[1] = c.k, ja.shape[2] = c.v;
+    ja.y[0] = c.q_out, ja.y[1] = c.k_out, ja.y[2] = c.v_out;
+    ja.NG = 3, ja.NL = 1, ja.EPI = 0, ja.x = c.x;
+    ja.norm_delta = c.delta, ja.norm_weight = c.norm_weight, ja.x_sum = c.x_sum, ja.norm_eps = c.eps;
+    StripJob jc = {};
+    jc.shape[0] = c.o, jc.y[0] = c.y, jc.NG = 1, jc.NL = 1, jc.EPI = 0, jc.x = c.att_out;
+    StripPlan pa, pc;
+    dim3 ga, gc;
+    int rc;
+    if ((rc = build_job(ja, 1, ws, ws_bytes, P.a, pa, ga)) != HQQ_OK || (rc = build_job(jc, 1, ws, ws_bytes, P.c, pc, gc)) != HQQ_OK)
+        return rc;
+    for (const StripPlan *pl : {&pa, &pc})
+        if (pl->MT != 1 || pl->S != 1 || pl->D != 1 || pl->WAVES != 16 || pl->BK != 1)
+            return HQQ_E_UNSUPPORTED;
+    if (pa.SKIND != pc.SKIND || pa.ZKIND != pc.ZKIND)
+        return HQQ_E_UNSUPPORTED;
+    if (!ws || ws_bytes < kHeadBytes)
+        return HQQ_E_WORKSPACE;
+    // the chain's counters: the last words of the counter region (tile counters are not used by blocks that hold all of K)
+    int *chain = reinterpret_cast<int *>(static_cast<char *>(ws) + kCounterBytes) - CHAIN_WORDS;
+    P.nA = (int)(ga.y * ga.z);
+    const int nC = (int)(gc.y * gc.z);
+    P.a.chain = P.c.chain = chain;
+    P.a.chain_blocks = P.nA, P.c.chain_blocks = nC;
+    P.att = ChainAttentionArgs{c.q_out, c.k_out, c.v_out, c.cos_t, c.sin_t, c.pos, c.cache_k, c.cache_v, c.max_len,
+                               c.n_heads / c.n_kv_heads, c.n_heads, c.att_out};
+    if (!aligned16(c.cache_k) || !aligned16(c.cache_v) || !aligned16(c.att_out) || (reinterpret_cast<uintptr_t>(c.q_out) & 3u) ||
+        (reinterpret_cast<uintptr_t>(c.k_out) & 3u) || (reinterpret_cast<uintptr_t>(c.v_out) & 3u))
+        return HQQ_E_ALIGN;
+    blocks = P.nA + c.n_heads + nC;
+    nt = c.max_len <= 512 ? 256 : 1024;
+    return HQQ_OK;
+}
+
+size_t attention_chain_error_offset() { return kCounterBytes - (CHAIN_WORDS - CHAIN_ERROR) * sizeof(int); }
+
+bool attention_chain_supported(const AttentionChain &c)
+{
+    ChainParams P;
+    int blocks, nt;
+    // planned against a stand-in workspace address: only sizes and shapes are looked at
+    alignas(256) static char head[1];
+    return plan_attention_chain(c, head, kHeadBytes, P, blocks, nt) == HQQ_OK;
+}
+
+int launch_attention_chain(const AttentionChain &c, void *ws, size_t ws_bytes, hipStream_t s)
+{
+    ChainParams P;
+    int blocks = 0, nt = 0;
+    const int rc = plan_attention_chain(c, ws, ws_bytes, P, blocks, nt);
+    if (rc != HQQ_OK)
+        return rc;
+    const size_t lds = (size_t)c.max_len * sizeof(float);
+    const bool f16_tables = table_kind(c.q->scale) == TK_F16;
+    if (nt == 256) {
+        if (f16_tables)
+            attention_chain_kernel<4, TK_F16, TK_F16, 128, 256><<<blocks, 1024, lds, s>>>(P);
+        else
+            attention_chain_kernel<4, TK_U8_COLS, TK_U8_SCALAR, 128, 256><<<blocks, 1024, lds, s>>>(P);
+    } else {
+        if (f16_tables)
+            attention_chain_kernel<4, TK_F16, TK_F16, 128, 1024><<<blocks, 1024, lds, s>>>(P);
+        else
+            attention_chain_kernel<4, TK_U8_COLS, TK_U8_SCALAR, 128, 1024><<<blocks, 1024, lds, s>>>(P);
+    }
+    return launch_status();
 }
 
 // bytes of workspace the three launches above can need for these shapes (0 when the strip kernel does not take them)

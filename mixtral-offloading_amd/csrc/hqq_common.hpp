@@ -174,6 +174,25 @@ int launch_strip_gate_up_pair_routed(const hqq_linear *w1, const hqq_linear *w3,
                                      const f16 *gate_w, int n_experts, int *sel_out, f16 *rw_out, f16 *h0, f16 *h1,
                                      void *ws, size_t ws_bytes, hipStream_t s, const StripIndex &ix);
 size_t strip_job_workspace_bytes(const hqq_linear *const *layers, int count, int NL, int64_t M);
+// The attention part of a decoder layer at one token as one launch: q/k/v projections of weight * rmsnorm(x + delta)
+// (x + delta to x_sum), rope + cache append + attention per head, output projection into y.  q_out, k_out, v_out and
+// att_out are scratch rows the parts hand over through.  Needs the workspace head (zero between launches).
+struct AttentionChain {
+    const hqq_linear *q, *k, *v, *o;
+    const f16 *x, *delta, *norm_weight;
+    float eps;
+    f16 *x_sum;
+    f16 *q_out, *k_out, *v_out, *att_out;
+    const f16 *cos_t, *sin_t;
+    const int64_t *pos;
+    f16 *cache_k, *cache_v;
+    int64_t max_len;
+    int n_heads, n_kv_heads, head_dim;
+    f16 *y;
+};
+bool attention_chain_supported(const AttentionChain &c);
+size_t attention_chain_error_offset(); // of the chain's error word inside the workspace
+int launch_attention_chain(const AttentionChain &c, void *ws, size_t ws_bytes, hipStream_t s);
 int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s);
 size_t workspace_head_bytes();
 bool tile_supported(const hqq_linear *l, int64_t M);

@@ -21,6 +21,7 @@ lib = ctypes.CDLL(LIB_PATH)
 
 HQQ_TABLE_F16, HQQ_TABLE_U8 = 0, 1
 FAM_GENERAL, FAM_SMALLBATCH, FAM_TILE, FAM_VEC3, FAM_LDS = 0, 1, 2, 3, 4
+HQQ_E_UNSUPPORTED = -6  # the library does not take the configuration (include/hqq_mi355x.h)
 
 
 class HqqTable(ctypes.Structure):
@@ -77,6 +78,11 @@ _SIGNATURES = {
                                        c_void_p, c_void_p, c_void_p, c_void_p]),
     "hqq_attention_decode": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
+    "hqq_attention_chain_workspace_bytes": (c_size_t, []),
+    "hqq_attention_chain_error_offset": (c_size_t, []),
+    "hqq_attention_chain": (c_int, [_P(HqqLinear)] * 4 + [c_void_p, c_void_p, c_void_p, ctypes.c_float] + [c_void_p] * 5
+                            + [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_int32, c_void_p,
+                               c_void_p, c_size_t, c_void_p]),
     "hqq_probe_stream_read": (c_int, [c_void_p, c_size_t, c_void_p, c_void_p]),
     "hqq_slab_h2d_async": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
     "hqq_stream_wait_event": (c_int, [c_void_p, c_void_p]),

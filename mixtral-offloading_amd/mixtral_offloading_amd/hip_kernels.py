@@ -384,6 +384,60 @@ def matmul_group_norm(group: LinearGroup, x: torch.Tensor, delta: Optional[torch
     return outs
 
 
+class AttentionChain:
+    """The attention part of a decoder layer at one token as one launch (``hqq_attention_chain``): input norm + q/k/v,
+    rope + cache append + attention, output projection.  ``supported`` turns False at the first call the library
+    refuses (shapes outside the chained kernel); the caller then makes the three calls."""
+
+    def __init__(self, qkv: LinearGroup, o_desc):
+        self.qkv, self.o = qkv, o_desc
+        self.supported = qkv.supported and len(qkv.descs) == 3
+        self._scratch = None
+
+    def __call__(self, x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                 x_sum: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, pos: torch.Tensor, cache_k: torch.Tensor,
+                 cache_v: torch.Tensor) -> Optional[torch.Tensor]:
+        """Returns the output projection's result (1, hidden), or None when the shapes are not taken."""
+        q, k, v = self.qkv.descs
+        n_kv, max_len, hd = cache_k.shape
+        n_heads = q.N // hd
+        assert x.dtype == torch.float16 and x.is_contiguous() and x.numel() == q.K and x.device == q.device
+        assert x_sum.dtype == torch.float16 and x_sum.numel() == q.K and x_sum.data_ptr() != x.data_ptr()
+        assert weight.dtype == torch.float16 and weight.numel() == q.K
+        assert cache_k.is_contiguous() and cache_v.is_contiguous() and k.N == n_kv * hd == v.N and n_heads * hd == q.N
+        assert pos.dtype == torch.int64 and pos.is_cuda and cos.shape[-1] == hd and cos.is_contiguous() and sin.is_contiguous()
+        assert cos.shape[0] >= max_len and sin.shape[0] >= max_len, "rope tables shorter than the KV cache"
+        if self._scratch is None or self._scratch.device != x.device:
+            self._scratch = torch.zeros(2 * q.N + 2 * k.N, device=x.device, dtype=torch.float16)
+        sc = self._scratch
+        qs, ks, vs, atts = sc[:q.N], sc[q.N:q.N + k.N], sc[q.N + k.N:q.N + 2 * k.N], sc[q.N + 2 * k.N:]
+        y = torch.empty((1, self.o.N), device=x.device, dtype=torch.float16)
+        with _on(x.device):
+            ws = workspace(x.device, int(_lib.lib.hqq_attention_chain_workspace_bytes()))
+            rc = _lib.lib.hqq_attention_chain(q.ref, k.ref, v.ref, self.o.ref, x.data_ptr(),
+                                              delta.data_ptr() if delta is not None else None, weight.data_ptr(), float(eps),
+                                              x_sum.data_ptr(), qs.data_ptr(), ks.data_ptr(), vs.data_ptr(), atts.data_ptr(),
+                                              cos.data_ptr(), sin.data_ptr(), pos.data_ptr(), cache_k.data_ptr(),
+                                              cache_v.data_ptr(), max_len, n_heads, n_kv, hd, y.data_ptr(), ws.data_ptr(),
+                                              ws.numel(), _lib.current_stream_ptr(x.device))
+        if rc == _lib.HQQ_E_UNSUPPORTED:
+            self.supported = False
+            return None
+        _lib.check(rc, "hqq_attention_chain")
+        return y
+
+
+def attention_chain_error(device) -> bool:
+    """Whether a chained launch on one of this device's workspaces has ever given up a wait (it never should): reads
+    a word per workspace back from the device, so call it outside the decode loop."""
+    off = int(_lib.lib.hqq_attention_chain_error_offset())
+    bad = False
+    for (index, _stream), ws in list(_workspaces.items()):
+        if index == device.index and ws.numel() >= off + 4:
+            bad = bad or bool(ws[off:off + 4].view(torch.int32).item())
+    return bad
+
+
 def router_top2(x: torch.Tensor, gate_weight: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
                 logits: Optional[torch.Tensor] = None) -> None:
     """Router of one token into device tensors ``sel`` (int32[2]) and ``weights`` (fp16[2])

@@ -147,6 +147,11 @@ class DecodeGraph:
         self.routed = all(hip_kernels.moe_pair_routed_supported(t, cfg.hidden_size, cfg.num_local_experts) for t in self.tables)
         self.qkv = [hip_kernels.LinearGroup([p._desc() for p in (l.self_attn.q_proj, l.self_attn.k_proj, l.self_attn.v_proj)])
                     for l in model.model.layers]
+        # norm + q/k/v, attention and o_proj as ONE launch (model.chain_attention = True).  Off by default here: in a
+        # replayed graph the three launches follow each other without host gaps and the chained launch measured
+        # 27 us per layer against their 25 (its two hand-overs through memory cost what two launch boundaries do, and
+        # the heads run slower while the output projection's weights stream in beside them)
+        self.chain = [hip_kernels.AttentionChain(g, l.self_attn.o_proj._desc()) for g, l in zip(self.qkv, model.model.layers)]
         self.cache = model.new_cache(max_len)
         mk = dict(device=dev)
         self.tok = torch.zeros(1, dtype=torch.int64, **mk)
@@ -175,17 +180,24 @@ class DecodeGraph:
         x, spare = self.x, self.x2  # the residual stream alternates between two buffers where the norm is fused
         x.copy_(m.model.embed_tokens(self.tok))
         delta = None
-        for layer, (ck, cv), table, qkv in zip(m.model.layers, self.cache, self.tables, self.qkv):
+        chained = getattr(m, "chain_attention", False)
+        for layer, (ck, cv), table, qkv, chain in zip(m.model.layers, self.cache, self.tables, self.qkv, self.chain):
             attn = layer.self_attn
-            if qkv.supported:
-                # residual add, input norm and the three projections in one launch
-                q, k, v = hip_kernels.matmul_group_norm(qkv, x, delta, layer.input_layernorm.weight, eps, spare)
+            attn_out = None
+            if chained and chain.supported:
+                attn_out = chain(x, delta, layer.input_layernorm.weight, eps, spare, m.rotary.cos, m.rotary.sin, self.pos, ck, cv)
+            if attn_out is not None:
                 x, spare = spare, x
             else:
-                hip_kernels.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps, self.xn)
-                q, k, v = attn.q_proj(self.xn), attn.k_proj(self.xn), attn.v_proj(self.xn)
-            out = hip_kernels.attention_decode(q, k, v, m.rotary.cos, m.rotary.sin, self.pos, ck, cv, self.att)
-            attn_out = attn.o_proj(out)
+                if qkv.supported:
+                    # residual add, input norm and the three projections in one launch
+                    q, k, v = hip_kernels.matmul_group_norm(qkv, x, delta, layer.input_layernorm.weight, eps, spare)
+                    x, spare = spare, x
+                else:
+                    hip_kernels.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps, self.xn)
+                    q, k, v = attn.q_proj(self.xn), attn.k_proj(self.xn), attn.v_proj(self.xn)
+                out = hip_kernels.attention_decode(q, k, v, m.rotary.cos, m.rotary.sin, self.pos, ck, cv, self.att)
+                attn_out = attn.o_proj(out)
             if self.routed:
                 # post-attention norm, router and both experts in two launches
                 hip_kernels.moe_pair_routed(table, x, attn_out, layer.post_attention_layernorm.weight, eps, spare,
@@ -285,6 +297,7 @@ class MixtralForCausalLM(nn.Module):
                       qkv=[hip_kernels.LinearGroup([p._desc() for p in (l.self_attn.q_proj, l.self_attn.k_proj, l.self_attn.v_proj)])
                            for l in self.model.layers])
             st["sel"], st["guess"] = st["sel4"][0:2], st["sel4"][2:4]  # one copy to the host brings both
+            st["chain"] = [None] * len(self.model.layers)
             self._token_bufs = st
         return st
 
@@ -303,6 +316,9 @@ class MixtralForCausalLM(nn.Module):
         # speculative expert loads (self.speculate, off by default): the next layer's experts are guessed one layer ahead
         speculate = bool(getattr(self, "speculate", False))
         trace = getattr(self, "attention_trace", None)  # a list: (layer, start event, end event) around each attention
+        # norm + q/k/v, attention and o_proj as one launch where it fits: on by default here, where every launch costs
+        # host time (all experts resident: 197 -> 209 tok/s)
+        chained = getattr(self, "chain_attention", True)
         st["pos"].fill_(start)
         x.copy_(self.model.embed_tokens(token.view(1)))
         delta = None
@@ -311,20 +327,37 @@ class MixtralForCausalLM(nn.Module):
             qkv = st["qkv"][i]
             if qkv.descs[0] is not attn.q_proj._desc():  # the layer's tensors were replaced since the group was made
                 qkv = st["qkv"][i] = hip_kernels.LinearGroup([p._desc() for p in (attn.q_proj, attn.k_proj, attn.v_proj)])
-            if qkv.supported:
-                q, k, v = hip_kernels.matmul_group_norm(qkv, x, delta, layer.input_layernorm.weight, eps, spare)
-                x, spare = spare, x
-            else:
-                hip_kernels.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps, xn)
-                q, k, v = attn.q_proj(xn), attn.k_proj(xn), attn.v_proj(xn)
-            if trace is not None:
+                st["chain"][i] = None
+            chain = st["chain"][i]
+            if chain is None or chain.o is not attn.o_proj._desc():
+                chain = st["chain"][i] = hip_kernels.AttentionChain(qkv, attn.o_proj._desc())
+            if trace is not None:  # the interval of the layer's attention part (one launch when chained, else the kernel)
                 trace.append((i, torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)))
-                trace[-1][1].record()
-            out = hip_kernels.attention_decode(q, k, v, self.rotary.cos, self.rotary.sin, st["pos"], ck, cv, st["att"])
-            if trace is not None:
-                trace[-1][2].record()
+            attn_out = None
+            if chained and chain.supported:
+                if trace is not None:
+                    trace[-1][1].record()
+                attn_out = chain(x, delta, layer.input_layernorm.weight, eps, spare, self.rotary.cos, self.rotary.sin,
+                                 st["pos"], ck, cv)
+            if attn_out is not None:
+                x, spare = spare, x
+                if trace is not None:
+                    trace[-1][2].record()
+            else:
+                if qkv.supported:
+                    q, k, v = hip_kernels.matmul_group_norm(qkv, x, delta, layer.input_layernorm.weight, eps, spare)
+                    x, spare = spare, x
+                else:
+                    hip_kernels.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps, xn)
+                    q, k, v = attn.q_proj(xn), attn.k_proj(xn), attn.v_proj(xn)
+                if trace is not None:
+                    trace[-1][1].record()
+                out = hip_kernels.attention_decode(q, k, v, self.rotary.cos, self.rotary.sin, st["pos"], ck, cv, st["att"])
+                if trace is not None:
+                    trace[-1][2].record()
+                attn_out = attn.o_proj(out)
             moe_block = layer.block_sparse_moe
-            hip_kernels.add_rmsnorm_router(x, attn.o_proj(out), layer.post_attention_layernorm.weight, eps, xn,
+            hip_kernels.add_rmsnorm_router(x, attn_out, layer.post_attention_layernorm.weight, eps, xn,
                                            moe_block.gate.weight, st["sel"], st["rw"])
             nxt = self.model.layers[i + 1].block_sparse_moe if speculate and i + 1 < len(self.model.layers) else None
             if nxt is not None:
