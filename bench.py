@@ -285,6 +285,16 @@ def survey_section(dev):
             fam = lib.hqq_matmul_kernel_family(layers[0].ref, m)
             add(f"matmul {tag} M={m} (family {fam})", timed(f, 48 if m <= 16 else 16), wbytes + 2 * m * (n + k), 2.0 * m * n * k,
                 ceiling=m <= 16)
+            if (nbits, n, m) in ((2, 14336, 128), (2, 14336, 512)) and fam != _lib.FAM_LDS:
+                # the other prefill kernel (weights de-quantised into LDS), forced, beside the one the library picks
+
+                def g(i):
+                    rc = lib.hqq_matmul_transpose_ex(layers[i % nl].ref, x.data_ptr(), m, y.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                     _lib.FAM_LDS, stream.cuda_stream)
+                    if rc != 0:
+                        raise _lib.HqqError(rc, "hqq_matmul_transpose_ex")
+
+                add(f"matmul {tag} M={m} (family {_lib.FAM_LDS}, forced)", timed(g, 16), wbytes + 2 * m * (n + k), 2.0 * m * n * k)
         del layers
         torch.cuda.empty_cache()
     return rows
