@@ -181,11 +181,12 @@ int launch_attention_decode(const f16 *q, const f16 *k, const f16 *v, const f16 
         return HQQ_E_ALIGN;
     const size_t lds = (size_t)max_len * sizeof(float);
     const int group = n_heads / n_kv_heads;
-    if (head_dim == 128 && max_len <= 512)
+    const int64_t small = attention_block_threads(max_len) == 256 ? max_len : 0;
+    if (head_dim == 128 && max_len <= small)
         attention_decode_kernel<128, 256><<<n_heads, 256, lds, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len, group, out);
     else if (head_dim == 128)
         attention_decode_kernel<128, 1024><<<n_heads, 1024, lds, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len, group, out);
-    else if (max_len <= 512)
+    else if (max_len <= small)
         attention_decode_kernel<64, 256><<<n_heads, 256, lds, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len, group, out);
     else
         attention_decode_kernel<64, 1024><<<n_heads, 1024, lds, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len, group, out);

@@ -1276,7 +1276,7 @@ static int plan_attention_chain(const AttentionChain &c, void *ws, size_t ws_byt
         (reinterpret_cast<uintptr_t>(c.k_out) & 3u) || (reinterpret_cast<uintptr_t>(c.v_out) & 3u))
         return HQQ_E_ALIGN;
     blocks = P.nA + c.n_heads + nC;
-    nt = c.max_len <= 512 ? 256 : 1024;
+    nt = attention_block_threads(c.max_len);
     return HQQ_OK;
 }
 
