@@ -12,6 +12,9 @@ constexpr float kXsScale = 32.0f;    // xs = 32 * s * x keeps small activations 
 // Head of every workspace, zero between launches: one arrival counter per tile, then the accumulation slots of the
 // split-K decode launches (one 64-bit word per output of the launch).
 constexpr size_t kCounterBytes = 64 * 1024;
+// the last 4 KB of the counter region hold the words of chained launches (chain_parts.hpp): tile counters stay below
+constexpr size_t kChainBytes = 4 * 1024;
+constexpr size_t kTileCounterBytes = kCounterBytes - kChainBytes;
 constexpr size_t kSlotBytes = 512 * 1024;
 constexpr size_t kHeadBytes = kCounterBytes + kSlotBytes;
 // A slot holds the sum of the K blocks' partial results as a fixed-point number (26 fractional bits, kept in bits

@@ -843,11 +843,11 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl, int64_t ti
     pl.RB = l->group_size / 16;
     pl.NS = (int)(l->K / kSlab);
     pl.MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
-    if (pl.GP > 65535 || pl.RB > 65535 || (int64_t)pl.GP * pl.RB * sizeof(int) > kCounterBytes)
+    if (pl.GP > 65535 || pl.RB > 65535 || (int64_t)pl.GP * pl.RB * sizeof(int) > kTileCounterBytes)
         return false;
     // Shape of the split: S slabs per wave, KS waves per layer, BK blocks along K.
     const int64_t tiles = tiles_all > 0 ? tiles_all : (int64_t)pl.GP * pl.RB;
-    if (tiles * sizeof(int) > kCounterBytes)
+    if (tiles * sizeof(int) > kTileCounterBytes)
         return false;
     const int max_waves = pl.MT == 1 ? 16 : 8; // wider batches need more registers and LDS staging per wave
     int S = 1, BK = 1;
@@ -1265,6 +1265,7 @@ static int plan_attention_chain(const AttentionChain &c, void *ws, size_t ws_byt
     if (!ws || ws_bytes < kHeadBytes)
         return HQQ_E_WORKSPACE;
     // the chain's counters: the last words of the counter region (tile counters are not used by blocks that hold all of K)
+    static_assert(CHAIN_WORDS * sizeof(int) <= kChainBytes, "the chain's words fit the space kept for them");
     int *chain = reinterpret_cast<int *>(static_cast<char *>(ws) + kCounterBytes) - CHAIN_WORDS;
     P.nA = (int)(ga.y * ga.z);
     const int nC = (int)(gc.y * gc.z);
@@ -1281,15 +1282,6 @@ static int plan_attention_chain(const AttentionChain &c, void *ws, size_t ws_byt
 }
 
 size_t attention_chain_error_offset() { return kCounterBytes - (CHAIN_WORDS - CHAIN_ERROR) * sizeof(int); }
-
-bool attention_chain_supported(const AttentionChain &c)
-{
-    ChainParams P;
-    int blocks, nt;
-    // planned against a stand-in workspace address: only sizes and shapes are looked at
-    alignas(256) static char head[1];
-    return plan_attention_chain(c, head, kHeadBytes, P, blocks, nt) == HQQ_OK;
-}
 
 int launch_attention_chain(const AttentionChain &c, void *ws, size_t ws_bytes, hipStream_t s)
 {

@@ -448,7 +448,7 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, W3Plan &pl)
     if (tune)
         pl.S = tuning_int("HQQ_W3_S", pl.S) == 2 ? 2 : pl.S;
     pl.KS = (pl.SB + pl.S - 1) / pl.S;
-    if ((int64_t)pl.P * NL > 65535 || pl.RB > 65535 || (int64_t)pl.P * pl.RB * NL * sizeof(int) > kCounterBytes)
+    if ((int64_t)pl.P * NL > 65535 || pl.RB > 65535 || (int64_t)pl.P * pl.RB * NL * sizeof(int) > kTileCounterBytes)
         return false;
     return true;
 }

@@ -190,7 +190,6 @@ struct AttentionChain {
     int n_heads, n_kv_heads, head_dim;
     f16 *y;
 };
-bool attention_chain_supported(const AttentionChain &c);
 size_t attention_chain_error_offset(); // of the chain's error word inside the workspace
 int launch_attention_chain(const AttentionChain &c, void *ws, size_t ws_bytes, hipStream_t s);
 int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s);
