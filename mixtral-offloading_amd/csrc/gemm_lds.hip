@@ -272,8 +272,6 @@ __global__ __launch_bounds__(kLThreads, 2) void gemm_lds_kernel(LdsParams p)
             }
 #pragma unroll
             for (int i = 0; i < F; ++i) {
-                constexpr int dummy = 0;
-                (void)dummy;
                 const int pos = NBITS * (F - 1 - i);
 #pragma unroll
                 for (int v = 0; v < NW / 2; ++v) { // eight columns = one 128-bit piece
