@@ -130,6 +130,34 @@ def test_expert_cache_loads_match_resident_results_and_lru_counts():
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("buffers", [1, 2])
+@pytest.mark.parametrize("unordered", [True, False])
+def test_one_call_for_more_experts_than_the_group_has_slots(buffers, unordered):
+    """A prompt routes tokens to every expert of a layer in one call while only two fit on the device: a slot must
+    not be loaded over before the expert in it has been handed out and used, whatever the order.  Experts big
+    enough (6 MB) that a copy takes longer than the kernels around it, over several rounds, against the same
+    experts kept resident."""
+    kw = dict(layers=1, hidden=1024, ffn=4096, seed=11, heads=8, kv_heads=2)
+    model_off, cfg = _small_setup(offload_per_layer=6, main_per_layer=2, buffers=buffers, **kw)
+    model_res, _ = _small_setup(offload_per_layer=0, main_per_layer=8, buffers=1, **kw)
+    c_off, c_res = model_off.expert_cache, model_res.expert_cache
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    x = torch.randn((3, cfg.hidden_size), device="cuda", generator=gen).half()
+    want = {e: expert(x).clone() for (_, e), expert in c_res.load_experts(*[(0, e) for e in range(8)], unordered=True)}
+    rng = np.random.default_rng(4)
+    for rnd in range(6):
+        req = rng.permutation(8).tolist()
+        seen = []
+        for (_, e), expert in c_off.load_experts(*[(0, e) for e in req], unordered=unordered):
+            seen.append(e)
+            y = expert(x)
+            assert torch.equal(y, want[e]), (rnd, e, seen)
+        assert sorted(seen) == list(range(8))
+        if not unordered:
+            assert seen == req
+    torch.cuda.synchronize()
+
+
 def test_cache_error_paths():
     model, cfg = _small_setup(layers=1, offload_per_layer=6, main_per_layer=2, buffers=1)
     c = model.expert_cache
