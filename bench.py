@@ -270,6 +270,14 @@ def survey_section(dev):
         add(f"pack   {tag}", timed(lambda i: pk[0](codes[i % 4]), 12), n * k + cbytes)
         add(f"unpack {tag}", timed(lambda i: pk[1](packed[i % 4]), 12), n * k + cbytes)
         add(f"dequantize {tag}", timed(lambda i: hip_kernels.dequantize(layers[i % nl]), 12), wbytes + 2 * n * k)
+        if gs in hip_kernels.QUANTIZE_GROUP_SIZES and n == 14336:
+            # the quantiser on fp16 weights of the shape: reads 2 bytes and writes one unpacked code per weight
+            wsrc = [torch.randn((n, k), device=dev).half() * 0.02 for _ in range(3)]
+            with torch.cuda.stream(stream):
+                add(f"quantize (min-max) {tag}", timed(lambda i: hip_kernels.quantize_groups(wsrc[i % 3], gs, nbits), 9), 3 * n * k)
+                add(f"quantize (solver, 20 iterations at most) {tag}",
+                    timed(lambda i: hip_kernels.quantize_groups(wsrc[i % 3], gs, nbits, iters=20), 6), 5 * n * k)
+            del wsrc
         del codes, packed
         for m in batches:
             x = torch.randn((m, k), device=dev).half()

@@ -708,6 +708,28 @@ int hqq_attention_decode(const void *q_f16, const void *k_f16, const void *v_f16
                                    n_kv_heads, head_dim, (f16 *)out_f16, (hipStream_t)stream);
 }
 
+size_t hqq_quantize_workspace_bytes(void) { return quantize_workspace_bytes(); }
+
+int hqq_quantize_groups(const void *w, int32_t w_is_fp32, int64_t rows, int64_t cols, int32_t nbits, int32_t round_zero,
+                        int32_t iters, float lp_norm, float beta, float kappa, void *codes_u8, void *inv_scale_f32,
+                        void *zero_f32, void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!w || !codes_u8 || !inv_scale_f32 || !zero_f32)
+        return HQQ_E_NULL;
+    return launch_quantize_groups(w, w_is_fp32, rows, cols, nbits, round_zero, iters, lp_norm, beta, kappa,
+                                  static_cast<uint8_t *>(codes_u8), static_cast<float *>(inv_scale_f32),
+                                  static_cast<float *>(zero_f32), workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int hqq_quantize_whole(const void *x_f32, int64_t n, int32_t nbits, void *codes_u8, void *inv_scale_f32, void *zero_f32,
+                       void *stream)
+{
+    if (!x_f32 || !codes_u8 || !inv_scale_f32 || !zero_f32)
+        return HQQ_E_NULL;
+    return launch_quantize_whole(static_cast<const float *>(x_f32), n, nbits, static_cast<uint8_t *>(codes_u8),
+                                 static_cast<float *>(inv_scale_f32), static_cast<float *>(zero_f32), (hipStream_t)stream);
+}
+
 size_t hqq_attention_chain_workspace_bytes(void) { return workspace_head_bytes(); }
 
 size_t hqq_attention_chain_error_offset(void) { return attention_chain_error_offset(); }

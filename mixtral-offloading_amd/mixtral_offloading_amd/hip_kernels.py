@@ -37,6 +37,9 @@ def _on(device: torch.device):
     return torch.cuda.device(device)
 
 
+kHeadReserve = 1 << 20  # the head of a workspace belongs to the kernels' counters and slots: other scratch goes past it
+
+
 def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     """Per (device, stream) scratch for split-K partial sums; grows on demand.
     Calls on one stream are ordered, so sharing it between them is safe."""
@@ -382,6 +385,45 @@ def matmul_group_norm(group: LinearGroup, x: torch.Tensor, delta: Optional[torch
                                                   float(eps), x_sum.data_ptr(), ys, ws.data_ptr(), ws.numel(),
                                                   _lib.current_stream_ptr(x.device)), "hqq_matmul_group_norm")
     return outs
+
+
+QUANTIZE_GROUP_SIZES = (8, 16, 32, 64, 128)
+
+
+def quantize_groups(w: torch.Tensor, group_size: int, nbits: int, round_zero: bool = False, iters: int = 0,
+                    lp_norm: float = 0.7, beta: float = 10.0, kappa: float = 1.01):
+    """hqq's ``Quantizer.quantize`` for ``axis=0`` grouping on the GPU (``hqq_quantize_groups``): ``w`` (fp16 or fp32,
+    contiguous, any shape) is read as ``(group_size, numel / group_size)`` whose columns are the groups.  ``iters`` > 0
+    runs hqq's solver for the zero point.  Returns ``(codes uint8 (group_size, cols), scale fp32 (1, cols), zero fp32
+    (1, cols))`` with ``scale`` already inverted, as hqq's meta holds it."""
+    assert w.is_cuda and w.is_contiguous() and w.dtype in (torch.float16, torch.float32)
+    assert group_size in QUANTIZE_GROUP_SIZES and w.numel() % group_size == 0 and w.numel() > 0
+    cols = w.numel() // group_size
+    codes = torch.empty((group_size, cols), dtype=torch.uint8, device=w.device)
+    scale = torch.empty((1, cols), dtype=torch.float32, device=w.device)
+    zero = torch.empty((1, cols), dtype=torch.float32, device=w.device)
+    with _on(w.device):
+        ws = workspace(w.device, int(_lib.lib.hqq_quantize_workspace_bytes()) + kHeadReserve)
+        # past the head of the shared workspace (counters that must stay zero between launches)
+        base = ws.data_ptr() + kHeadReserve
+        _lib.check(_lib.lib.hqq_quantize_groups(w.data_ptr(), int(w.dtype == torch.float32), group_size, cols, nbits,
+                                                int(bool(round_zero)), int(iters), float(lp_norm), float(beta), float(kappa),
+                                                codes.data_ptr(), scale.data_ptr(), zero.data_ptr(), base,
+                                                ws.numel() - kHeadReserve, _lib.current_stream_ptr(w.device)),
+                   "hqq_quantize_groups")
+    return codes, scale, zero
+
+
+def quantize_whole(x: torch.Tensor, nbits: int):
+    """``Quantizer.quantize(channel_wise=False)`` on the GPU: one scale and zero for the whole fp32 tensor.
+    Returns ``(codes uint8 of x's shape, scale fp32 scalar tensor (inverted), zero fp32 scalar tensor)``."""
+    assert x.is_cuda and x.is_contiguous() and x.dtype == torch.float32 and x.numel() > 0
+    codes = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    sz = torch.empty(2, dtype=torch.float32, device=x.device)
+    with _on(x.device):
+        _lib.check(_lib.lib.hqq_quantize_whole(x.data_ptr(), x.numel(), nbits, codes.data_ptr(), sz[0:1].data_ptr(),
+                                               sz[1:2].data_ptr(), _lib.current_stream_ptr(x.device)), "hqq_quantize_whole")
+    return codes, sz[0], sz[1]
 
 
 class AttentionChain:

@@ -82,6 +82,27 @@ class Quantizer:
         assert axis in (0, 1)
         if group_size is not None:
             assert tensor.numel() % group_size == 0
+        max_v = 2 ** nbits - 1
+        if tensor.is_cuda and tensor.numel() > 0 and tensor.dtype in (torch.float16, torch.float32):
+            # the library's quantiser for the two forms this path uses; anything else goes through the tensor ops below
+            from . import hip_kernels
+            got = None
+            if channel_wise and axis == 0 and group_size in hip_kernels.QUANTIZE_GROUP_SIZES:
+                iters = cls.OPT_PARAMS["iters"] if optimize else 0
+                got = hip_kernels.quantize_groups(tensor.contiguous(), group_size, nbits, round_zero, iters,
+                                                  cls.OPT_PARAMS["lp_norm"], cls.OPT_PARAMS["beta"], cls.OPT_PARAMS["kappa"])
+            elif not channel_wise and not round_zero:
+                got = hip_kernels.quantize_whole(tensor.float().contiguous(), nbits)
+            if got is not None:
+                W_q, inv_scale, zero = got
+                meta = {"nbits": nbits, "group_size": group_size, "shape": tensor.shape, "scale": inv_scale, "zero": zero,
+                        "axis": axis, "packing": cls.bit_to_packing[nbits]}
+                if bitpack:
+                    W_q = cls.pack[meta["packing"]](W_q)
+                else:
+                    W_q = W_q.to(tensor.dtype)
+                    meta["packing"] = None
+                return W_q, meta
         W = tensor.float()
         shape = W.shape
         if group_size is not None and channel_wise:
@@ -92,7 +113,6 @@ class Quantizer:
         else:
             _min = W.min(axis=axis, keepdim=True)[0]
             _max = W.max(axis=axis, keepdim=True)[0]
-        max_v = 2 ** nbits - 1
         scale = (max_v / (_max - _min)).clamp(max=2e4)
         zero = -_min * scale
         if round_zero:
@@ -109,10 +129,12 @@ class Quantizer:
             meta["packing"] = None
         return W_q, meta
 
-    @staticmethod
-    def optimize_weights(tensor, scale, zero, min_max, axis=0, opt_params=None, verbose=False):
+    OPT_PARAMS = {"lp_norm": 0.7, "beta": 1e1, "kappa": 1.01, "iters": 20}
+
+    @classmethod
+    def optimize_weights(cls, tensor, scale, zero, min_max, axis=0, opt_params=None, verbose=False):
         """Half-quadratic proximal refinement of the zero point (lp norm 0.7)."""
-        p = {"lp_norm": 0.7, "beta": 1e1, "kappa": 1.01, "iters": 20}
+        p = dict(cls.OPT_PARAMS)
         if opt_params:
             p.update(opt_params)
         lp, beta, kappa = p["lp_norm"], p["beta"], p["kappa"]
