@@ -258,13 +258,14 @@ int hqq_attention_chain(const hqq_linear *q, const hqq_linear *k, const hqq_line
  *      absolute error no longer falls), then q = clamp(round(w * scale + zero), 0, 2^nbits - 1).  Outputs: codes
  *      uint8 (rows, cols), unpacked; inv_scale fp32 (cols) = 1 / scale; zero fp32 (cols).  The workspace (8-byte
  *      aligned, hqq_quantize_workspace_bytes()) is only needed when iters > 0.  hqq_quantize_whole is the one-group
- *      form (channel_wise = False, the zero table's 8-bit meta): min and max over all n fp32 values.               */
+ *      form (channel_wise = False, the zero table's 8-bit meta): min and max over all n fp32 values; it always needs
+ *      the workspace.                                                                                              */
 size_t hqq_quantize_workspace_bytes(void);
 int hqq_quantize_groups(const void *w, int32_t w_is_fp32, int64_t rows, int64_t cols, int32_t nbits, int32_t round_zero,
                         int32_t iters, float lp_norm, float beta, float kappa, void *codes_u8, void *inv_scale_f32,
                         void *zero_f32, void *workspace, size_t workspace_bytes, void *stream);
 int hqq_quantize_whole(const void *x_f32, int64_t n, int32_t nbits, void *codes_u8, void *inv_scale_f32, void *zero_f32,
-                       void *stream);
+                       void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- measurement aid, no counterpart in the reference: a plain 128-bit streaming read of `bytes` bytes (16-byte aligned)
  *      that computes nothing; sink_u32 is one device word that is never written in practice.  Its duration is the

@@ -722,12 +722,13 @@ int hqq_quantize_groups(const void *w, int32_t w_is_fp32, int64_t rows, int64_t 
 }
 
 int hqq_quantize_whole(const void *x_f32, int64_t n, int32_t nbits, void *codes_u8, void *inv_scale_f32, void *zero_f32,
-                       void *stream)
+                       void *workspace, size_t workspace_bytes, void *stream)
 {
     if (!x_f32 || !codes_u8 || !inv_scale_f32 || !zero_f32)
         return HQQ_E_NULL;
     return launch_quantize_whole(static_cast<const float *>(x_f32), n, nbits, static_cast<uint8_t *>(codes_u8),
-                                 static_cast<float *>(inv_scale_f32), static_cast<float *>(zero_f32), (hipStream_t)stream);
+                                 static_cast<float *>(inv_scale_f32), static_cast<float *>(zero_f32), workspace,
+                                 workspace_bytes, (hipStream_t)stream);
 }
 
 size_t hqq_attention_chain_workspace_bytes(void) { return workspace_head_bytes(); }

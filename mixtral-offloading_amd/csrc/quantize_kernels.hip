@@ -192,13 +192,28 @@ __global__ void quantize_clear_kernel(double *err, int *stop)
         *stop = 0;
 }
 
-// one group for the whole tensor (channel_wise = False): one block finds min and max, then every element is coded
-__global__ __launch_bounds__(1024) void quantize_whole_kernel(const float *x, int64_t n, float max_v, uint8_t *codes,
-                                                              float *inv_scale, float *zero_out)
+// One group for the whole tensor (channel_wise = False).  Three launches: the extremes are cleared, every block
+// folds its share of the tensor into them (floats ordered as integers, so that integer atomics find min and max),
+// then every element is coded.
+__device__ __forceinline__ int ordered(float v) // monotonic map of fp32 onto int32
 {
-    __shared__ float mn_s[16], mx_s[16];
-    float mn = x[0], mx = x[0];
-    for (int64_t i = threadIdx.x; i < n; i += 1024) {
+    const int b = __builtin_bit_cast(int, v);
+    return b >= 0 ? b : b ^ 0x7fffffff;
+}
+__device__ __forceinline__ float unordered(int o) { return __builtin_bit_cast(float, o >= 0 ? o : o ^ 0x7fffffff); }
+
+__global__ void whole_clear_kernel(int *extremes)
+{
+    extremes[0] = 0x7fffffff; // min
+    extremes[1] = (int)0x80000000; // max
+}
+
+__global__ __launch_bounds__(256) void whole_extremes_kernel(const float *x, int64_t n, int *extremes)
+{
+    __shared__ float mn_s[4], mx_s[4];
+    const int64_t first = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    float mn = x[first < n ? first : 0], mx = mn;
+    for (int64_t i = first; i < n; i += (int64_t)gridDim.x * 256) {
         mn = __builtin_fminf(mn, x[i]);
         mx = __builtin_fmaxf(mx, x[i]);
     }
@@ -210,21 +225,29 @@ __global__ __launch_bounds__(1024) void quantize_whole_kernel(const float *x, in
     if ((threadIdx.x & 63) == 0)
         mn_s[threadIdx.x >> 6] = mn, mx_s[threadIdx.x >> 6] = mx;
     __syncthreads();
-    mn = mn_s[0], mx = mx_s[0];
-#pragma unroll
-    for (int i = 1; i < 16; ++i) {
-        mn = __builtin_fminf(mn, mn_s[i]);
-        mx = __builtin_fmaxf(mx, mx_s[i]);
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < 4; ++i) {
+            mn = __builtin_fminf(mn, mn_s[i]);
+            mx = __builtin_fmaxf(mx, mx_s[i]);
+        }
+        atomicMin(&extremes[0], ordered(mn));
+        atomicMax(&extremes[1], ordered(mx));
     }
+}
+
+__global__ __launch_bounds__(256) void whole_codes_kernel(const float *x, int64_t n, float max_v, const int *extremes,
+                                                          uint8_t *codes, float *inv_scale, float *zero_out)
+{
+    const float mn = unordered(extremes[0]), mx = unordered(extremes[1]);
     float scale = max_v / (mx - mn);
     scale = scale < 2e4f ? scale : 2e4f;
     const float zero = -mn * scale;
-    for (int64_t i = threadIdx.x; i < n; i += 1024) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
         float q = __builtin_rintf(x[i] * scale + zero);
         q = __builtin_fminf(__builtin_fmaxf(q, 0.f), max_v);
         codes[i] = (uint8_t)q;
     }
-    if (threadIdx.x == 0) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
         *inv_scale = 1.0f / scale;
         *zero_out = zero;
     }
@@ -295,11 +318,19 @@ int launch_quantize_groups(const void *w, int fp32_in, int64_t rows, int64_t col
     }
 }
 
-int launch_quantize_whole(const float *x, int64_t n, int nbits, uint8_t *codes, float *inv_scale, float *zero, hipStream_t s)
+int launch_quantize_whole(const float *x, int64_t n, int nbits, uint8_t *codes, float *inv_scale, float *zero, void *ws,
+                          size_t ws_bytes, hipStream_t s)
 {
     if (n < 1 || nbits < 1 || nbits > 8)
         return HQQ_E_SHAPE;
-    quantize_whole_kernel<<<1, 1024, 0, s>>>(x, n, (float)((1 << nbits) - 1), codes, inv_scale, zero);
+    if (!ws || ws_bytes < quantize_workspace_bytes() || (reinterpret_cast<uintptr_t>(ws) & 7u))
+        return HQQ_E_WORKSPACE;
+    int *extremes = static_cast<int *>(ws);
+    int64_t blocks = (n + 256 * 8 - 1) / (256 * 8);
+    blocks = blocks < 1 ? 1 : (blocks > 2048 ? 2048 : blocks);
+    whole_clear_kernel<<<1, 1, 0, s>>>(extremes);
+    whole_extremes_kernel<<<(unsigned)blocks, 256, 0, s>>>(x, n, extremes);
+    whole_codes_kernel<<<(unsigned)blocks, 256, 0, s>>>(x, n, (float)((1 << nbits) - 1), extremes, codes, inv_scale, zero);
     return launch_status();
 }
 

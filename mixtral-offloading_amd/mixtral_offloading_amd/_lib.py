@@ -86,7 +86,7 @@ _SIGNATURES = {
     "hqq_quantize_workspace_bytes": (c_size_t, []),
     "hqq_quantize_groups": (c_int, [c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, ctypes.c_float,
                                     ctypes.c_float, ctypes.c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
-    "hqq_quantize_whole": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "hqq_quantize_whole": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hqq_probe_stream_read": (c_int, [c_void_p, c_size_t, c_void_p, c_void_p]),
     "hqq_slab_h2d_async": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
     "hqq_stream_wait_event": (c_int, [c_void_p, c_void_p]),

@@ -421,8 +421,10 @@ def quantize_whole(x: torch.Tensor, nbits: int):
     codes = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
     sz = torch.empty(2, dtype=torch.float32, device=x.device)
     with _on(x.device):
+        ws = workspace(x.device, int(_lib.lib.hqq_quantize_workspace_bytes()) + kHeadReserve)
         _lib.check(_lib.lib.hqq_quantize_whole(x.data_ptr(), x.numel(), nbits, codes.data_ptr(), sz[0:1].data_ptr(),
-                                               sz[1:2].data_ptr(), _lib.current_stream_ptr(x.device)), "hqq_quantize_whole")
+                                               sz[1:2].data_ptr(), ws.data_ptr() + kHeadReserve, ws.numel() - kHeadReserve,
+                                               _lib.current_stream_ptr(x.device)), "hqq_quantize_whole")
     return codes, sz[0], sz[1]
 
 
