@@ -33,6 +33,20 @@ def test_min_max_quantiser_equals_the_oracle_bit_for_bit(nbits, gs, round_zero, 
     assert np.array_equal(gzero.cpu().numpy().view(np.uint32), zero.reshape(1, -1).view(np.uint32))
 
 
+@pytest.mark.parametrize("gs,cols,off", [(16, 1613, 0), (32, 2047, 1), (64, 999, 2), (128, 2272, 3), (8, 1, 0), (16, 6, 1)])
+def test_ragged_column_counts_and_unaligned_starts(gs, cols, off):
+    """Column counts that are no multiple of the groups a thread takes, and tensors that start at any element of an
+    allocation: the kernel falls back to narrower accesses and the result is the same."""
+    from mixtral_offloading_amd import hip_kernels
+    rng = np.random.default_rng(gs + cols)
+    for dtype in (np.float16, np.float32):
+        w = rng.standard_normal(gs * cols + off).astype(dtype)
+        q, scale, zero = o.hqq_quantize_tensor(w[off:].reshape(gs, cols), 4, gs, round_zero=True)
+        gq, gscale, gzero = hip_kernels.quantize_groups(torch.from_numpy(w).cuda()[off:], gs, 4, round_zero=True)
+        assert np.array_equal(gq.cpu().numpy(), q)
+        assert np.array_equal(gscale.cpu().numpy(), scale.reshape(1, -1)) and np.array_equal(gzero.cpu().numpy(), zero.reshape(1, -1))
+
+
 def test_constant_and_tiny_groups():
     """max = min gives an infinite quotient that hqq clamps to 2e4; the codes are then all equal."""
     from mixtral_offloading_amd import hip_kernels
