@@ -230,6 +230,18 @@ int hqq_attention_decode(const void *q_f16, const void *k_f16, const void *v_f16
                          const int64_t *pos, void *cache_k_f16, void *cache_v_f16, int64_t max_len, int32_t n_heads,
                          int32_t n_kv_heads, int32_t head_dim, void *out_f16, void *stream);
 
+/* ---- the same with a workspace (256-byte aligned, zero-filled once, at least hqq_attention_decode_workspace_bytes()):
+ *      for caches longer than 1024 positions the positions of a head are then split over up to 8 blocks (one per
+ *      thousand positions attended so far), each leaving its share's maximum, sum and un-normalised output in the
+ *      workspace, and the block that finishes last adds them up.  Probabilities stay fp32 in this form,
+ *      so its results agree with hqq_attention_decode's within fp16 rounding, not bit for bit.  The workspace query
+ *      returns 0 for caches the one-block kernel keeps (then both entry points are the same).                       */
+size_t hqq_attention_decode_workspace_bytes(int64_t max_len, int32_t n_heads, int32_t head_dim);
+int hqq_attention_decode_ws(const void *q_f16, const void *k_f16, const void *v_f16, const void *cos_f16, const void *sin_f16,
+                            const int64_t *pos, void *cache_k_f16, void *cache_v_f16, int64_t max_len, int32_t n_heads,
+                            int32_t n_kv_heads, int32_t head_dim, void *out_f16, void *workspace, size_t workspace_bytes,
+                            void *stream);
+
 /* ---- the attention part of a decoder layer at one token as ONE launch: hqq_matmul_group_norm (input norm + q, k, v
  *      of x + delta, x + delta to x_sum), hqq_attention_decode and hqq_matmul_transpose (o_proj) into y, with the same
  *      bits as those three calls.  The parts run as blocks of one grid in that order and hand over through the scratch
@@ -237,7 +249,8 @@ int hqq_attention_decode(const void *q_f16, const void *k_f16, const void *v_f16
  *      workspace head (hqq_workspace_init once; at least hqq_attention_chain_workspace_bytes()): the output projection
  *      has fetched its weights by the time the heads are done.  (HF transformers' Mixtral attention in the reference;
  *      the projections are src/custom_layers.py:55-92.)  HQQ_E_UNSUPPORTED for shapes outside it (then make the three
- *      calls): 4-bit projections without bias whose K fits one block (K <= 4096), head_dim 128, max_len <= 4096.
+ *      calls): 4-bit projections without bias whose K fits one block (K <= 4096), head_dim 128, max_len <= 1024 (the
+ *      caches the one-block attention kernel keeps).
  *      A wait that does not end (it cannot, by the order of the blocks) gives up after about a quarter of a second and
  *      sets the int at hqq_attention_chain_error_offset() bytes into the workspace, which is otherwise zero.          */
 size_t hqq_attention_chain_workspace_bytes(void);

@@ -766,4 +766,26 @@ int hqq_attention_chain(const hqq_linear *q, const hqq_linear *k, const hqq_line
     return launch_attention_chain(c, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
+size_t hqq_attention_decode_workspace_bytes(int64_t max_len, int32_t n_heads, int32_t head_dim)
+{
+    if (max_len < 1 || n_heads < 1 || (head_dim != 64 && head_dim != 128))
+        return 0;
+    return attention_workspace_bytes(max_len, n_heads, head_dim);
+}
+
+int hqq_attention_decode_ws(const void *q_f16, const void *k_f16, const void *v_f16, const void *cos_f16, const void *sin_f16,
+                            const int64_t *pos, void *cache_k_f16, void *cache_v_f16, int64_t max_len, int32_t n_heads,
+                            int32_t n_kv_heads, int32_t head_dim, void *out_f16, void *workspace, size_t workspace_bytes,
+                            void *stream)
+{
+    if (!q_f16 || !k_f16 || !v_f16 || !cos_f16 || !sin_f16 || !pos || !cache_k_f16 || !cache_v_f16 || !out_f16)
+        return HQQ_E_NULL;
+    const size_t need = hqq_attention_decode_workspace_bytes(max_len, n_heads, head_dim);
+    if (need > 0 && (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)))
+        return HQQ_E_WORKSPACE;
+    return launch_attention_decode((const f16 *)q_f16, (const f16 *)k_f16, (const f16 *)v_f16, (const f16 *)cos_f16,
+                                   (const f16 *)sin_f16, pos, (f16 *)cache_k_f16, (f16 *)cache_v_f16, max_len, n_heads,
+                                   n_kv_heads, head_dim, (f16 *)out_f16, (hipStream_t)stream, workspace, workspace_bytes);
+}
+
 } // extern "C"

@@ -167,11 +167,241 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(const f16 *__restr
                            CHAIN_NONE, nullptr, 0);
 }
 
+// Long caches: the positions of a head are split over several blocks, so that the walk over the cache is shared by
+// more compute units than there are heads.  Block (head, part) attends its share of positions 0 .. pos and leaves the
+// largest score m, the sum l of exp(score - m) and the un-normalised output sum(exp(score - m) * v) of that share in
+// the workspace (device-scope stores); the block of a head that counts itself last adds the shares up,
+//     out = sum_p o_p * exp(m_p - m) / sum_p l_p * exp(m_p - m),   m = max_p m_p,
+// so nobody waits for anybody.  Scores are rounded as in the one-block kernel (fp16(q . k) / sqrt(hd)); the
+// probabilities stay fp32 here (a share does not know the whole sum, so they cannot be rounded to fp16 before they
+// multiply the values as the one-block kernel does): the results agree within fp16 rounding, not bit for bit.
+constexpr int kSplitRecord(int hd) { return hd + 2; } // floats a block leaves: m, l, o[hd]
+constexpr int64_t kSplitRows = 1024;                   // positions per block from which a split pays
+
+template <int HD>
+__global__ __launch_bounds__(1024) void attention_split_kernel(const f16 *__restrict__ q_in, const f16 *__restrict__ k_in,
+                                                                const f16 *__restrict__ v_in, const f16 *__restrict__ cos_t,
+                                                                const f16 *__restrict__ sin_t, const int64_t *__restrict__ pos_p,
+                                                                f16 *__restrict__ cache_k, f16 *__restrict__ cache_v,
+                                                                int64_t max_len, int group, int parts, float *part_out,
+                                                                int *counters, f16 *__restrict__ out)
+{
+    constexpr int NT = 1024, NW = NT / 64, LP = HD / 8, ROWS = NT / LP, NPART = ROWS / 16;
+    extern __shared__ float score_lds[]; // the share's scores, then their exponentials
+    __shared__ __attribute__((aligned(16))) f16 q_lds[HD];
+    __shared__ __attribute__((aligned(16))) f16 k_lds[HD];
+    __shared__ float red_lds[2 * NW];
+    __shared__ float acc_lds[ROWS][HD];
+    __shared__ int last_lds;
+    const int h = (int)blockIdx.x / parts, sp = (int)blockIdx.x - h * parts, kv = h / group;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int d = tid < HD ? tid : 0, dr = d < HD / 2 ? d + HD / 2 : d - HD / 2;
+    const f16 qa = q_in[h * HD + d], qb = q_in[h * HD + dr];
+    const f16 ka = k_in[kv * HD + d], kb = k_in[kv * HD + dr];
+    const f16 vnew = v_in[kv * HD + d];
+    const int64_t pos = pos_p[0];
+    if (pos < 0 || pos >= max_len) // (every block of the launch leaves alike: no counter is touched)
+        return;
+    const f16 cs_d = cos_t[pos * HD + d], sn_d = sin_t[pos * HD + d];
+    // as many blocks as the positions so far give a thousand rows each (handing shares over costs about as much as
+    // walking a thousand rows): the others leave at once, and a single block writes the output itself
+    const int64_t n = pos + 1;
+    const int64_t want = (n + kSplitRows - 1) / kSplitRows;
+    const int eff = want < parts ? (int)want : parts;
+    if (sp >= eff)
+        return;
+    const int64_t chunk = (n + eff - 1) / eff;
+    const int64_t lo = (int64_t)sp * chunk, hi = lo + chunk < n ? lo + chunk : n; // empty when lo >= n
+    if (tid < HD) {
+        const f16 qr = d < HD / 2 ? -qb : qb, kr = d < HD / 2 ? -kb : kb;
+        const f16 qrot = (f16)(qa * cs_d) + (f16)(qr * sn_d);
+        const f16 krot = (f16)(ka * cs_d) + (f16)(kr * sn_d);
+        q_lds[d] = qrot;
+        k_lds[d] = krot;
+        if (sp == 0 && h % group == 0) { // (block 0 of a head always works)
+            cache_k[((int64_t)kv * max_len + pos) * HD + d] = krot;
+            cache_v[((int64_t)kv * max_len + pos) * HD + d] = vnew;
+        }
+    }
+    __syncthreads();
+    const int rsub = tid / LP, c8 = tid % LP; // LP lanes share a cache row, 16 bytes each
+    const float inv = 1.0f / __builtin_sqrtf((float)HD);
+    float mx = -3.0e38f;
+    {
+        const f16x8 qq = *reinterpret_cast<const f16x8 *>(q_lds + 8 * c8);
+        for (int64_t l0 = lo; l0 < hi; l0 += 4 * ROWS) {
+            f16x8 kk[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int64_t l = l0 + u * ROWS + rsub;
+                const int64_t lc = l < hi ? l : hi - 1;
+                if (lc == pos) // the new token's key is not in the cache yet for the other heads of its group
+                    kk[u] = *reinterpret_cast<const f16x8 *>(k_lds + 8 * c8);
+                else
+                    kk[u] = *reinterpret_cast<const f16x8 *>(cache_k + ((int64_t)kv * max_len + lc) * HD + 8 * c8);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                float acc = 0.f;
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    acc += (float)kk[u][t] * (float)qq[t];
+#pragma unroll
+                for (int off = LP / 2; off > 0; off >>= 1)
+                    acc += __shfl_xor(acc, off, 64);
+                const int64_t l = l0 + u * ROWS + rsub;
+                if (c8 == 0 && l < hi) {
+                    const float sc = (float)(f16)acc * inv;
+                    score_lds[l - lo] = sc;
+                    mx = fmaxf(mx, sc);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1)
+        mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    if (lane == 0)
+        red_lds[wave] = mx;
+    __syncthreads();
+    mx = red_lds[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w)
+        mx = fmaxf(mx, red_lds[w]);
+    float sum = 0.f;
+    for (int64_t i = tid; i < hi - lo; i += NT) {
+        const float e = __expf(score_lds[i] - mx);
+        score_lds[i] = e;
+        sum += e;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0)
+        red_lds[NW + wave] = sum;
+    __syncthreads();
+    sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w)
+        sum += red_lds[NW + w];
+
+    float o[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+        o[t] = 0.f;
+    for (int64_t l0 = lo; l0 < hi; l0 += 4 * ROWS) {
+        f16x8 vv[4];
+        float pr[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t l = l0 + u * ROWS + rsub;
+            const int64_t lc = l < hi ? l : hi - 1;
+            const f16 *vrow = lc == pos ? v_in + kv * HD : cache_v + ((int64_t)kv * max_len + lc) * HD;
+            vv[u] = *reinterpret_cast<const f16x8 *>(vrow + 8 * c8);
+            pr[u] = l < hi ? score_lds[lc - lo] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                o[t] += pr[u] * (float)vv[u][t];
+    }
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+        acc_lds[rsub][8 * c8 + t] = o[t];
+    __syncthreads();
+    static_assert(ROWS % 16 == 0 && NT >= HD * NPART, "one thread per column and group of sixteen partial outputs");
+    if (tid < HD * NPART) {
+        const int pt = tid / HD, dcol = tid % HD;
+        float a = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            a += acc_lds[16 * pt + r][dcol];
+        acc_lds[16 * pt][dcol] = a;
+    }
+    __syncthreads();
+    if (eff == 1) {
+        if (tid < HD) {
+            float a = 0.f;
+#pragma unroll
+            for (int pt = 0; pt < NPART; ++pt)
+                a += acc_lds[16 * pt][tid];
+            out[h * HD + tid] = (f16)(a / sum);
+        }
+        return;
+    }
+    // the share's record, at device scope: the block that adds the shares up may run on another XCD
+    float *const mine = part_out + ((int64_t)h * parts + sp) * kSplitRecord(HD);
+    if (tid < HD) {
+        float a = 0.f;
+#pragma unroll
+        for (int pt = 0; pt < NPART; ++pt)
+            a += acc_lds[16 * pt][tid];
+        __hip_atomic_store(mine + 2 + tid, a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (tid == 0) {
+        __hip_atomic_store(mine, mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + 1, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_s_waitcnt(0); // every store of this thread is acknowledged
+    __syncthreads();
+    if (tid == 0) {
+        const int prev = __hip_atomic_fetch_add(&counters[h], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (prev == eff - 1) // every share is there: leave the counter ready for the next launch
+            __hip_atomic_store(&counters[h], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last_lds = prev == eff - 1;
+    }
+    __syncthreads();
+    if (!last_lds || tid >= HD)
+        return;
+    const float *const rec = part_out + (int64_t)h * parts * kSplitRecord(HD);
+    // every share's record requested in one batch (at most eight), then added up in a fixed order: the result does not
+    // depend on which block came last
+    constexpr int kMaxParts = 8;
+    float ms[kMaxParts], ls[kMaxParts], os[kMaxParts];
+#pragma unroll
+    for (int p = 0; p < kMaxParts; ++p) {
+        const float *r = rec + (p < eff ? p : 0) * kSplitRecord(HD);
+        ms[p] = __hip_atomic_load(r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ls[p] = __hip_atomic_load(r + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        os[p] = __hip_atomic_load(r + 2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    float m = -3.0e38f;
+#pragma unroll
+    for (int p = 0; p < kMaxParts; ++p)
+        m = p < eff ? fmaxf(m, ms[p]) : m;
+    float tot = 0.f, acc = 0.f;
+#pragma unroll
+    for (int p = 0; p < kMaxParts; ++p) {
+        const float f = p < eff ? __expf(ms[p] - m) : 0.f;
+        tot += ls[p] * f;
+        acc += os[p] * f;
+    }
+    out[h * HD + tid] = (f16)(acc / tot);
+}
+
 } // namespace
+
+// blocks per head: one up to 1024 positions (the one-block kernel, whose roundings are the reference ops'), then one
+// per thousand positions of the cache, eight at most; how many of them a launch uses follows the position
+int attention_parts(int64_t max_len)
+{
+    const int forced = tuning_int("HQQ_ATT_PARTS", 0);
+    if (forced > 0)
+        return forced < 8 ? forced : 8;
+    const int64_t want = (max_len + kSplitRows - 1) / kSplitRows;
+    return want < 1 ? 1 : (want > 8 ? 8 : (int)want);
+}
+
+size_t attention_workspace_bytes(int64_t max_len, int n_heads, int head_dim)
+{
+    const int parts = attention_parts(max_len);
+    if (parts <= 1)
+        return 0;
+    return 256 + (((size_t)n_heads * sizeof(int) + 255) & ~(size_t)255) + (size_t)n_heads * parts * kSplitRecord(head_dim) * sizeof(float);
+}
 
 int launch_attention_decode(const f16 *q, const f16 *k, const f16 *v, const f16 *cos_t, const f16 *sin_t, const int64_t *pos,
                             f16 *cache_k, f16 *cache_v, int64_t max_len, int n_heads, int n_kv_heads, int head_dim, f16 *out,
-                            hipStream_t s)
+                            hipStream_t s, void *ws, size_t ws_bytes)
 {
     if (n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads != 0 || max_len < 1 || max_len > 16000)
         return HQQ_E_SHAPE;
@@ -179,8 +409,25 @@ int launch_attention_decode(const f16 *q, const f16 *k, const f16 *v, const f16 
         return HQQ_E_UNSUPPORTED;
     if (!aligned16(cache_k) || !aligned16(cache_v))
         return HQQ_E_ALIGN;
-    const size_t lds = (size_t)max_len * sizeof(float);
     const int group = n_heads / n_kv_heads;
+    const int parts = attention_parts(max_len);
+    // with a workspace (zero-filled once; the counters in it are left at zero) long caches are split over blocks
+    if (parts > 1 && ws && ws_bytes >= attention_workspace_bytes(max_len, n_heads, head_dim) &&
+        (reinterpret_cast<uintptr_t>(ws) & 255u) == 0 && (int64_t)n_heads * parts <= 65535) {
+        int *counters = reinterpret_cast<int *>(static_cast<char *>(ws) + 256);
+        float *part_out = reinterpret_cast<float *>(static_cast<char *>(ws) + 256 + (((size_t)n_heads * sizeof(int) + 255) & ~(size_t)255));
+        // a block's share: the cache over all blocks, or everything so far while that is a thousand rows or fewer
+        const int64_t even = (max_len + parts - 1) / parts, few = max_len < kSplitRows ? max_len : kSplitRows;
+        const size_t lds_part = (size_t)(even > few ? even : few) * sizeof(float);
+        if (head_dim == 128)
+            attention_split_kernel<128><<<n_heads * parts, 1024, lds_part, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len,
+                                                                                  group, parts, part_out, counters, out);
+        else
+            attention_split_kernel<64><<<n_heads * parts, 1024, lds_part, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len,
+                                                                                 group, parts, part_out, counters, out);
+        return launch_status();
+    }
+    const size_t lds = (size_t)max_len * sizeof(float);
     const int64_t small = attention_block_threads(max_len) == 256 ? max_len : 0;
     if (head_dim == 128 && max_len <= small)
         attention_decode_kernel<128, 256><<<n_heads, 256, lds, s>>>(q, k, v, cos_t, sin_t, pos, cache_k, cache_v, max_len, group, out);

@@ -1236,9 +1236,9 @@ static int plan_attention_chain(const AttentionChain &c, void *ws, size_t ws_byt
 {
     if (!c.q || !c.k || !c.v || !c.o)
         return HQQ_E_NULL;
-    // (past 4096 positions the score row no longer fits beside the projections' staging buffers)
+    // (caches the attention launch splits over several blocks per head are left to it: the chain has one block per head)
     if (c.head_dim != 128 || c.n_heads < 1 || c.n_kv_heads < 1 || c.n_heads % c.n_kv_heads != 0 || c.max_len < 1 ||
-        c.max_len > 4096)
+        attention_parts(c.max_len) != 1)
         return HQQ_E_UNSUPPORTED;
     if (c.q->N != (int64_t)c.n_heads * c.head_dim || c.k->N != (int64_t)c.n_kv_heads * c.head_dim || c.v->N != c.k->N ||
         c.o->K != c.q->N || c.q->nbits != 4 || !same_family(c.q, c.o))

@@ -237,7 +237,9 @@ int launch_add_rmsnorm_router(f16 *x, const f16 *delta, const f16 *weight, float
                               const f16 *gate_w, int n_experts, int *sel, f16 *weights, f16 *logits, hipStream_t s);
 int launch_attention_decode(const f16 *q, const f16 *k, const f16 *v, const f16 *cos_t, const f16 *sin_t, const int64_t *pos,
                             f16 *cache_k, f16 *cache_v, int64_t max_len, int n_heads, int n_kv_heads, int head_dim, f16 *out,
-                            hipStream_t s);
+                            hipStream_t s, void *ws = nullptr, size_t ws_bytes = 0);
+int attention_parts(int64_t max_len); // blocks per head of the attention launch
+size_t attention_workspace_bytes(int64_t max_len, int n_heads, int head_dim);
 int launch_silu_mul(const f16 *a, const f16 *b, f16 *h, int64_t count, hipStream_t s);
 int launch_scale_store(const f16 *src, f16 *dst, const f16 *row_scale, int accumulate, int64_t M, int64_t N,
                        hipStream_t s);

@@ -87,6 +87,9 @@ _SIGNATURES = {
     "hqq_quantize_groups": (c_int, [c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, ctypes.c_float,
                                     ctypes.c_float, ctypes.c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hqq_quantize_whole": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hqq_attention_decode_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32]),
+    "hqq_attention_decode_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hqq_probe_stream_read": (c_int, [c_void_p, c_size_t, c_void_p, c_void_p]),
     "hqq_slab_h2d_async": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
     "hqq_stream_wait_event": (c_int, [c_void_p, c_void_p]),

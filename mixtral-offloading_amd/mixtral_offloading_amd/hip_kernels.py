@@ -523,9 +523,14 @@ def add_rmsnorm_router(x: torch.Tensor, delta: Optional[torch.Tensor], weight: t
     return out
 
 
+_attention_workspaces = {}  # (device, stream) -> zero-filled bytes for the split attention launch
+
+
 def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
-                     pos: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """Rope, cache append and attention of one new token; ``pos`` is an int64 device tensor with the position."""
+                     pos: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, out: torch.Tensor,
+                     split: bool = True) -> torch.Tensor:
+    """Rope, cache append and attention of one new token; ``pos`` is an int64 device tensor with the position.
+    Caches longer than 512 positions are split over several blocks per head unless ``split`` is False."""
     n_kv, max_len, hd = cache_k.shape
     n_heads = q.numel() // hd
     assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous() and cache_k.is_contiguous() and cache_v.is_contiguous()
@@ -534,6 +539,19 @@ def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: tor
     # the kernel bounds the device-side position by the cache length only: the rope tables must cover the cache
     assert cos.shape[0] >= max_len and sin.shape[0] >= max_len, "rope tables shorter than the KV cache"
     with _on(q.device):
+        need = int(_lib.lib.hqq_attention_decode_workspace_bytes(max_len, n_heads, hd))
+        if need and split:
+            # long caches: a head's positions over several blocks, their shares added up through a workspace of the
+            # launch's own (its counters must stay zero between launches, so nothing else may write there)
+            key = (q.device.index, torch.cuda.current_stream(q.device).cuda_stream)
+            ws = _attention_workspaces.get(key)
+            if ws is None or ws.numel() < need:
+                ws = _attention_workspaces[key] = torch.zeros(need, dtype=torch.uint8, device=q.device)
+            _lib.check(_lib.lib.hqq_attention_decode_ws(q.data_ptr(), k.data_ptr(), v.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+                                                        pos.data_ptr(), cache_k.data_ptr(), cache_v.data_ptr(), max_len, n_heads,
+                                                        n_kv, hd, out.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                        _lib.current_stream_ptr(q.device)), "hqq_attention_decode_ws")
+            return out
         _lib.check(_lib.lib.hqq_attention_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), cos.data_ptr(), sin.data_ptr(),
                                                  pos.data_ptr(), cache_k.data_ptr(), cache_v.data_ptr(), max_len, n_heads,
                                                  n_kv, hd, out.data_ptr(), _lib.current_stream_ptr(q.device)),

@@ -370,3 +370,38 @@ def test_attention_decode_against_torch_ops(heads, kv, hd, pos, L):
     assert torch.equal(ck2, ck) and torch.equal(cv2, cv)  # the rotated key and the value landed in the cache, bit-exact
     err = (out.float() - want.float()).abs().max()
     assert float(err) <= 4e-3 * max(1.0, float(want.float().abs().max()))
+
+
+@pytest.mark.parametrize("heads,kv,hd,pos,L", [(32, 8, 128, 0, 2048), (32, 8, 128, 1, 2048), (32, 8, 128, 1023, 2048), (32, 8, 128, 1024, 2048),
+                                               (32, 8, 128, 2047, 2048), (32, 8, 128, 5, 4096), (32, 8, 128, 3000, 4096),
+                                               (32, 8, 128, 4095, 4096), (8, 8, 64, 1100, 1200), (4, 2, 64, 2900, 3000), (8, 2, 128, 15999, 16000)])
+def test_split_attention_against_the_one_block_kernel(heads, kv, hd, pos, L):
+    """Caches past 512 positions: a head's positions over two to eight blocks, shares added up by the block that
+    finishes last.  Against the one-block kernel (itself checked against the torch ops above) within fp16 rounding of
+    the output -- its probabilities stay fp32 --, the cache bit for bit, and twice in a row (the counters in the
+    workspace must be back at zero)."""
+    from mixtral_offloading_amd import hip_kernels, _lib
+    from mixtral_offloading_amd.mixtral_model import Rotary
+    assert _lib.lib.hqq_attention_decode_workspace_bytes(L, heads, hd) > 0
+    g = torch.Generator(device="cuda").manual_seed(heads + pos + L)
+    rot = Rotary(hd, L, 1e6, torch.device("cuda"))
+    ck = torch.randn((kv, L, hd), device="cuda", generator=g).half()
+    cv = torch.randn((kv, L, hd), device="cuda", generator=g).half()
+    for rep in range(2):
+        q = torch.randn((1, heads * hd), device="cuda", generator=g).half()
+        k = torch.randn((1, kv * hd), device="cuda", generator=g).half()
+        v = torch.randn((1, kv * hd), device="cuda", generator=g).half()
+        ck1, cv1, ck2, cv2 = ck.clone(), cv.clone(), ck.clone(), cv.clone()
+        p = torch.tensor([pos], device="cuda")
+        want = torch.empty((1, heads * hd), dtype=torch.float16, device="cuda")
+        got = torch.empty_like(want)
+        hip_kernels.attention_decode(q, k, v, rot.cos, rot.sin, p, ck1, cv1, want, split=False)
+        hip_kernels.attention_decode(q, k, v, rot.cos, rot.sin, p, ck2, cv2, got)
+        assert torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
+        err = (got.float() - want.float()).abs().max()
+        assert float(err) <= 4e-3 * max(1.0, float(want.float().abs().max())), float(err)
+    # a position outside the cache: nothing written, nothing counted
+    before = ck.clone()
+    hip_kernels.attention_decode(q, k, v, rot.cos, rot.sin, torch.tensor([L], device="cuda"), ck, cv, got)
+    torch.cuda.synchronize()
+    assert torch.equal(ck, before)
