@@ -346,10 +346,21 @@ __global__ __launch_bounds__(kLThreads, 2) void gemm_lds_kernel(LdsParams p)
         load_w(Wn, ls + 5);
         stage_x(Xn, (ls + 1) & 1);
         load_x(Xn, ls + 3);
-        if (ls < nsteps)
-            mma(ls & 1);
+        mma(ls & 1); // (steps come in fours, so every iteration of the loop below has a step to multiply)
         stage_t(Tn, ls & 1);
         load_t(Tn, ls + 6);
+        if constexpr (BMT >= 64) {
+            // Ask the scheduler to thread the rebuilding of the next step's weights (VALU, LDS) through this step's
+            // MFMAs: left to itself it runs the phases one after the other, and a block of four waves has nothing else
+            // to overlap them with (128 columns, 512 rows of 14336x4096: 144 us without, 97 us with).
+#pragma unroll
+            for (int i = 0; i < RBW * CBW * 2; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x002, 8, 0); // up to eight VALU
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // one LDS read
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // one LDS write
+            }
+        }
         __syncthreads();
     };
     for (int ls = 0; ls < nsteps; ls += 4) {
