@@ -18,6 +18,7 @@
 #include "table_reader.hpp"
 
 #include <cstdlib>
+#include <type_traits>
 
 namespace hqq {
 using gemv::gload;
@@ -263,6 +264,8 @@ __global__ __launch_bounds__(JW * NFW * KW * 64) void gemm_tile2_kernel(TilePara
     constexpr int NW = NWK * KW;      // waves per block
     constexpr int MB = BM / 16;
     constexpr int XP = BM + 2;
+    // the widest batch tile runs its loop as a software pipeline (compute_pipelined below)
+    constexpr bool PIPE = KW == 1 && BM >= 128;
     // With K parts every wave stages an x tile of its own and the steps of the loop need no block barrier: the
     // waves of a block share nothing until their sums meet at the end.
     constexpr bool PRIV = KW > 1;
@@ -373,7 +376,9 @@ __global__ __launch_bounds__(JW * NFW * KW * 64) void gemm_tile2_kernel(TilePara
             if (XCH * XT == BM * 8 || tk + c * XT < BM * 8)
                 *reinterpret_cast<u32x4 *>(&x_lds[buf][xi][xdst[c]]) = o;
         }
-        if (tlane) {
+        // (at the widest tile the lanes past the table rows store their twin's values a second time: no branch, so
+        // that the step stays one scheduling region)
+        if (tlane || PIPE) {
             f16x2 s01, s23, z01, z23;
             if constexpr (SKIND == TK_F16) {
                 s01 = as_f16x2(r.sf.x), s23 = as_f16x2(r.sf.y);
@@ -402,7 +407,23 @@ __global__ __launch_bounds__(JW * NFW * KW * 64) void gemm_tile2_kernel(TilePara
         for (int b = 0; b < MB; ++b)
             acc[i][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    auto compute = [&](const u32x4 cw, int buf) __attribute__((always_inline)) {
+    // The constants of this wave's fields for the pipelined loop (f0 is uniform over the wave, so the selects are
+    // scalar).  The exponent pattern is kept in a vector register: with mask and pattern both scalar operands the
+    // field merge would take two instructions (and, or) instead of one.
+    uint32_t f_mask[FW], f_expo[FW];
+    f16x2 f_off[FW];
+#pragma unroll
+    for (int i = 0; i < FW; ++i) {
+        f_mask[i] = f0 ? WField<NBITS>::mask(i + (NFW - 1) * FW) : WField<NBITS>::mask(i);
+        f_expo[i] = f0 ? WField<NBITS>::expo(i + (NFW - 1) * FW) : WField<NBITS>::expo(i);
+        const f16 offv = (f16)(f0 ? WField<NBITS>::offset(i + (NFW - 1) * FW) : WField<NBITS>::offset(i));
+        f_off[i] = (f16x2){offv, offv};
+        if constexpr (PIPE)
+            asm volatile("" : "+v"(f_expo[i]));
+    }
+
+    // the narrower tiles: groups one after the other
+    auto compute_simple = [&](const u32x4 cw, int buf) __attribute__((always_inline)) {
         const uint32_t d[4] = {cw.x, cw.y, cw.z, cw.w};
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
@@ -436,6 +457,57 @@ __global__ __launch_bounds__(JW * NFW * KW * 64) void gemm_tile2_kernel(TilePara
         }
     };
 
+    // One step: 2 * FW groups (column half h, field i) of MB MFMAs that share an A operand.  Written as a pipeline
+    // -- the weights of group g + 1 are rebuilt and the tables of group g + 2 read while the MFMAs of group g run --
+    // because a wave has at most one other wave on its SIMD to hide latencies behind.
+    auto compute_pipelined = [&](const u32x4 cw, int buf) __attribute__((always_inline)) {
+        constexpr int NG = 2 * FW;
+        const uint32_t d[4] = {cw.x, cw.y, cw.z, cw.w};
+        u32x4 S[2], Z[2];
+        f16x8 A[2];
+        f16x8 B[2][MB];
+        auto read_tables = [&](int g) __attribute__((always_inline)) {
+            const int h = g / FW, i = g % FW;
+            S[g & 1] = *reinterpret_cast<const u32x4 *>(&s_lds[buf][wave][((i * 2 + h) * 4 + kg) * 8]);
+            Z[g & 1] = *reinterpret_cast<const u32x4 *>(&z_lds[buf][wave][((i * 2 + h) * 4 + kg) * 8]);
+        };
+        auto read_x = [&](int h) __attribute__((always_inline)) {
+#pragma unroll
+            for (int b = 0; b < MB; ++b)
+                B[h][b] = *reinterpret_cast<const f16x8 *>(&x_lds[buf][xi][(((h * 4 + kg) * XP) + b * 16 + rr) * 8]);
+        };
+        auto build = [&](int g) __attribute__((always_inline)) {
+            const int h = g / FW, i = g % FW;
+            const uint32_t d0 = d[2 * h], d1 = d[2 * h + 1];
+            const uint32_t src[4] = {d0, d0 >> 8, d1, d1 >> 8};
+            u32x4 Au;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const f16x2 q = as_f16x2((f_mask[i] & src[t]) | (~f_mask[i] & f_expo[i])) - f_off[i]; // exact code
+                const f16x2 w = (q - as_f16x2(Z[g & 1][t])) * as_f16x2(S[g & 1][t]); // two fp16 roundings, as the reference
+                Au[t] = __builtin_bit_cast(uint32_t, w);
+            }
+            A[g & 1] = __builtin_bit_cast(f16x8, Au);
+        };
+        read_tables(0);
+        read_x(0);
+        if constexpr (NG > 1)
+            read_tables(1);
+        build(0);
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            if (g + 1 < NG)
+                build(g + 1);
+            if (g + 2 < NG)
+                read_tables(g + 2);
+            if (g == 0)
+                read_x(1);
+#pragma unroll
+            for (int b = 0; b < MB; ++b)
+                acc[g % FW][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[g & 1], B[g / FW][b], acc[g % FW][b], 0, 0, 0);
+        }
+    };
+
     // Step s is worked on from LDS half (s - s_begin) & 1 while step s + 1 is staged into the other half; the
     // register sets that step s + 1 leaves are refilled with the x tile of step s + 3 and the weights of step s + 5.
     Regs T0, T1, T2, T3;
@@ -460,20 +532,49 @@ __global__ __launch_bounds__(JW * NFW * KW * 64) void gemm_tile2_kernel(TilePara
         }
     };
     staged();
-    auto step = [&](Regs &Tn, XRegs &Xn, int buf, int s) __attribute__((always_inline)) {
-        if (s < s_end)
-            compute(cw, buf);
+    // guard: whether the step may lie past the end of the block's K range (then it only moves data).  Without the
+    // branch a step is one scheduling region, which the hints below shape: after every MFMA a few of the VALU
+    // instructions that rebuild the next group's weights, stage the next step and form the addresses of later ones.
+    auto step = [&](auto guard, Regs &Tn, XRegs &Xn, int buf, int s) __attribute__((always_inline)) {
+        if constexpr (PIPE) {
+            if (!decltype(guard)::value || s < s_end)
+                compute_pipelined(cw, buf);
+        } else {
+            if (s < s_end)
+                compute_simple(cw, buf);
+        }
         stage(Tn, Xn, buf ^ 1);
         cw = Tn.cw;
         issue_x(Xn, s + 3);
         issue(Tn, s + 5);
+        if constexpr (PIPE && !decltype(guard)::value) {
+#pragma unroll
+            for (int n = 0; n < 2 * FW * MB; ++n) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x002, 5, 0); // up to five VALU
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // one LDS read
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // one LDS write
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // one global load
+            }
+        }
         staged();
     };
-    for (int s = s_begin; s < (KW > 1 ? s_stop : s_end); s += 4) {
-        step(T1, X1, 0, s);
-        step(T2, X0, 1, s + 1);
-        step(T3, X1, 0, s + 2);
-        step(T0, X0, 1, s + 3);
+    constexpr std::true_type guarded{};
+    constexpr std::false_type whole{};
+    int s = s_begin;
+    if constexpr (PIPE) {
+        for (; s + 4 <= s_end; s += 4) {
+            step(whole, T1, X1, 0, s);
+            step(whole, T2, X0, 1, s + 1);
+            step(whole, T3, X1, 0, s + 2);
+            step(whole, T0, X0, 1, s + 3);
+        }
+    }
+    for (; s < (KW > 1 ? s_stop : s_end); s += 4) {
+        step(guarded, T1, X1, 0, s);
+        step(guarded, T2, X0, 1, s + 1);
+        step(guarded, T3, X1, 0, s + 2);
+        step(guarded, T0, X0, 1, s + 3);
     }
 
     if constexpr (KW > 1) {
