@@ -213,6 +213,24 @@ int hqq_router_top2(const void *x_f16, const void *gate_w_f16, int32_t n_experts
 int hqq_add_rmsnorm(void *x_f16, const void *delta_f16, const void *weight_f16, float eps, void *y_f16, int64_t hidden,
                     void *stream);
 
+/* ---- the same three for the `rows` tokens of a prompt pass (the reference runs HF transformers' Mixtral layer over
+ *      the whole prompt, src/custom_layers.py:270-282 its router): row r of x / delta / y is r * hidden elements
+ *      further, sel_out is [rows][2], weights_f16_out [rows][2], logits_f16_out [rows][n_experts] (or NULL).  Row by
+ *      row the results are those of the one-token calls.                                                           */
+int hqq_add_rmsnorm_rows(void *x_f16, const void *delta_f16, const void *weight_f16, float eps, void *y_f16, int64_t rows,
+                         int64_t hidden, void *stream);
+int hqq_router_top2_rows(const void *x_f16, const void *gate_w_f16, int32_t n_experts, int64_t rows, int64_t hidden,
+                         int32_t *sel_out, void *weights_f16_out, void *logits_f16_out, void *stream);
+
+/* ---- rotary embedding and KV-cache append of `rows` new tokens at positions start .. start + rows - 1 (HF
+ *      transformers' apply_rotary_pos_emb in the reference's Mixtral attention): q (rows, n_heads*head_dim) is rotated
+ *      in place, the rotated k (rows, n_kv_heads*head_dim) and v are written to cache_k / cache_v
+ *      [n_kv_heads][max_len][head_dim].  cos / sin are tables [positions][head_dim] at least start + rows long;
+ *      start + rows <= max_len, head_dim even and <= 256.  Arithmetic as in hqq_attention_decode.                  */
+int hqq_rope_append_rows(void *q_f16, const void *k_f16, const void *v_f16, const void *cos_f16, const void *sin_f16,
+                         int64_t start, int64_t rows, void *cache_k_f16, void *cache_v_f16, int64_t max_len,
+                         int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, void *stream);
+
 /* ---- hqq_add_rmsnorm followed by hqq_router_top2 on its output y, in one launch: the post-attention norm of a
  *      decoder layer and the router that reads it (src/custom_layers.py:276-282).  x and y as hqq_add_rmsnorm gives
  *      them; logits as hqq_router_top2 up to the order of the fp32 sums.                                           */

@@ -686,6 +686,35 @@ int hqq_add_rmsnorm(void *x_f16, const void *delta_f16, const void *weight_f16, 
                               (hipStream_t)stream);
 }
 
+int hqq_add_rmsnorm_rows(void *x_f16, const void *delta_f16, const void *weight_f16, float eps, void *y_f16, int64_t rows,
+                         int64_t hidden, void *stream)
+{
+    if (!x_f16 || !weight_f16 || !y_f16)
+        return HQQ_E_NULL;
+    return launch_add_rmsnorm((f16 *)x_f16, (const f16 *)delta_f16, (const f16 *)weight_f16, eps, (f16 *)y_f16, hidden,
+                              (hipStream_t)stream, rows);
+}
+
+int hqq_router_top2_rows(const void *x_f16, const void *gate_w_f16, int32_t n_experts, int64_t rows, int64_t hidden,
+                         int32_t *sel_out, void *weights_f16_out, void *logits_f16_out, void *stream)
+{
+    if (!x_f16 || !gate_w_f16 || !sel_out || !weights_f16_out)
+        return HQQ_E_NULL;
+    return launch_router_top2((const f16 *)x_f16, (const f16 *)gate_w_f16, n_experts, hidden, sel_out,
+                              (f16 *)weights_f16_out, (f16 *)logits_f16_out, (hipStream_t)stream, rows);
+}
+
+int hqq_rope_append_rows(void *q_f16, const void *k_f16, const void *v_f16, const void *cos_f16, const void *sin_f16,
+                         int64_t start, int64_t rows, void *cache_k_f16, void *cache_v_f16, int64_t max_len,
+                         int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, void *stream)
+{
+    if (!q_f16 || !k_f16 || !v_f16 || !cos_f16 || !sin_f16 || !cache_k_f16 || !cache_v_f16)
+        return HQQ_E_NULL;
+    return launch_rope_append_rows((f16 *)q_f16, (const f16 *)k_f16, (const f16 *)v_f16, (const f16 *)cos_f16,
+                                   (const f16 *)sin_f16, start, rows, (f16 *)cache_k_f16, (f16 *)cache_v_f16, max_len,
+                                   n_heads, n_kv_heads, head_dim, (hipStream_t)stream);
+}
+
 int hqq_add_rmsnorm_router(void *x_f16, const void *delta_f16, const void *weight_f16, float eps, void *y_f16,
                            int64_t hidden, const void *gate_w_f16, int32_t n_experts, int32_t *sel_out,
                            void *weights_f16_out, void *logits_f16_out, void *stream)

@@ -16,6 +16,11 @@ __global__ __launch_bounds__(64 * kMaxExperts) void router_top2_kernel(const f16
     __shared__ float logit_lds[kMaxExperts];
     __shared__ float prob_lds[kMaxExperts];
     const int lane = threadIdx.x & 63, e = threadIdx.x >> 6;
+    // one block per token (row)
+    x += (int64_t)blockIdx.x * hidden;
+    sel += 2 * blockIdx.x, weights += 2 * blockIdx.x;
+    if (logits_out)
+        logits_out += (int64_t)blockIdx.x * n_experts;
     if (e < n_experts) {
         const f16 *row = w + (int64_t)e * hidden;
         float acc = 0.f;
@@ -43,6 +48,10 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(f16 *__restrict__ x, c
 {
     __shared__ float part_lds[4];
     const int tid = threadIdx.x;
+    // one block per token (row)
+    x += (int64_t)blockIdx.x * hidden, y += (int64_t)blockIdx.x * hidden;
+    if (delta)
+        delta += (int64_t)blockIdx.x * hidden;
     float ss = 0.f;
     for (int k = tid * 8; k < hidden; k += 256 * 8) {
         f16x8 v = *reinterpret_cast<const f16x8 *>(x + k);
@@ -378,6 +387,41 @@ __global__ __launch_bounds__(1024) void attention_split_kernel(const f16 *__rest
     out[h * HD + tid] = (f16)(acc / tot);
 }
 
+// Rotary embedding and KV-cache append for `rows` new tokens of one sequence at positions start .. start + rows - 1
+// (the prompt pass): q (rows, n_heads * hd) is rotated in place, the rotated keys and the values go to
+// cache_k / cache_v [n_kv][max_len][hd].  Block (token, head), head < n_heads a query head, else a key/value head;
+// the arithmetic is the one-token kernel's: fp16(x * cos) + fp16(rotate_half(x) * sin), three fp16 roundings.
+__global__ __launch_bounds__(256) void rope_append_rows_kernel(f16 *__restrict__ q, const f16 *__restrict__ k,
+                                                               const f16 *__restrict__ v, const f16 *__restrict__ cos_t,
+                                                               const f16 *__restrict__ sin_t, int64_t start, int n_heads,
+                                                               int n_kv, int hd, f16 *__restrict__ cache_k,
+                                                               f16 *__restrict__ cache_v, int64_t max_len)
+{
+    const int t = blockIdx.x, hh = blockIdx.y, d = threadIdx.x;
+    const int64_t pos = start + t;
+    const bool on = d < hd;
+    const int dc = on ? d : 0;
+    const int dr = dc < hd / 2 ? dc + hd / 2 : dc - hd / 2;
+    const f16 cs = cos_t[pos * hd + dc], sn = sin_t[pos * hd + dc];
+    if (hh < n_heads) {
+        f16 *row = q + ((int64_t)t * n_heads + hh) * hd;
+        const f16 a = row[dc], b = row[dr];
+        __syncthreads(); // every element is read before any is overwritten
+        const f16 r = dc < hd / 2 ? -b : b;
+        if (on)
+            row[dc] = (f16)(a * cs) + (f16)(r * sn);
+    } else {
+        const int kvh = hh - n_heads;
+        const f16 *row = k + ((int64_t)t * n_kv + kvh) * hd;
+        const f16 a = row[dc], b = row[dr];
+        const f16 r = dc < hd / 2 ? -b : b;
+        if (on) {
+            cache_k[((int64_t)kvh * max_len + pos) * hd + dc] = (f16)(a * cs) + (f16)(r * sn);
+            cache_v[((int64_t)kvh * max_len + pos) * hd + dc] = v[((int64_t)t * n_kv + kvh) * hd + dc];
+        }
+    }
+}
+
 } // namespace
 
 // blocks per head: one up to 1024 positions (the one-block kernel, whose roundings are the reference ops'), then one
@@ -441,23 +485,26 @@ int launch_attention_decode(const f16 *q, const f16 *k, const f16 *v, const f16 
 }
 
 int launch_router_top2(const f16 *x, const f16 *w, int n_experts, int64_t hidden, int *sel, f16 *weights, f16 *logits,
-                       hipStream_t s)
+                       hipStream_t s, int64_t rows)
 {
+    if (rows < 1 || rows > 0x7fffffff)
+        return HQQ_E_SHAPE;
     if (n_experts < 2 || n_experts > kMaxExperts || hidden % 8 != 0 || hidden <= 0 || hidden > (1 << 24))
         return HQQ_E_SHAPE;
     if (!aligned16(x) || !aligned16(w))
         return HQQ_E_ALIGN;
-    router_top2_kernel<<<1, 64 * kMaxExperts, 0, s>>>(x, w, n_experts, (int)hidden, sel, weights, logits);
+    router_top2_kernel<<<(unsigned)rows, 64 * kMaxExperts, 0, s>>>(x, w, n_experts, (int)hidden, sel, weights, logits);
     return launch_status();
 }
 
-int launch_add_rmsnorm(f16 *x, const f16 *delta, const f16 *weight, float eps, f16 *y, int64_t hidden, hipStream_t s)
+int launch_add_rmsnorm(f16 *x, const f16 *delta, const f16 *weight, float eps, f16 *y, int64_t hidden, hipStream_t s,
+                       int64_t rows)
 {
-    if (hidden % 8 != 0 || hidden <= 0 || hidden > (1 << 24))
+    if (hidden % 8 != 0 || hidden <= 0 || hidden > (1 << 24) || rows < 1 || rows > 0x7fffffff)
         return HQQ_E_SHAPE;
     if (!aligned16(x) || !aligned16(weight) || !aligned16(y) || (delta && !aligned16(delta)))
         return HQQ_E_ALIGN;
-    add_rmsnorm_kernel<<<1, 256, 0, s>>>(x, delta, weight, eps, y, (int)hidden);
+    add_rmsnorm_kernel<<<(unsigned)rows, 256, 0, s>>>(x, delta, weight, eps, y, (int)hidden);
     return launch_status();
 }
 
@@ -480,6 +527,19 @@ int launch_add_rmsnorm_router(f16 *x, const f16 *delta, const f16 *weight, float
     else
         add_rmsnorm_router_kernel<<<1, 256, 0, s>>>(x, delta, weight, eps, y, (int)hidden, gate_w, n_experts, sel, weights,
                                                     logits);
+    return launch_status();
+}
+
+int launch_rope_append_rows(f16 *q, const f16 *k, const f16 *v, const f16 *cos_t, const f16 *sin_t, int64_t start,
+                            int64_t rows, f16 *cache_k, f16 *cache_v, int64_t max_len, int n_heads, int n_kv_heads,
+                            int head_dim, hipStream_t s)
+{
+    if (head_dim < 2 || head_dim > 256 || head_dim % 2 != 0 || n_heads < 1 || n_kv_heads < 1 || n_heads + n_kv_heads > 65535 ||
+        rows < 1 || rows > 0x7fffffff || start < 0 || start + rows > max_len)
+        return HQQ_E_SHAPE;
+    const dim3 grid((unsigned)rows, (unsigned)(n_heads + n_kv_heads));
+    rope_append_rows_kernel<<<grid, 256, 0, s>>>(q, k, v, cos_t, sin_t, start, n_heads, n_kv_heads, head_dim, cache_k,
+                                                 cache_v, max_len);
     return launch_status();
 }
 

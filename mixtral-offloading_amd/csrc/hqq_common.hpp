@@ -231,8 +231,12 @@ int launch_vec3_gate(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, i
 int launch_vec3_down(const hqq_linear *w2, const f16 *a, const f16 *b, int64_t M, f16 *y, void *ws, size_t ws_bytes,
                      const SmallBatchEpilogue &ep, hipStream_t s, const StripIndex *ix = nullptr);
 int launch_router_top2(const f16 *x, const f16 *w, int n_experts, int64_t hidden, int *sel, f16 *weights, f16 *logits,
-                       hipStream_t s);
-int launch_add_rmsnorm(f16 *x, const f16 *delta, const f16 *weight, float eps, f16 *y, int64_t hidden, hipStream_t s);
+                       hipStream_t s, int64_t rows = 1);
+int launch_add_rmsnorm(f16 *x, const f16 *delta, const f16 *weight, float eps, f16 *y, int64_t hidden, hipStream_t s,
+                       int64_t rows = 1);
+int launch_rope_append_rows(f16 *q, const f16 *k, const f16 *v, const f16 *cos_t, const f16 *sin_t, int64_t start,
+                            int64_t rows, f16 *cache_k, f16 *cache_v, int64_t max_len, int n_heads, int n_kv_heads,
+                            int head_dim, hipStream_t s);
 int launch_add_rmsnorm_router(f16 *x, const f16 *delta, const f16 *weight, float eps, f16 *y, int64_t hidden,
                               const f16 *gate_w, int n_experts, int *sel, f16 *weights, f16 *logits, hipStream_t s);
 int launch_attention_decode(const f16 *q, const f16 *k, const f16 *v, const f16 *cos_t, const f16 *sin_t, const int64_t *pos,

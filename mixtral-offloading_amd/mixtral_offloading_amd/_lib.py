@@ -74,6 +74,10 @@ _SIGNATURES = {
                                       _P(c_void_p), c_void_p, c_size_t, c_void_p]),
     "hqq_router_top2": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "hqq_add_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, ctypes.c_float, c_void_p, c_int64, c_void_p]),
+    "hqq_add_rmsnorm_rows": (c_int, [c_void_p, c_void_p, c_void_p, ctypes.c_float, c_void_p, c_int64, c_int64, c_void_p]),
+    "hqq_router_top2_rows": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "hqq_rope_append_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p,
+                                     c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "hqq_add_rmsnorm_router": (c_int, [c_void_p, c_void_p, c_void_p, ctypes.c_float, c_void_p, c_int64, c_void_p, c_int32,
                                        c_void_p, c_void_p, c_void_p, c_void_p]),
     "hqq_attention_decode": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,

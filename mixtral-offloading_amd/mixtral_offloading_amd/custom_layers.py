@@ -270,11 +270,16 @@ class SparseMoeWrapper(nn.Module):
     def forward(self, hidden_states: torch.Tensor):
         batch_size, sequence_length, hidden_dim = hidden_states.shape
         hidden_states = hidden_states.reshape(-1, hidden_dim)
-        router_logits = self.gate(hidden_states)  # (tokens, n_experts)
-        routing_weights = F.softmax(router_logits, dim=1, dtype=torch.float)
-        routing_weights, selected_experts = torch.topk(routing_weights, self.top_k, dim=-1)
-        routing_weights /= routing_weights.sum(dim=-1, keepdim=True)
-        routing_weights = routing_weights.to(hidden_states.dtype)
+        if (hidden_states.is_cuda and hidden_states.dtype == torch.float16 and self.top_k == 2 and self.num_experts <= 16
+                and hidden_dim % 8 == 0 and self.gate.bias is None and hidden_states.is_contiguous()):
+            # the five lines below as one launch (one block per token)
+            selected_experts, routing_weights, router_logits = hip_kernels.router_top2_rows(hidden_states, self.gate.weight)
+        else:
+            router_logits = self.gate(hidden_states)  # (tokens, n_experts)
+            routing_weights = F.softmax(router_logits, dim=1, dtype=torch.float)
+            routing_weights, selected_experts = torch.topk(routing_weights, self.top_k, dim=-1)
+            routing_weights /= routing_weights.sum(dim=-1, keepdim=True)
+            routing_weights = routing_weights.to(hidden_states.dtype)
 
         tokens = hidden_states.shape[0]
         final_hidden_states = torch.zeros((tokens, hidden_dim), dtype=hidden_states.dtype, device=hidden_states.device)

@@ -523,6 +523,56 @@ def add_rmsnorm_router(x: torch.Tensor, delta: Optional[torch.Tensor], weight: t
     return out
 
 
+def add_rmsnorm_rows(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``add_rmsnorm`` over the rows of ``x`` (tokens, hidden): ``x += delta`` in place (when given), returns
+    ``weight * rmsnorm(x)`` row by row."""
+    assert x.dtype == torch.float16 and x.dim() == 2 and x.is_contiguous() and x.shape[1] == weight.numel()
+    assert delta is None or (delta.dtype == torch.float16 and delta.shape == x.shape and delta.is_contiguous())
+    if out is None:
+        out = torch.empty_like(x)
+    assert out.dtype == torch.float16 and out.shape == x.shape and out.is_contiguous()
+    with _on(x.device):
+        _lib.check(_lib.lib.hqq_add_rmsnorm_rows(x.data_ptr(), delta.data_ptr() if delta is not None else None,
+                                                 weight.data_ptr(), float(eps), out.data_ptr(), x.shape[0], x.shape[1],
+                                                 _lib.current_stream_ptr(x.device)), "hqq_add_rmsnorm_rows")
+    return out
+
+
+def router_top2_rows(x: torch.Tensor, gate_weight: torch.Tensor):
+    """Router of every row of ``x`` (tokens, hidden) (reference src/custom_layers.py:276-282): returns ``sel``
+    int32 (tokens, 2), ``weights`` fp16 (tokens, 2), ``logits`` fp16 (tokens, n_experts)."""
+    n_experts, hidden = gate_weight.shape
+    assert x.dtype == torch.float16 and x.dim() == 2 and x.is_contiguous() and x.shape[1] == hidden
+    assert gate_weight.dtype == torch.float16 and gate_weight.is_contiguous()
+    rows = x.shape[0]
+    sel = torch.empty((rows, 2), dtype=torch.int32, device=x.device)
+    weights = torch.empty((rows, 2), dtype=torch.float16, device=x.device)
+    logits = torch.empty((rows, n_experts), dtype=torch.float16, device=x.device)
+    with _on(x.device):
+        _lib.check(_lib.lib.hqq_router_top2_rows(x.data_ptr(), gate_weight.data_ptr(), n_experts, rows, hidden,
+                                                 sel.data_ptr(), weights.data_ptr(), logits.data_ptr(),
+                                                 _lib.current_stream_ptr(x.device)), "hqq_router_top2_rows")
+    return sel, weights, logits
+
+
+def rope_append_rows(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, start: int,
+                     cache_k: torch.Tensor, cache_v: torch.Tensor) -> torch.Tensor:
+    """Rotary embedding of ``q`` (tokens, heads, hd; in place) and ``k`` (tokens, kv_heads, hd) at positions ``start``
+    onwards; the rotated keys and ``v`` are written to the caches (kv_heads, max_len, hd).  Returns ``q``."""
+    T, n_heads, hd = q.shape
+    n_kv, max_len = cache_k.shape[0], cache_k.shape[1]
+    for t in (q, k, v, cos, sin, cache_k, cache_v):
+        assert t.dtype == torch.float16 and t.is_contiguous()
+    assert k.shape == (T, n_kv, hd) and v.shape == (T, n_kv, hd) and cache_v.shape == cache_k.shape
+    assert cos.shape[1] == hd and cos.shape[0] >= start + T and sin.shape == cos.shape and start + T <= max_len
+    with _on(q.device):
+        _lib.check(_lib.lib.hqq_rope_append_rows(q.data_ptr(), k.data_ptr(), v.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+                                                 int(start), T, cache_k.data_ptr(), cache_v.data_ptr(), max_len, n_heads,
+                                                 n_kv, hd, _lib.current_stream_ptr(q.device)), "hqq_rope_append_rows")
+    return q
+
+
 _attention_workspaces = {}  # (device, stream) -> zero-filled bytes for the split attention launch
 
 

@@ -23,7 +23,14 @@ class RMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(hidden_size, dtype=torch.float16, device=device), requires_grad=False)
         self.variance_epsilon = eps
 
-    def forward(self, x):
+    def forward(self, x, delta=None):
+        """``weight * rmsnorm(x)``; with ``delta`` (device path only) ``x += delta`` in place first."""
+        if x.is_cuda and x.dtype == torch.float16 and x.dim() == 2 and x.is_contiguous():
+            from . import hip_kernels
+
+            return hip_kernels.add_rmsnorm_rows(x, delta, self.weight, self.variance_epsilon)
+        if delta is not None:
+            x.add_(delta)
         xf = x.float()
         xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
         return self.weight * xf.to(x.dtype)
@@ -41,6 +48,18 @@ class Rotary:
     def rotate_half(x):
         h = x.shape[-1] // 2
         return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
+
+    def causal_bias(self, T, start, g):
+        """fp32 (g * T, start + T): 0 where row r (token r % T at position start + r % T) may attend, -inf elsewhere.
+        The last one made is kept: the layers of a pass all ask for the same one."""
+        key = (T, start, g)
+        if getattr(self, "_bias_key", None) != key:
+            dev = self.cos.device
+            tok = torch.arange(T, device=dev).repeat(g)  # row -> token index
+            allowed = torch.arange(start + T, device=dev)[None, :] <= (start + tok)[:, None]
+            self._bias = torch.zeros(allowed.shape, dtype=torch.float32, device=dev).masked_fill_(~allowed, float("-inf"))
+            self._bias_key = key
+        return self._bias
 
     def apply(self, q, k, positions):
         cos, sin = self.cos[positions][:, None, :], self.sin[positions][:, None, :]  # (T, 1, hd)
@@ -67,18 +86,22 @@ class Attention(nn.Module):
         q = self.q_proj(x).view(T, self.num_heads, self.head_dim)
         k = self.k_proj(x).view(T, self.num_kv_heads, self.head_dim)
         v = self.v_proj(x).view(T, self.num_kv_heads, self.head_dim)
-        positions = torch.arange(start, start + T, device=x.device)
-        q, k = rotary.apply(q, k, positions)
-        cache_k[:, start:start + T] = k.transpose(0, 1)
-        cache_v[:, start:start + T] = v.transpose(0, 1)
-        keys, values = cache_k[:, :start + T], cache_v[:, :start + T]  # (kv, L, hd)
         g = self.num_heads // self.num_kv_heads
+        if x.is_cuda and q.dtype == torch.float16 and cache_k.is_contiguous() and cache_v.is_contiguous():
+            # rope of q (in place) and k, and the cache append, in one launch
+            from . import hip_kernels
+
+            hip_kernels.rope_append_rows(q, k, v, rotary.cos, rotary.sin, start, cache_k, cache_v)
+        else:
+            positions = torch.arange(start, start + T, device=x.device)
+            q, k = rotary.apply(q, k, positions)
+            cache_k[:, start:start + T] = k.transpose(0, 1)
+            cache_v[:, start:start + T] = v.transpose(0, 1)
+        keys, values = cache_k[:, :start + T], cache_v[:, :start + T]  # (kv, L, hd)
         qh = q.transpose(0, 1).reshape(self.num_kv_heads, g * T, self.head_dim)  # heads of a kv group, then tokens
-        scores = torch.bmm(qh, keys.transpose(1, 2)).float() / math.sqrt(self.head_dim)  # (kv, g*T, L)
-        if T > 1:
-            tok = torch.arange(T, device=x.device).repeat(g)  # row -> token index
-            allowed = torch.arange(start + T, device=x.device)[None, :] <= (start + tok)[:, None]
-            scores = scores.masked_fill(~allowed[None], float("-inf"))
+        scores = torch.bmm(qh, keys.transpose(1, 2)).float()  # (kv, g*T, L)
+        # scaled, and every position after a row's own token at -inf (the same table for every layer of a pass)
+        scores = torch.add(rotary.causal_bias(T, start, g), scores, alpha=1.0 / math.sqrt(self.head_dim))
         probs = torch.softmax(scores, dim=-1).to(x.dtype)
         out = torch.bmm(probs, values)  # (kv, g*T, hd)
         out = out.view(self.num_kv_heads, g, T, self.head_dim).permute(2, 0, 1, 3).reshape(T, -1)
@@ -102,7 +125,14 @@ class DecoderLayer(nn.Module):
         self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps, device)
         self.block_sparse_moe = MoePlaceholder(config, device)
 
-    def forward(self, x, rotary, cache_k, cache_v, start):
+    def forward(self, x, rotary, cache_k, cache_v, start, inplace=False):
+        """x (T, hidden).  With ``inplace`` the residual stream is updated in x itself (the caller owns it)."""
+        if x.is_cuda and x.dtype == torch.float16 and x.is_contiguous():
+            if not inplace:
+                x = x.clone()
+            attn = self.self_attn(self.input_layernorm(x), rotary, cache_k, cache_v, start)
+            moe_out, _ = self.block_sparse_moe(self.post_attention_layernorm(x, attn)[None])  # x += attn, then the norm
+            return x.add_(moe_out[0])
         x = x + self.self_attn(self.input_layernorm(x), rotary, cache_k, cache_v, start)
         moe_out, _ = self.block_sparse_moe(self.post_attention_layernorm(x)[None])
         return x + moe_out[0]
@@ -390,9 +420,9 @@ class MixtralForCausalLM(nn.Module):
     @torch.inference_mode()
     def forward_tokens(self, input_ids: torch.Tensor, cache, start: int) -> torch.Tensor:
         """Any number of tokens of one sequence, layer by layer with torch ops around the quantized linears."""
-        x = self.model.embed_tokens(input_ids)
+        x = self.model.embed_tokens(input_ids)  # a new tensor: the layers update it in place
         for layer, (ck, cv) in zip(self.model.layers, cache):
-            x = layer(x, self.rotary, ck, cv, start)
+            x = layer(x, self.rotary, ck, cv, start, inplace=True)
         return self.lm_head(self.model.norm(x))
 
     @torch.inference_mode()

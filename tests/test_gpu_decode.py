@@ -405,3 +405,74 @@ def test_split_attention_against_the_one_block_kernel(heads, kv, hd, pos, L):
     hip_kernels.attention_decode(q, k, v, rot.cos, rot.sin, torch.tensor([L], device="cuda"), ck, cv, got)
     torch.cuda.synchronize()
     assert torch.equal(ck, before)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,hidden", [(1, 256), (7, 1024), (128, 4096), (33, 5120)])
+@pytest.mark.parametrize("with_delta", [False, True])
+def test_add_rmsnorm_rows_equals_the_one_row_call(rows, hidden, with_delta):
+    from mixtral_offloading_amd import hip_kernels
+    g = torch.Generator(device="cuda").manual_seed(rows * hidden)
+    x = torch.randn((rows, hidden), device="cuda", generator=g).half()
+    d = torch.randn((rows, hidden), device="cuda", generator=g).half() if with_delta else None
+    w = (1 + 0.1 * torch.randn(hidden, device="cuda", generator=g)).half()
+    xs = x.clone()
+    ys = hip_kernels.add_rmsnorm_rows(xs, d, w, 1e-5)
+    for r in sorted({0, rows // 2, rows - 1}):
+        x1, y1 = x[r:r + 1].clone(), torch.empty((1, hidden), dtype=torch.float16, device="cuda")
+        hip_kernels.add_rmsnorm(x1, d[r:r + 1].clone() if with_delta else None, w, 1e-5, y1)
+        assert torch.equal(xs[r:r + 1], x1) and torch.equal(ys[r:r + 1], y1)
+    x_want = x + d if with_delta else x
+    xf = x_want.float()
+    want = w * (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)).half()
+    assert torch.equal(xs, x_want)
+    assert float((ys.float() - want.float()).abs().max()) <= 2e-3 * float(want.float().abs().max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,n_experts,hidden", [(1, 8, 256), (128, 8, 4096), (19, 4, 1024), (64, 16, 512)])
+def test_router_top2_rows_equals_the_one_row_call_and_the_reference_lines(rows, n_experts, hidden):
+    from mixtral_offloading_amd import hip_kernels
+    g = torch.Generator(device="cuda").manual_seed(rows + hidden)
+    x = torch.randn((rows, hidden), device="cuda", generator=g).half()
+    gw = (0.05 * torch.randn((n_experts, hidden), device="cuda", generator=g)).half()
+    sel, rw, lg = hip_kernels.router_top2_rows(x, gw)
+    for r in sorted({0, rows // 2, rows - 1}):
+        s1, w1 = torch.zeros(2, dtype=torch.int32, device="cuda"), torch.zeros(2, dtype=torch.float16, device="cuda")
+        l1 = torch.zeros(n_experts, dtype=torch.float16, device="cuda")
+        hip_kernels.router_top2(x[r:r + 1].clone(), gw, s1, w1, l1)
+        assert torch.equal(sel[r], s1) and torch.equal(rw[r], w1) and torch.equal(lg[r], l1)
+    # the reference's five lines (src/custom_layers.py:276-282) in torch
+    logits = torch.nn.functional.linear(x, gw)
+    p = torch.softmax(logits, dim=1, dtype=torch.float)
+    pw, ps = torch.topk(p, 2, dim=-1)
+    pw = (pw / pw.sum(dim=-1, keepdim=True)).half()
+    assert float((lg.float() - logits.float()).abs().max()) <= 4e-3 * max(1.0, float(logits.float().abs().max()))
+    top = logits.float().sort(dim=1, descending=True).values
+    clear = ((top[:, 0] - top[:, 1]) > 0.02) & ((top[:, 1] - top[:, 2]) > 0.02)  # rows without a near-tie
+    assert int(clear.sum()) >= rows // 2
+    assert torch.equal(sel[clear].long(), ps[clear])
+    assert float((rw[clear].float() - pw[clear].float()).abs().max()) <= 2e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,heads,kv,hd,start,L", [(128, 32, 8, 128, 0, 130), (5, 32, 8, 128, 37, 64), (1, 4, 4, 64, 9, 10),
+                                                   (17, 8, 2, 64, 0, 17)])
+def test_rope_append_rows_equals_the_torch_ops(T, heads, kv, hd, start, L):
+    from mixtral_offloading_amd import hip_kernels
+    from mixtral_offloading_amd.mixtral_model import Rotary
+    g = torch.Generator(device="cuda").manual_seed(T * hd + start)
+    rot = Rotary(hd, L + 3, 1e6, torch.device("cuda"))
+    q = torch.randn((T, heads, hd), device="cuda", generator=g).half()
+    k = torch.randn((T, kv, hd), device="cuda", generator=g).half()
+    v = torch.randn((T, kv, hd), device="cuda", generator=g).half()
+    ck = torch.randn((kv, L, hd), device="cuda", generator=g).half()
+    cv = torch.randn((kv, L, hd), device="cuda", generator=g).half()
+    ck_want, cv_want = ck.clone(), cv.clone()
+    q_want, k_want = rot.apply(q, k, torch.arange(start, start + T, device="cuda"))
+    ck_want[:, start:start + T] = k_want.transpose(0, 1)
+    cv_want[:, start:start + T] = v.transpose(0, 1)
+    out = hip_kernels.rope_append_rows(q, k, v, rot.cos, rot.sin, start, ck, cv)
+    assert out is q and torch.equal(q, q_want) and torch.equal(ck, ck_want) and torch.equal(cv, cv_want)
+    with pytest.raises(Exception):  # past the end of the cache
+        hip_kernels.rope_append_rows(q, k, v, rot.cos, rot.sin, L - T + 1, ck, cv)
