@@ -308,6 +308,28 @@ def survey_section(dev):
     return rows
 
 
+def prefill_section(dev, tokens=128, repeats=3):
+    """The prompt pass alone (all experts resident): milliseconds for `tokens` tokens through the 32 layers."""
+    import torch
+
+    from mixtral_offloading_amd import build_model as bm
+
+    cfg = bm.mixtral_config()
+    off = bm.OffloadConfig(main_size=32 * 8, offload_size=0, buffer_size=4, offload_per_layer=0)
+    model = bm.build_model(dev, bm.default_quant_config(), off, model_config=cfg, seed=0, max_positions=1024)
+    gen = torch.Generator(device=dev).manual_seed(1)
+    prompt = torch.randint(0, cfg.vocab_size, (tokens,), device=dev, generator=gen)
+    cache = model.new_cache(tokens + 2)
+    model.forward(prompt, cache, 0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(repeats):
+        model.forward(prompt, cache, 0)
+    torch.cuda.synchronize()
+    return {"prefill_tokens": tokens, "prefill_ms": round((time.perf_counter() - t0) / repeats * 1e3, 2),
+            "model": "Mixtral-8x7B architecture, 32 layers, random-init, attention 4-bit g64, experts 2-bit g16"}
+
+
 def decode_section(dev, tokens_resident=256, tokens_offload=256):
     """Tokens per second of the whole model; every figure is measured between synchronisations
     around the decode loop, prompt processing excluded."""
@@ -432,6 +454,8 @@ def main():
     ap.add_argument("--experts", type=int, default=8, help="distinct experts the steps rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the whole-model decode section")
+    ap.add_argument("--prefill-only", type=int, default=0, metavar="TOKENS",
+                    help="time only the prompt pass of the whole model over TOKENS tokens and print that (for profiling)")
     ap.add_argument("--survey", action="store_true",
                     help="also time every kernel of the path (packers, de-quantiser, 2/3/4-bit matmuls at the Mixtral-8x7B "
                          "shapes and batches) and add the table as 'kernels'")
@@ -450,6 +474,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.prefill_only:
+        print(json.dumps(prefill_section(dev, args.prefill_only)))
+        return
     m = args.batch
     experts = [make_expert(i, dev) for i in range(args.experts)]
     descs = [(e[0]._desc(), e[1]._desc(), e[2]._desc()) for e in experts]
