@@ -310,3 +310,62 @@ def test_speculative_prefetch_overlaps_attention_and_keeps_the_tokens():
     for (layer, e), c0, c1 in copies:
         overlapping += any(l == layer and a0 < c1 and c0 < a1 for l, a0, a1 in att)
     assert overlapping >= 0.5 * len(copies), (overlapping, len(copies))
+
+
+def test_prompt_in_two_passes_equals_one_pass_and_the_torch_op_layer():
+    """The prompt pass through the row kernels (residual add + norm, router, rope + cache append of all tokens): a prompt
+    fed as 10 + 6 tokens gives the logits and caches of the 16 tokens at once, and a layer gives what the same layer
+    gives with torch ops for norm, rope, cache append and router (the path CPU tensors take, here forced)."""
+    from mixtral_offloading_amd import hip_kernels
+    model, cfg = _small_setup(layers=2, offload_per_layer=0, main_per_layer=8, seed=6)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    prompt = torch.randint(0, cfg.vocab_size, (16,), device="cuda", generator=g)
+    cache_a, cache_b = model.new_cache(20), model.new_cache(20)
+    whole = model.forward(prompt, cache_a, 0).float()
+    first = model.forward(prompt[:10], cache_b, 0).float()
+    second = model.forward(prompt[10:], cache_b, 10).float()
+    both = torch.cat((first, second))
+    assert float((both - whole).abs().max()) <= 2e-2 * float(whole.abs().max()) + 1e-3
+    for (ka, va), (kb, vb) in zip(cache_a, cache_b):
+        assert float((ka.float() - kb.float()).abs().max()) <= 2e-2 and float((va.float() - vb.float()).abs().max()) <= 2e-2
+
+    with torch.inference_mode():
+        # one layer against itself with the torch ops: rows kernels switched off by handing the layer fp16 tensors through
+        # the reference formulas
+        layer = model.model.layers[0]
+        x = torch.randn((12, cfg.hidden_size), device="cuda", generator=g).half()
+        ck, cv = (t.clone() for t in model.new_cache(16)[0])
+        got = layer(x, model.rotary, ck, cv, 2)
+        ck2, cv2 = (t.clone() for t in model.new_cache(16)[0])
+
+        def norm(mod, t):
+            tf = t.float()
+            return mod.weight * (tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + mod.variance_epsilon)).half()
+
+        att, hd = layer.self_attn, cfg.hidden_size // cfg.num_attention_heads
+        h = norm(layer.input_layernorm, x)
+        q = att.q_proj(h).view(12, att.num_heads, hd)
+        k = att.k_proj(h).view(12, att.num_kv_heads, hd)
+        v = att.v_proj(h).view(12, att.num_kv_heads, hd)
+        q, k = model.rotary.apply(q, k, torch.arange(2, 14, device="cuda"))
+        ck2[:, 2:14], cv2[:, 2:14] = k.transpose(0, 1), v.transpose(0, 1)
+        assert torch.equal(ck[:, 2:14], ck2[:, 2:14]) and torch.equal(cv[:, 2:14], cv2[:, 2:14])
+        grp = att.num_heads // att.num_kv_heads
+        qh = q.transpose(0, 1).reshape(att.num_kv_heads, grp * 12, hd)
+        scores = torch.bmm(qh, ck2[:, :14].transpose(1, 2)).float() / hd ** 0.5
+        tok = torch.arange(12, device="cuda").repeat(grp)
+        allowed = torch.arange(14, device="cuda")[None, :] <= (2 + tok)[:, None]
+        probs = torch.softmax(scores.masked_fill(~allowed[None], float("-inf")), dim=-1).half()
+        o_ = torch.bmm(probs, cv2[:, :14]).view(att.num_kv_heads, grp, 12, hd).permute(2, 0, 1, 3).reshape(12, -1)
+        x1 = x + att.o_proj(o_)
+        h2 = norm(layer.post_attention_layernorm, x1)
+        moe = layer.block_sparse_moe
+        logits = moe.gate(h2)
+        pw, ps = torch.topk(torch.softmax(logits, dim=1, dtype=torch.float), 2, dim=-1)
+        pw = (pw / pw.sum(dim=-1, keepdim=True)).half()
+        want = x1.clone()
+        for t in range(12):
+            for slot in range(2):
+                (_, _), expert = next(iter(moe.experts.load_experts((0, int(ps[t, slot])))))
+                want[t] += (pw[t, slot] * expert(h2[t:t + 1]))[0]
+        assert float((got.float() - want.float()).abs().max()) <= 2e-2 * float(want.float().abs().max()) + 1e-3
