@@ -21,9 +21,20 @@
 // A gate of three or four rows whose blocks hold all of K is launched as two passes of the two-row kernel (batch
 // rows 0-1 and 2-3) in one grid, the two passes of a tile next to each other in launch order.
 //
-// Lane roles inside a slab.  Code lanes: (rr = lane & 15, kg = lane >> 4) own packed row jp + (16*rb + rr)*GP,
-// bytes 64*s + 16*kg .. +15 for step s.  Table lanes: (ti = lane >> 4 < F, kq = lane & 15) own table row F*jp + ti,
-// columns 16*kq .. 16*kq+15, i.e. step kq >> 2, MFMA lane group kq & 3.
+// Lane roles inside a slab, batches of two and four rows.  Code lanes: (rr = lane & 15, kg = lane >> 4) own packed
+// row jp + (16*rb + rr)*GP, bytes 64*s + 16*kg .. +15 for step s.  Table lanes: (ti = lane >> 4 < F, kq = lane & 15)
+// own table row F*jp + ti, columns 16*kq .. 16*kq+15, i.e. step kq >> 2, MFMA lane group kq & 3.
+//
+// Single rows (the decode step) use another layout, in which neither the codes nor the folded activations pass
+// through LDS.  A lane (phi = lane & 3, rho = (lane >> 2) & 3, g = lane >> 4) owns the 16 columns 64*g + 16*phi .. +15
+// of the slab: as a code lane of the tile rows 4*R + rho (R = 0..3, one 128-bit load each: four consecutive lanes read
+// 64 consecutive bytes, a wave load covers 256 contiguous bytes of four rows), as a table lane of table row
+// F*jp + rho.  The MFMA's sixteen A rows are (rho, phi): four tile rows, each at four column phases; its sixteen B
+// columns are (field, phi), the lane's own 16 folded activations.  Output (row (rho, phi), column (i, phi)) of the
+// MFMA whose A operand is field i masked in place is the partial sum of tile row rho, field i, over the columns of
+// phase phi; the other columns pair a field with another field's scales and are never read.  So one B operand
+// serves all four fields and all four row groups, a lane builds it from the table entries it loaded itself, and the
+// four phases of a row are added once per wave, at the end.
 #include "attention_parts.hpp"
 #include "chain_parts.hpp"
 #include "gemv_parts.hpp"
@@ -126,11 +137,13 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
     constexpr int XS_HALVES = 4 * STEP_HALVES;
     // Codes are staged through LDS for batches of one and two rows; at four rows the activation staging already
     // takes most of the LDS a wave can have, and there the codes are loaded straight into the MFMA layout.
-    constexpr bool STAGE = MT <= 2;
+    constexpr bool PHASE = MT == 1; // single rows: the (row, phase) x (field, phase) layout, nothing but x through LDS
+    constexpr bool STAGE = MT == 2; // codes staged through LDS
+    constexpr bool XSTAGE = MT <= 2; // x reaches the table lanes through LDS
     constexpr int CODE_PITCH = kSlab + 16; // bytes per tile row in the staging buffer: the pad spreads the rows over the banks
-    __shared__ __attribute__((aligned(16))) f16 xs_lds[WAVES][XS_HALVES];
+    __shared__ __attribute__((aligned(16))) f16 xs_lds[PHASE ? 1 : WAVES][PHASE ? 8 : XS_HALVES];
     __shared__ __attribute__((aligned(16))) uint8_t code_lds[STAGE ? WAVES : 1][STAGE ? 16 * CODE_PITCH : 16];
-    __shared__ __attribute__((aligned(16))) f16 xw_lds[STAGE ? WAVES : 1][STAGE ? 2 * ((MT + 1) / 2) : 1][STAGE ? kSlab : 8];
+    __shared__ __attribute__((aligned(16))) f16 xw_lds[XSTAGE ? WAVES : 1][XSTAGE ? 2 * ((MT + 1) / 2) : 1][XSTAGE ? kSlab : 8];
     __shared__ float bias_lds[WAVES][F][MT];
     __shared__ __attribute__((aligned(16))) float red_lds[WAVES][16][MT][F];
     __shared__ __attribute__((aligned(16))) float fin_lds[2][16][MT][F];
@@ -174,10 +187,8 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
     if constexpr (ROUTED) {
         // every block routes for itself (the router's rows come from L2): which records to read is known only then
         const bool writer = origin;
-        // the router's scratch shares the code staging buffer, which nothing touches before the first slab is worked
-        // on: with an LDS array of its own the block no longer fits twice into a compute unit
-        static_assert(!ROUTED || sizeof(code_lds) >= sizeof(NormRouteLds<8>), "router scratch does not fit the staging buffer");
-        NormRouteLds<8> &route_lds = *reinterpret_cast<NormRouteLds<8> *>(&code_lds[0][0]);
+        __shared__ __attribute__((aligned(16))) uint8_t route_raw[ROUTED ? sizeof(NormRouteLds<8>) : 16];
+        NormRouteLds<8> &route_lds = *reinterpret_cast<NormRouteLds<8> *>(&route_raw[0]);
         uint32_t recw[REC_PER];
 #pragma unroll
         for (int q = 0; q < REC_PER; ++q) {
@@ -240,7 +251,9 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
     const int M = MT == 1 ? 1 : (p.M - 2 * pass < MT ? p.M - 2 * pass : MT);
 
     const int rr = lane & 15, kg = lane >> 4;
-    const int ti = lane >> 4, kq = lane & 15;
+    // table lane: table row ti of the tile, columns 16*kq .. 16*kq+15 of the slab
+    const int ti = PHASE ? (lane >> 2) & 3 : lane >> 4;
+    const int kq = PHASE ? 4 * (lane >> 4) + (lane & 3) : lane & 15;
     const bool tlane = ti < F;     // lanes that own table entries (all of them for 2-bit codes)
     const int ti_l = ti & (F - 1); // the other lanes repeat a table lane's loads, so that issuing loads never diverges
 
@@ -250,10 +263,12 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
     // through an LDS staging buffer.  Loading straight into that layout puts four different rows into every group of
     // four lanes and costs four times the address cycles; with twelve loads per slab that pipeline, not HBM, then
     // bounds the kernel.
-    const int lrow = lane >> 4, lchunk = lane & 15;
-    const uint32_t crow = STAGE ? ((uint32_t)jp + (uint32_t)(16 * rb + lrow) * (uint32_t)GP) * (uint32_t)K + (uint32_t)(16 * lchunk)
-                                : ((uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)GP) * (uint32_t)K + (uint32_t)(16 * kg);
-    const uint32_t crow_step = STAGE ? 4u * (uint32_t)GP * (uint32_t)K : 64u; // four tile rows further / next step
+    // Single rows read the same way, and because an MFMA row may be any (tile row, column phase) pair they need no
+    // staging: the lane's 16 bytes of tile rows 4*i + ti are its A operands as they arrive.
+    const int lrow = PHASE ? ti : lane >> 4, lchunk = PHASE ? kq : lane & 15;
+    const uint32_t crow = STAGE || PHASE ? ((uint32_t)jp + (uint32_t)(16 * rb + lrow) * (uint32_t)GP) * (uint32_t)K + (uint32_t)(16 * lchunk)
+                                         : ((uint32_t)jp + (uint32_t)(16 * rb + rr) * (uint32_t)GP) * (uint32_t)K + (uint32_t)(16 * kg);
+    const uint32_t crow_step = STAGE || PHASE ? 4u * (uint32_t)GP * (uint32_t)K : 64u; // four tile rows further / next step
     const f16 *xl = p.x + layer * p.x_lstride + pass * 2 * K;
 
     auto issue = [&](SlabRegs<MT, SKIND, ZKIND> &r, int slab) __attribute__((always_inline)) {
@@ -275,7 +290,7 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
         // x: one coalesced piece per pair of batch rows (16 bytes per lane, 32 lanes per row)
         if constexpr (ROUTED) {
             // the row is in LDS already
-        } else if constexpr (STAGE) {
+        } else if constexpr (XSTAGE) {
             if (chain != CHAIN_LAST) { // (the last role reads its activations after the wait)
 #pragma unroll
                 for (int j = 0; j < (MT + 1) / 2; ++j) {
@@ -320,22 +335,24 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
     // Column m of the MFMA result depends on column m of B only, and columns m >= M are never read back, so lanes
     // past the batch simply re-read a valid column instead of needing zeros.
     const int mcol = lane & 15;
-    f16 *xs_w = &xs_lds[wave][0];
+    f16 *xs_w = &xs_lds[PHASE ? 0 : wave][0];
     const f16 *xs_r = xs_w + (kg * MT + (mcol < M ? mcol : 0)) * ENTRY;
 
-    f32x4 acc[F];
+    // single rows: one accumulator per (row group R, field i) at acc[R * F + i]
+    constexpr int NACC = PHASE ? 4 * F : F;
+    f32x4 acc[NACC];
 #pragma unroll
-    for (int i = 0; i < F; ++i)
+    for (int i = 0; i < NACC; ++i)
         acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float bias_acc[MT];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
         bias_acc[m] = 0.f;
 
-    uint8_t *code_w = &code_lds[wave][0];
+    uint8_t *code_w = &code_lds[STAGE ? wave : 0][0];
     auto compute = [&](const SlabRegs<MT, SKIND, ZKIND> &r, int slab) __attribute__((always_inline)) {
         // ------------------------------------------------------------ staging: x and the codes change lanes through LDS
-        if constexpr (STAGE) {
+        if constexpr (XSTAGE) {
 #pragma unroll
             for (int j = 0; j < (ROUTED ? 0 : (MT + 1) / 2); ++j) {
                 u32x4 xv = r.xw[j];
@@ -352,6 +369,8 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
                 }
                 *reinterpret_cast<u32x4 *>(&xw_lds[wave][2 * j + (lane >> 5)][8 * (lane & 31)]) = xv;
             }
+        }
+        if constexpr (STAGE) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
                 *reinterpret_cast<u32x4 *>(code_w + (4 * i + lrow) * CODE_PITCH + 16 * lchunk) = r.cw[i];
@@ -360,6 +379,7 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         // ------------------------------------------------------------ table phase, once per slab
+        f16x8 Bop[2] = {}; // single rows: the lane's own B operands, columns 0-7 and 8-15 of its 16
         if (tlane) {
             f16x2 sv[8], zv[8];
             const f16x2 sms = as_h2(r.sms * 0x10001u), smz = as_h2(r.smz * 0x10001u);
@@ -379,7 +399,7 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
                     if constexpr (ROUTED) {
                         const u32x4 *xp = reinterpret_cast<const u32x4 *>(&xn_lds[slab * kSlab + 16 * kq]);
                         x0 = xp[0], x1 = xp[1];
-                    } else if constexpr (STAGE) {
+                    } else if constexpr (XSTAGE) {
                         const u32x4 *xp = reinterpret_cast<const u32x4 *>(&xw_lds[wave][m][16 * kq]);
                         x0 = xp[0], x1 = xp[1];
                     } else {
@@ -396,10 +416,37 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
                         // B-operand order inside an 8-column block: columns (0,2,1,3,4,6,5,7)
                         const f16x2 *q = &a[4 * h];
                         const f16x8 o = {q[0].x, q[1].x, q[0].y, q[1].y, q[2].x, q[3].x, q[2].y, q[3].y};
-                        *reinterpret_cast<f16x8 *>(dst + (h * 4 * MT + m) * ENTRY) = o;
+                        if constexpr (PHASE)
+                            Bop[h] = o;
+                        else
+                            *reinterpret_cast<f16x8 *>(dst + (h * 4 * MT + m) * ENTRY) = o;
                     }
                 }
             }
+        }
+        if constexpr (PHASE) {
+            // -------------------------------------------------------- code phase, single rows: 4 row groups x 2 halves x F MFMAs
+            // straight from the registers the loads filled; B is the lane's own
+#pragma unroll
+            for (int R = 0; R < 4; ++R) {
+                const uint32_t d[4] = {r.cw[R].x, r.cw[R].y, r.cw[R].z, r.cw[R].w};
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const uint32_t d0 = d[2 * h], d1 = d[2 * h + 1];
+                    const uint32_t d0s = d0 >> 8, d1s = d1 >> 8;
+#pragma unroll
+                    for (int i = 0; i < F; ++i) {
+                        const uint32_t mk = Field<NBITS>::mask(i);
+                        const u32x4 Au = {d0 & mk, d0s & mk, d1 & mk, d1s & mk};
+                        acc[R * F + i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, Au), Bop[h], acc[R * F + i], 0, 0, 0);
+                    }
+                }
+            }
+            // the next slab's x overwrites this one's in LDS: keep that behind the table phase's reads
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            return;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -469,7 +516,7 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
         CHAIN_STAMP(p.chain, 1);
         if (threadIdx.x == 0)
             chain_passed(p.chain, p.chain_blocks);
-        if constexpr (STAGE && !ROUTED) {
+        if constexpr (XSTAGE && !ROUTED) {
             if (wave_on) {
 #pragma unroll
                 for (int i = 0; i < D; ++i) {
@@ -530,8 +577,36 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
     }
 
     // ---------------------------------------------------------------- wave tile -> LDS (zero term removed, unscaled)
+    if constexpr (PHASE) {
+        // The zero term of the lane's field: its 16 lanes are the four phases (neighbours) in each of the four lane groups.
+        float bz = bias_acc[0];
+        bz += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, bz), 0xB1, 0xF, 0xF, true));
+        bz += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, bz), 0x4E, 0xF, 0xF, true));
+        bz += __shfl_xor(bz, 16, kWave);
+        bz += __shfl_xor(bz, 32, kWave);
+        bz *= 1.0f / kXsScale;
+        // Lane (column c = lane & 15, group gq = lane >> 4) holds rows (rho = gq, phi = v) of column c in element v; the sum
+        // it wants is the one whose phase is the column's own, of the field the column belongs to.
+        const int phi = lane & 3, gq = lane >> 4;
+        float un = Field<NBITS>::unscale(0);
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
+        for (int i = 1; i < F; ++i)
+            un = ti == i ? Field<NBITS>::unscale(i) : un;
+#pragma unroll
+        for (int R = 0; R < 4; ++R) {
+            f32x4 t = acc[R * F];
+#pragma unroll
+            for (int i = 1; i < F; ++i)
+                t = ti == i ? acc[R * F + i] : t;
+            float e = phi == 0 ? t[0] : (phi == 1 ? t[1] : (phi == 2 ? t[2] : t[3]));
+            e += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, e), 0xB1, 0xF, 0xF, true));
+            e += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, e), 0x4E, 0xF, 0xF, true));
+            if (phi == 0 && tlane)
+                red_lds[wave][4 * R + gq][0][ti] = __builtin_fmaf(e, un, -bz);
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < (PHASE ? 0 : MT); ++m) {
         const float v = row16_sum(bias_acc[m]);
         if (tlane && kq == 0)
             bias_lds[wave][ti][m] = v * (1.0f / kXsScale);
@@ -539,7 +614,7 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    if (mcol < MT) {
+    if (!PHASE && mcol < MT) {
         float bz[F];
 #pragma unroll
         for (int i = 0; i < F; ++i)
