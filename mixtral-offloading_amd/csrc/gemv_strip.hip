@@ -101,7 +101,18 @@ struct StripParams {
     // chain_parts.hpp): the words of the chain and how many blocks of the launch have this one's role.
     int *chain;
     int chain_blocks;
+#ifdef HQQ_TUNING_BUILD
+    int skip; // timing experiments (results are then wrong): 1 leaves out the code phase, 2 the table phase
+    unsigned long long *stamps; // per-wave time stamps, [block][16 waves][16], or null
+#endif
 };
+#ifdef HQQ_TUNING_BUILD
+#define HQQ_SKIP(p, bit) (((p).skip & (bit)) != 0)
+#define STRIP_STAMP(i) do { if (p.stamps) st[i] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define HQQ_SKIP(p, bit) false
+#define STRIP_STAMP(i)
+#endif
 
 template <int MT, int SKIND, int ZKIND> struct SlabRegs {
     Raw16<SKIND> s;
@@ -126,6 +137,24 @@ template <int NBITS, int MT, int S, int D, int WAVES, int SKIND, int ZKIND, int 
 __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, const int by, const int bzi, const int chain)
 {
     static_assert(!NORM || (MT == 1 && WAVES >= 4), "the fused norm is for single rows and blocks of four waves and more");
+#ifdef HQQ_TUNING_BUILD
+    unsigned long long st[16] = {};
+#endif
+    STRIP_STAMP(0);
+    // Every kernel argument the prologue reads is fetched here, in one batch: read where they are used, they come in
+    // four or five scalar loads one after the other (each waits for the branch before it), 0.15 us apiece before the
+    // first weight load can be issued.
+    {
+        const StripLayer &A = p.layer[0], &B = p.layer[1];
+        asm volatile("" ::"s"(p.table), "s"(p.sel), "s"(p.x), "s"(p.x_lstride), "s"(p.K), "s"(p.M), "s"(p.passes), "s"(p.RB),
+                     "s"(p.NS), "s"(p.KS), "s"(p.BK), "s"(p.NL), "s"(p.grp[0].z_begin), "s"(p.grp[0].GP), "s"(p.grp[0].N),
+                     "s"(p.grp[1].z_begin), "s"(p.grp[2].z_begin), "s"(p.grp[3].z_begin), "s"(p.table_stride), "s"(p.table_first),
+                     "s"(p.sel_gstride), "s"(p.sel_lstride), "s"(p.first_lstride));
+        if constexpr (!GROUPED)
+            asm volatile("" ::"s"(A.codes), "s"(A.sq), "s"(A.zq), "s"(A.s_ms), "s"(A.s_mz), "s"(A.z_ms), "s"(A.z_mz), "s"(A.s_cols),
+                         "s"(A.s_inv), "s"(B.codes), "s"(B.sq), "s"(B.zq), "s"(B.s_ms), "s"(B.s_mz), "s"(B.z_ms), "s"(B.z_mz),
+                         "s"(B.s_cols), "s"(B.s_inv));
+    }
     const bool origin = bx == 0 && by == 0 && bzi == 0;
     const bool normed = NORM != 0 && chain != CHAIN_LAST; // whether the activations go through the norm
     if (chain == CHAIN_FIRST)
@@ -348,6 +377,14 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
 #pragma unroll
     for (int m = 0; m < MT; ++m)
         bias_acc[m] = 0.f;
+    // Single rows, 8-bit zeros under one whole-tensor meta pair: sum z * xs = zms * (sum zq * xs - zmz * sum xs), and
+    // both sums go to the matrix cores.  The zero bytes, masked in place like the codes (fp16 subnormals zq * 2^-24),
+    // are the A operand and the lane's own B operand the other: the diagonal of the result holds the lane's products
+    // added over the four lane groups; a second MFMA with A = 1 adds up xs alone.  (The zero is then not rounded to
+    // fp16 twice on the way, as the reference's is: the difference is below the rounding of the weights themselves.)
+    constexpr bool ZMFMA = PHASE && ZKIND == TK_U8_SCALAR;
+    f32x4 accz = {0.f, 0.f, 0.f, 0.f}, accx = {0.f, 0.f, 0.f, 0.f};
+    uint32_t zmeta_s = 0, zmeta_z = 0; // raw fp16 bits of the zero table's meta pair
 
     uint8_t *code_w = &code_lds[STAGE ? wave : 0][0];
     auto compute = [&](const SlabRegs<MT, SKIND, ZKIND> &r, int slab) __attribute__((always_inline)) {
@@ -380,12 +417,13 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         // ------------------------------------------------------------ table phase, once per slab
         f16x8 Bop[2] = {}; // single rows: the lane's own B operands, columns 0-7 and 8-15 of its 16
-        if (tlane) {
+        if (tlane && !HQQ_SKIP(p, 2)) {
             f16x2 sv[8], zv[8];
             const f16x2 sms = as_h2(r.sms * 0x10001u), smz = as_h2(r.smz * 0x10001u);
             const f16x2 zms = as_h2(r.zms * 0x10001u), zmz = as_h2(r.zmz * 0x10001u);
             decode16<SKIND>(r.s, sms, smz, sv);
-            decode16<ZKIND>(r.z, zms, zmz, zv);
+            if constexpr (!ZMFMA)
+                decode16<ZKIND>(r.z, zms, zmz, zv);
             const f16x2 k32 = {(f16)kXsScale, (f16)kXsScale};
 #pragma unroll
             for (int t = 0; t < 8; ++t)
@@ -409,7 +447,8 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
 #pragma unroll
                     for (int t = 0; t < 8; ++t) {
                         a[t] = sv[t] * as_h2(t < 4 ? x0[t & 3] : x1[t & 3]);
-                        bias_acc[m] = __builtin_amdgcn_fdot2(zv[t], a[t], bias_acc[m], false);
+                        if constexpr (!ZMFMA)
+                            bias_acc[m] = __builtin_amdgcn_fdot2(zv[t], a[t], bias_acc[m], false);
                     }
 #pragma unroll
                     for (int h = 0; h < 2; ++h) {
@@ -424,11 +463,24 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
                 }
             }
         }
+        if constexpr (ZMFMA) {
+            zmeta_s = r.zms, zmeta_z = r.zmz;
+            const u32x4 ones = {0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t z0 = r.z.q[2 * h], z1 = r.z.q[2 * h + 1];
+                const u32x4 Az = {z0 & 0x00FF00FFu, (z0 >> 8) & 0x00FF00FFu, z1 & 0x00FF00FFu, (z1 >> 8) & 0x00FF00FFu};
+                accz = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, Az), Bop[h], accz, 0, 0, 0);
+                accx = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, ones), Bop[h], accx, 0, 0, 0);
+            }
+        }
         if constexpr (PHASE) {
             // -------------------------------------------------------- code phase, single rows: 4 row groups x 2 halves x F MFMAs
             // straight from the registers the loads filled; B is the lane's own
 #pragma unroll
             for (int R = 0; R < 4; ++R) {
+                if (HQQ_SKIP(p, 1))
+                    break;
                 const uint32_t d[4] = {r.cw[R].x, r.cw[R].y, r.cw[R].z, r.cw[R].w};
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
@@ -503,11 +555,13 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
                 nv[c] = nv[c] + gload<f16x8>(p.norm_delta + kc);
         }
     }
+    STRIP_STAMP(1);
     if (wave_on) {
 #pragma unroll
         for (int i = 0; i < D; ++i)
             issue(regs[i], slab0 + i < p.NS ? slab0 + i : last);
     }
+    STRIP_STAMP(2);
     if (chain == CHAIN_LAST) {
         // the weights are on their way; now the activations: wait for the blocks that produce them, then read the slabs'
         // pieces at device scope (they may have been written through another XCD's L2)
@@ -573,21 +627,35 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
                 compute(regs[i % D], slab0 + i);
             if (i + D < S)
                 issue(regs[i % D], slab0 + i + D < p.NS ? slab0 + i + D : last);
+            if (i < 8)
+                STRIP_STAMP(3 + i);
         }
     }
 
     // ---------------------------------------------------------------- wave tile -> LDS (zero term removed, unscaled)
     if constexpr (PHASE) {
         // The zero term of the lane's field: its 16 lanes are the four phases (neighbours) in each of the four lane groups.
-        float bz = bias_acc[0];
-        bz += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, bz), 0xB1, 0xF, 0xF, true));
-        bz += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, bz), 0x4E, 0xF, 0xF, true));
-        bz += __shfl_xor(bz, 16, kWave);
-        bz += __shfl_xor(bz, 32, kWave);
+        const int phi = lane & 3, gq = lane >> 4;
+        float bz;
+        if constexpr (ZMFMA) {
+            // diagonal element (row = column) of lane (c, gq): gq == c >> 2, element c & 3; its four phases are neighbours
+            float zs = phi == 0 ? accz[0] : (phi == 1 ? accz[1] : (phi == 2 ? accz[2] : accz[3]));
+            float xsum = phi == 0 ? accx[0] : (phi == 1 ? accx[1] : (phi == 2 ? accx[2] : accx[3]));
+            const float zmsf = (float)__builtin_bit_cast(f16, (uint16_t)zmeta_s), zmzf = (float)__builtin_bit_cast(f16, (uint16_t)zmeta_z);
+            bz = zmsf * (zs * 16777216.0f - zmzf * xsum);
+            bz += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, bz), 0xB1, 0xF, 0xF, true));
+            bz += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, bz), 0x4E, 0xF, 0xF, true));
+            bz = __shfl(bz, (lane & 15) + 16 * ti, kWave); // from the lane group that holds the field's diagonal
+        } else {
+            bz = bias_acc[0];
+            bz += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, bz), 0xB1, 0xF, 0xF, true));
+            bz += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, bz), 0x4E, 0xF, 0xF, true));
+            bz += __shfl_xor(bz, 16, kWave);
+            bz += __shfl_xor(bz, 32, kWave);
+        }
         bz *= 1.0f / kXsScale;
         // Lane (column c = lane & 15, group gq = lane >> 4) holds rows (rho = gq, phi = v) of column c in element v; the sum
         // it wants is the one whose phase is the column's own, of the field the column belongs to.
-        const int phi = lane & 3, gq = lane >> 4;
         float un = Field<NBITS>::unscale(0);
 #pragma unroll
         for (int i = 1; i < F; ++i)
@@ -632,12 +700,99 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
                 *reinterpret_cast<float2 *>(dst) = make_float2(o[0], o[1]);
         }
     }
+    STRIP_STAMP(11);
     __syncthreads();
+    STRIP_STAMP(12);
 
-    // ---------------------------------------------------------------- block tile: 16 lanes per (layer, row, batch row)
     const bool alone = p.BK == 1;
     const int tile = bz * p.RB + rb;
     f16 *const y_rows = Gd.y + (int64_t)pass * 2 * N; // the pass's first batch row
+    // both projections rounded to fp16, SiLU in fp32 rounded once, product in fp16: as the reference's ops do
+    auto gate = [](float a, float b) __attribute__((always_inline)) -> f16 {
+        const float u = (float)(f16)a;
+        const f16 act = (f16)(u / (1.0f + __expf(-u)));
+        return act * (f16)b;
+    };
+    // two down projections, each rounded to fp16 and scaled by its routing weight, added in layer order: the bits
+    // two launches with row_scale (the second accumulating) would give
+    auto both = [&](float a, float b, int m, f16 prev) __attribute__((always_inline)) -> f16 {
+        const f16 t0 = (f16)a * p.row_scale[m], t1 = (f16)b * p.row_scale[p.rs_lstride + m];
+        return p.accumulate ? (f16)((f16)(prev + t0) + t1) : (f16)(t0 + t1);
+    };
+
+    // ---------------------------------------------------------------- a block that holds all of K finishes its tile
+    // A thread per (tile row, batch row) adds the waves' sums in wave order and applies the epilogue.
+    if (alone) {
+        for (int u = threadIdx.x; u < 16 * MT; u += WAVES * 64) {
+            const int r_t = u / MT, m_t = u % MT;
+            if (m_t >= M)
+                continue;
+            float o[2][F];
+#pragma unroll
+            for (int i = 0; i < F; ++i)
+                o[0][i] = o[1][i] = 0.f;
+            for (int w = 0; w < p.KS; ++w) {
+#pragma unroll
+                for (int l = 0; l < (EPI == 0 ? 1 : 2); ++l) {
+                    const float *src = &red_lds[l * p.KS + w][r_t][m_t][0];
+#pragma unroll
+                    for (int i = 0; i < F; ++i)
+                        o[l][i] += src[i];
+                }
+            }
+            const int r = 16 * rb + r_t;
+            const int64_t n = (int64_t)F * (jp + (int64_t)r * GP); // outputs n .. n+F-1
+            f16 *dst = y_rows + (int64_t)m_t * N + n;
+            f16 hv[F];
+#pragma unroll
+            for (int i = 0; i < F; ++i) {
+                if constexpr (EPI == 1) {
+                    hv[i] = gate(o[0][i], o[1][i]);
+                } else if constexpr (EPI == 2) {
+                    hv[i] = both(o[0][i], o[1][i], m_t, p.accumulate ? dst[i] : (f16)0);
+                } else {
+                    f16 val = (f16)o[0][i];
+                    if (Gd.bias)
+                        val = val + Gd.bias[n + i];
+                    if (p.row_scale)
+                        val = val * p.row_scale[m_t];
+                    if (p.accumulate)
+                        val = dst[i] + val;
+                    hv[i] = val;
+                }
+            }
+            if (EPI == 0 && chain == CHAIN_FIRST) { // read by later blocks of this grid, on any XCD: stored at device scope
+                if constexpr (F == 4)
+                    chain_store(dst, (f16x4){hv[0], hv[1], hv[2], hv[3]});
+                else
+                    chain_store(dst, (f16x2){hv[0], hv[1]});
+            } else if constexpr (F == 4) {
+                *reinterpret_cast<f16x4 *>(dst) = (f16x4){hv[0], hv[1], hv[2], hv[3]};
+            } else {
+                *reinterpret_cast<f16x2 *>(dst) = (f16x2){hv[0], hv[1]};
+            }
+        }
+#ifdef HQQ_TUNING_BUILD
+        STRIP_STAMP(13);
+        if (p.stamps && lane == 0) {
+            unsigned long long *d = p.stamps + ((size_t)((bzi * gridDim.y + by) * gridDim.x + bx) * 16 + wave) * 16;
+            for (int i = 0; i < 14; ++i)
+                d[i] = st[i];
+            d[14] = __builtin_amdgcn_s_getreg((31 << 11) | 4);  // HW_ID: wave, SIMD, CU, shader array and engine
+            d[15] = __builtin_amdgcn_s_getreg((31 << 11) | 20); // XCC_ID
+        }
+#endif
+        if (chain == CHAIN_FIRST) {
+            CHAIN_STAMP(p.chain, 2);
+            chain_signal(p.chain, CHAIN_FIRST_DONE, p.chain_blocks, CHAIN_GO_FIRST, kChainGoFirst);
+        }
+        if (chain != CHAIN_NONE)
+            CHAIN_STAMP(p.chain, 3);
+        return;
+    }
+
+
+    // ---------------------------------------------------------------- block tile: 16 lanes per (layer, row, batch row)
     for (int t = threadIdx.x; t < p.NL * 16 * MT * 16; t += WAVES * 64) {
         const int w = t & 15, u = t >> 4;
         const int l_t = u / (16 * MT), r_t = (u / MT) & 15, m_t = u % MT;
@@ -658,7 +813,7 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
             continue;
         const int r = 16 * rb + r_t;
         const int64_t n = (int64_t)F * (jp + (int64_t)r * GP); // outputs n .. n+F-1
-        if (!alone && (EPI == 1 || !p.slots)) {
+        if (EPI == 1 || !p.slots) {
             // device-scope stores: written through the (per-XCD, mutually non-coherent) L2 so that the finishing
             // block, which may run on another XCD, can read them without any cache-wide flush
             float *dst = (l_t ? Gd.part[1] : Gd.part[0]) + ((int64_t)kb * M + m_t) * N + n;
@@ -667,82 +822,10 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
                 __hip_atomic_store(dst + i, o[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             continue;
         }
-        if (EPI != 0 || !alone) {
-            float *dst = &fin_lds[l_t][r_t][m_t][0];
+        float *dst = &fin_lds[l_t][r_t][m_t][0];
 #pragma unroll
-            for (int i = 0; i < F; ++i)
-                dst[i] = o[i];
-        } else {
-            f16 *dst = y_rows + (int64_t)m_t * N + n;
-            f16 hv[F];
-#pragma unroll
-            for (int i = 0; i < F; ++i) {
-                f16 val = (f16)o[i];
-                if (Gd.bias)
-                    val = val + Gd.bias[n + i];
-                if (p.row_scale)
-                    val = val * p.row_scale[m_t];
-                if (p.accumulate)
-                    val = dst[i] + val;
-                hv[i] = val;
-            }
-            if (chain == CHAIN_FIRST) { // read by later blocks of this grid, on any XCD: stored at device scope
-                if constexpr (F == 4)
-                    chain_store(dst, (f16x4){hv[0], hv[1], hv[2], hv[3]});
-                else
-                    chain_store(dst, (f16x2){hv[0], hv[1]});
-            } else if constexpr (F == 4) {
-                *reinterpret_cast<f16x4 *>(dst) = (f16x4){hv[0], hv[1], hv[2], hv[3]};
-            } else {
-                *reinterpret_cast<f16x2 *>(dst) = (f16x2){hv[0], hv[1]};
-            }
-        }
-    }
-
-    // both projections rounded to fp16, SiLU in fp32 rounded once, product in fp16: as the reference's ops do
-    auto gate = [](float a, float b) __attribute__((always_inline)) -> f16 {
-        const float u = (float)(f16)a;
-        const f16 act = (f16)(u / (1.0f + __expf(-u)));
-        return act * (f16)b;
-    };
-    // two down projections, each rounded to fp16 and scaled by its routing weight, added in layer order: the bits
-    // two launches with row_scale (the second accumulating) would give
-    auto both = [&](float a, float b, int m, f16 prev) __attribute__((always_inline)) -> f16 {
-        const f16 t0 = (f16)a * p.row_scale[m], t1 = (f16)b * p.row_scale[p.rs_lstride + m];
-        return p.accumulate ? (f16)((f16)(prev + t0) + t1) : (f16)(t0 + t1);
-    };
-
-    if (alone) {
-        if constexpr (EPI != 0) {
-            __syncthreads();
-            for (int u = threadIdx.x; u < 16 * MT; u += WAVES * 64) {
-                const int r_t = u / MT, m_t = u % MT;
-                if (m_t >= M)
-                    continue;
-                const int r = 16 * rb + r_t;
-                const int64_t n = (int64_t)F * (jp + (int64_t)r * GP);
-                f16 *dst = y_rows + (int64_t)m_t * N + n;
-                f16 hv[F];
-#pragma unroll
-                for (int i = 0; i < F; ++i) {
-                    if constexpr (EPI == 1)
-                        hv[i] = gate(fin_lds[0][r_t][m_t][i], fin_lds[1][r_t][m_t][i]);
-                    else
-                        hv[i] = both(fin_lds[0][r_t][m_t][i], fin_lds[1][r_t][m_t][i], m_t, p.accumulate ? dst[i] : (f16)0);
-                }
-                if constexpr (F == 4)
-                    *reinterpret_cast<f16x4 *>(dst) = (f16x4){hv[0], hv[1], hv[2], hv[3]};
-                else
-                    *reinterpret_cast<f16x2 *>(dst) = (f16x2){hv[0], hv[1]};
-            }
-        }
-        if (chain == CHAIN_FIRST) {
-            CHAIN_STAMP(p.chain, 2);
-            chain_signal(p.chain, CHAIN_FIRST_DONE, p.chain_blocks, CHAIN_GO_FIRST, kChainGoFirst);
-        }
-        if (chain != CHAIN_NONE)
-            CHAIN_STAMP(p.chain, 3);
-        return;
+        for (int i = 0; i < F; ++i)
+            dst[i] = o[i];
     }
 
     // ---------------------------------------------------------------- accumulation slots: one atomic per output
@@ -841,8 +924,10 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
     }
 }
 
+// (single rows, several slabs per wave, one in flight: the form chosen for launches of more blocks than compute
+// units, which must fit four waves to a SIMD, i.e. stay within 128 registers, for two blocks to share a unit)
 template <int NBITS, int MT, int S, int D, int WAVES, int SKIND, int ZKIND, int EPI, bool GROUPED = false, int NORM = 0>
-__global__ __launch_bounds__(WAVES * 64) void gemv_strip_kernel(StripParams p)
+__global__ __launch_bounds__(WAVES * 64, (MT == 1 && S > 1 && D == 1 && WAVES == 8) ? 4 : 1) void gemv_strip_kernel(StripParams p)
 {
     strip_block<NBITS, MT, S, D, WAVES, SKIND, ZKIND, EPI, GROUPED, NORM>(p, (int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z, CHAIN_NONE);
 }
@@ -887,6 +972,10 @@ __global__ void zero_words_kernel(uint32_t *p, size_t n)
     for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
         p[i] = 0;
 }
+
+#ifdef HQQ_TUNING_BUILD
+unsigned long long *g_strip_stamps = nullptr; // device buffer the launches write their waves' time stamps to
+#endif
 
 struct StripPlan {
     int F, GP, RB, NS, MT, S, D, WAVES, KS, BK, SKIND, ZKIND;
@@ -970,7 +1059,12 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, StripPlan &pl, int64_t ti
         return false;
     pl.S = S, pl.KS = KS, pl.BK = BK;
     pl.WAVES = KS * NL > 8 ? 16 : (KS * NL > 4 ? 8 : 4);
-    pl.D = S < 2 ? S : 2; // slabs of a wave in flight at once
+    // Slabs of a wave in flight at once: two, with one block to a compute unit; one when the launch has more blocks
+    // than the chip has compute units (the gates of a token's two experts: 448), so that two blocks fit into a unit
+    // (under 128 registers a wave) and cover each other's waits (measured on the 32-layer decode step: 440 -> 483 tok/s).
+    pl.D = S < 2 ? S : 2;
+    if (pl.MT == 1 && S > 1)
+        pl.D = tuning_int("HQQ_STRIP_D", tiles * BK > 256 ? 1 : 2) == 1 ? 1 : 2;
     return true;
 }
 
@@ -1023,10 +1117,18 @@ void launch_depth(const StripParams &p, const StripPlan &pl, dim3 grid, hipStrea
 {
     if (pl.S == 1)
         launch_waves<NBITS, MT, 1, 1, EPI, GROUPED>(p, pl, grid, s);
-    else if (pl.S == 2)
+    else if (pl.S == 2 && (MT > 1 || pl.D == 2))
         launch_waves<NBITS, MT, 2, 2, EPI, GROUPED>(p, pl, grid, s);
-    else if constexpr (MT <= 2)
-        launch_waves<NBITS, MT, 4, 2, EPI, GROUPED>(p, pl, grid, s);
+    else if (pl.S == 2) {
+        if constexpr (MT == 1)
+            launch_waves<NBITS, MT, 2, 1, EPI, GROUPED>(p, pl, grid, s);
+    } else if (MT > 1 || pl.D == 2) {
+        if constexpr (MT <= 2)
+            launch_waves<NBITS, MT, 4, 2, EPI, GROUPED>(p, pl, grid, s);
+    } else {
+        if constexpr (MT == 1)
+            launch_waves<NBITS, MT, 4, 1, EPI, GROUPED>(p, pl, grid, s);
+    }
 }
 
 // several groups in one launch and the two-expert sum exist for single-row batches only (the decode step)
@@ -1165,6 +1267,10 @@ int build_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, StripPara
     if (!alone && ((j.EPI == 0 && j.NL == 1) || (j.EPI == 2 && j.NL == 2 && j.NG == 1)) && pl.BK <= 8 && slot * (int64_t)sizeof(unsigned long long) <= (int64_t)kSlotBytes)
         p.slots = reinterpret_cast<unsigned long long *>(base + kCounterBytes);
     p.row_scale = j.row_scale, p.rs_lstride = j.rs_lstride, p.accumulate = j.accumulate;
+#ifdef HQQ_TUNING_BUILD
+    p.skip = tuning_int("HQQ_STRIP_SKIP", 0);
+    p.stamps = g_strip_stamps;
+#endif
     if (j.norm_weight) {
         // every launch shape the planner can pick for these jobs has the fused-norm form except blocks under four waves
         const bool plain = j.EPI == 0 && j.NL == 1 && !j.gate_w;
@@ -1407,5 +1513,9 @@ int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s)
 }
 
 size_t workspace_head_bytes() { return kHeadBytes; }
+
+#ifdef HQQ_TUNING_BUILD
+extern "C" void hqq_tuning_strip_stamps(void *buf) { g_strip_stamps = static_cast<unsigned long long *>(buf); }
+#endif
 
 } // namespace hqq
