@@ -177,18 +177,55 @@ def random_desc(nbits, n, k, gs, seed, dev):
 PROFILE = os.path.join(ROOT, "profiles", "gemv_strip_kernel_ffn_2bit_g16_m1.txt")
 
 
+KERNEL_SOURCES = ("gemv_strip.hip", "gemv_parts.hpp")
+
+
+def kernel_source_hash():
+    """sha256 over the sources of the dominant kernel: the counter profile records the hash it was taken with."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "mixtral-offloading_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def profiled_traffic():
     """HBM bytes per launch of the dominant kernel as the tracked counter profile records them (a line
     `traffic_bytes_per_launch: <int>`, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this command scaled by a copy of
-    known size); None when the profile has no such line."""
+    known size).  The figure is a recorded one, not measured by this run: it is reported only when the profile's
+    `kernel_source_sha256:` line names the kernel sources as they are now, else None with the reason."""
+    traffic, taken_with = None, None
     try:
         with open(PROFILE) as f:
             for line in f:
                 if line.startswith("traffic_bytes_per_launch:"):
-                    return int(line.split(":")[1].split()[0].replace(",", ""))
+                    traffic = int(line.split(":")[1].split()[0].replace(",", ""))
+                if line.startswith("kernel_source_sha256:"):
+                    taken_with = line.split(":")[1].strip()
     except OSError:
-        pass
-    return None
+        return None, "no profile"
+    if traffic is None:
+        return None, "the profile has no traffic line"
+    try:
+        now = kernel_source_hash()
+    except OSError:
+        return None, "kernel sources not found"
+    if taken_with != now:
+        return None, f"the kernel sources changed since the profile was taken ({taken_with} -> {now})"
+    return traffic, f"recorded in the profile for kernel sources {now}"
+
+
+def load_probe():
+    """The streaming-read probe (csrc/probe/stream_read.hip), a library of its own beside the product's."""
+    import ctypes
+
+    path = os.path.join(ROOT, "mixtral-offloading_amd", "lib", "libhqq_probe.so")
+    lib = ctypes.CDLL(path)
+    lib.hqq_probe_stream_read.restype = ctypes.c_int
+    lib.hqq_probe_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p]
+    return lib
 
 
 def survey_section(dev):
@@ -199,6 +236,7 @@ def survey_section(dev):
     from mixtral_offloading_amd import _lib, hip_kernels, packing
 
     lib = _lib.lib
+    probe = load_probe()
     stream = torch.cuda.Stream(device=dev)
     rows = []
 
@@ -228,9 +266,9 @@ def survey_section(dev):
             slots = max(1, pool.numel() // span)
 
             def f(i):
-                rc = lib.hqq_probe_stream_read(pool.data_ptr() + (i % slots) * span, int(nbytes), sink.data_ptr(), stream.cuda_stream)
+                rc = probe.hqq_probe_stream_read(pool.data_ptr() + (i % slots) * span, int(nbytes), sink.data_ptr(), stream.cuda_stream)
                 if rc != 0:
-                    raise _lib.HqqError(rc, "hqq_probe_stream_read")
+                    raise RuntimeError(f"hqq_probe_stream_read: {rc}")
 
             ceilings[key] = timed(f, 48)
         return ceilings[key]
@@ -459,10 +497,15 @@ def main():
     ap.add_argument("--survey", action="store_true",
                     help="also time every kernel of the path (packers, de-quantiser, 2/3/4-bit matmuls at the Mixtral-8x7B "
                          "shapes and batches) and add the table as 'kernels'")
+    ap.add_argument("--kernel-hash", action="store_true", help="print the hash of the dominant kernel's sources (the "
+                    "counter profile records it beside its traffic figure) and exit")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain 256 MiB device copies, so that a counter run can scale FETCH_SIZE / WRITE_SIZE "
                          "by what the same counters read for a copy of known size")
     args = ap.parse_args()
+    if args.kernel_hash:
+        print(kernel_source_hash())
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: this build runs on a single MI355X (--gpus 1)", file=sys.stderr)
         sys.exit(2)
@@ -519,6 +562,31 @@ def main():
 
     ms_step = timed(ffn_step, args.warmup, args.steps)
     ms_gate = timed(gate_up_step, args.warmup, args.steps)
+
+    # Two reference points for the dominant kernel, timed the same way in the same process: the same launch on ONE
+    # expert (its 44 MB stay in the 256 MB last-level cache, so HBM is out of the picture), and a plain 128-bit
+    # streaming read of the launch's algorithmic bytes, rotating over more than 256 MB like the kernel itself.
+    def gate_up_resident(i):
+        w1, _, w3 = descs[0]
+        rc = lib.hqq_gate_up(w1.ref, w3.ref, x.data_ptr(), m, h.data_ptr(), ws.data_ptr(), ws.numel(), sp)
+        if rc != 0:
+            raise _lib.HqqError(rc, "hqq_gate_up")
+
+    ms_gate_resident = timed(gate_up_resident, args.warmup, args.steps)
+    probe = load_probe()
+    nbytes = gate_up_bytes(m)
+    span = (nbytes + 4095) // 4096 * 4096
+    slots = (320 << 20) // span + 1
+    pool = torch.empty(slots * span, dtype=torch.uint8, device=dev).fill_(3)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+
+    def stream_read_step(i):
+        rc = probe.hqq_probe_stream_read(pool.data_ptr() + (i % slots) * span, nbytes, sink.data_ptr(), sp)
+        if rc != 0:
+            raise RuntimeError(f"hqq_probe_stream_read: {rc}")
+
+    ms_read = timed(stream_read_step, args.warmup, args.steps)
+    del pool
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
@@ -528,6 +596,7 @@ def main():
         print(f"calibration: 4 device copies of {src.numel()} bytes (reads {src.numel()}, writes {src.numel()} each)",
               file=sys.stderr)
 
+    traffic, traffic_note = profiled_traffic()
     value = ffn_step_bytes(m) / (ms_step * 1e-3) / 1e9
     achieved = gate_up_bytes(m) / (ms_gate * 1e-3) / 1e9
     out = {
@@ -541,11 +610,14 @@ def main():
                    "bytes_per_step": ffn_step_bytes(m), "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     # read from the tracked counter profile (measured at batch 1 only)
-                     "traffic": profiled_traffic() if m == 1 else None,
-                     "traffic_source": "profiles/gemv_strip_kernel_ffn_2bit_g16_m1.txt",
+                     # a recorded figure, read from the tracked counter profile (taken at batch 1), not measured here
+                     "traffic": traffic if m == 1 else None,
+                     "traffic_source": "profiles/gemv_strip_kernel_ffn_2bit_g16_m1.txt: " + traffic_note,
                      "kernel": "gemv_strip_kernel<2,1,4,2,8,1,2,1,false,0> as launched by hqq_gate_up (w1 and w3 in one grid, one launch)",
-                     "bytes_per_launch": gate_up_bytes(m), "us_per_launch": round(ms_gate * 1e3, 3)},
+                     "bytes_per_launch": gate_up_bytes(m), "us_per_launch": round(ms_gate * 1e3, 3),
+                     "us_per_launch_cache_resident": round(ms_gate_resident * 1e3, 3),
+                     "stream_read_us": round(ms_read * 1e3, 3),
+                     "frac_of_stream_read": round(ms_read / ms_gate, 4)},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(experts[0], x, attention=make_attention(dev))

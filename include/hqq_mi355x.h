@@ -298,11 +298,6 @@ int hqq_quantize_groups(const void *w, int32_t w_is_fp32, int64_t rows, int64_t 
 int hqq_quantize_whole(const void *x_f32, int64_t n, int32_t nbits, void *codes_u8, void *inv_scale_f32, void *zero_f32,
                        void *workspace, size_t workspace_bytes, void *stream);
 
-/* ---- measurement aid, no counterpart in the reference: a plain 128-bit streaming read of `bytes` bytes (16-byte aligned)
- *      that computes nothing; sink_u32 is one device word that is never written in practice.  Its duration is the
- *      ceiling for any launch that must fetch the same bytes, which is what bench.py --survey prints beside each GEMV. */
-int hqq_probe_stream_read(const void *src, size_t bytes, void *sink_u32, void *stream);
-
 /* ---- which kernel family a call would use (for tests and profiles): 0 general, 1 MFMA small-batch, 2 MFMA tile,
  *      3 three-bit vector kernel, 4 MFMA kernel with weights dequantised into shared memory (reads 3-bit words as
  *      they are stored).                                                                                              */

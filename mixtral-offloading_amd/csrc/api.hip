@@ -389,9 +389,11 @@ constexpr int kMaxDevices = 64;
 static std::mutex scratch_mutex;
 static void *scratch_ptr[kMaxDevices]; // per device, null until the first call there
 
-// the device address of `scratch` on the current device; the first call on a device also clears the head
-// (counters and accumulation slots) with the fill kernel, on the caller's stream
-static int static_scratch(void **out, hipStream_t s)
+// The device address of `scratch` on the current device.  Nothing is cleared here: a file-scope device array is
+// zero when the module is loaded, and every launch leaves the head (counters, accumulation slots) at zero again.  (A
+// fill recorded on the first caller's stream would not be ordered against a first call on another stream, and a
+// captured one would be replayed with every graph launch.)
+static int static_scratch(void **out)
 {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
@@ -407,9 +409,6 @@ static int static_scratch(void **out, hipStream_t s)
             return static_cast<int>(e);
         if (!ptr || (reinterpret_cast<uintptr_t>(ptr) & 255u))
             return HQQ_E_ALIGN;
-        const int rc = launch_zero_workspace_head(ptr, kStaticScratchBytes, s);
-        if (rc != HQQ_OK)
-            return rc;
         scratch_ptr[dev] = ptr;
     }
     *out = scratch_ptr[dev];
@@ -430,7 +429,7 @@ int hqq_expert_ffn_static(const hqq_linear *w1, const hqq_linear *w2, const hqq_
     if (hqq_expert_ffn_workspace_bytes(w1, w2, w3, M) > kStaticScratchBytes)
         return HQQ_E_WORKSPACE; // beyond the built-in scratch: use hqq_expert_ffn with a workspace of the caller's
     void *ws = nullptr;
-    if ((rc = static_scratch(&ws, (hipStream_t)stream)) != HQQ_OK)
+    if ((rc = static_scratch(&ws)) != HQQ_OK)
         return rc;
     return hqq_expert_ffn(w1, w2, w3, x_f16, M, y_f16, row_scale_f16, accumulate, ws, kStaticScratchBytes, stream);
 }

@@ -366,26 +366,6 @@ bool dequantize_words(const hqq_linear *l, const Table &sc, const Table &zr, f16
     return true;
 }
 
-// Plain streaming read: every thread takes 128-bit words a grid stride apart, four in flight.  It computes nothing
-// (the words are folded into one value that is stored only if it has an impossible bit pattern), so its duration is
-// what the memory system needs to deliver `bytes` to a launch: the ceiling a GEMV over the same bytes is measured
-// against.
-__global__ __launch_bounds__(512) void stream_read_kernel(const u32x4 *__restrict__ src, size_t n16, uint32_t *sink)
-{
-    u32x4 a = {0, 0, 0, 0};
-    size_t i = (size_t)blockIdx.x * 512 + threadIdx.x;
-    const size_t stride = (size_t)gridDim.x * 512;
-    for (; i + 3 * stride < n16; i += 4 * stride) {
-        const u32x4 v0 = src[i], v1 = src[i + stride], v2 = src[i + 2 * stride], v3 = src[i + 3 * stride];
-        a ^= v0 ^ v1 ^ v2 ^ v3;
-    }
-    for (; i < n16; i += stride)
-        a ^= src[i];
-    const uint32_t v = a.x ^ a.y ^ a.z ^ a.w;
-    if (v == 0x9e3779b9u && (a.x & a.y & a.z) == 0x7f4a7c15u)
-        sink[0] = v;
-}
-
 } // namespace
 
 int launch_silu_mul(const f16 *a, const f16 *b, f16 *h, int64_t count, hipStream_t s)
@@ -495,22 +475,6 @@ int hqq_dequantize(const hqq_linear *l, void *w_out_f16, void *stream)
         dequantize_kernel<2><<<grid_for(total), kThreads, 0, s>>>(l->codes, sc, zr, l->N, l->K, G, (f16 *)w_out_f16);
     else
         dequantize_kernel<3><<<grid_for(total), kThreads, 0, s>>>(l->codes, sc, zr, l->N, l->K, G, (f16 *)w_out_f16);
-    return launch_status();
-}
-
-int hqq_probe_stream_read(const void *src, size_t bytes, void *sink_u32, void *stream)
-{
-    if (!src || !sink_u32)
-        return HQQ_E_NULL;
-    if (reinterpret_cast<uintptr_t>(src) & 15u)
-        return HQQ_E_ALIGN;
-    const size_t n16 = bytes / 16;
-    if (n16 == 0)
-        return HQQ_OK;
-    size_t blocks = (n16 + 4 * 512 - 1) / (4 * 512);
-    blocks = blocks < 1 ? 1 : (blocks > 2048 ? 2048 : blocks);
-    stream_read_kernel<<<dim3((unsigned)blocks), dim3(512), 0, (hipStream_t)stream>>>(static_cast<const u32x4 *>(src), n16,
-                                                                                   static_cast<uint32_t *>(sink_u32));
     return launch_status();
 }
 

@@ -94,7 +94,6 @@ _SIGNATURES = {
     "hqq_attention_decode_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32]),
     "hqq_attention_decode_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_size_t, c_void_p]),
-    "hqq_probe_stream_read": (c_int, [c_void_p, c_size_t, c_void_p, c_void_p]),
     "hqq_slab_h2d_async": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
     "hqq_stream_wait_event": (c_int, [c_void_p, c_void_p]),
     "hqq_lru_create": (c_void_p, [c_int32, c_int32]),

@@ -471,14 +471,18 @@ class AttentionChain:
         return y
 
 
-def attention_chain_error(device) -> bool:
+def attention_chain_error(device, clear: bool = False) -> bool:
     """Whether a chained launch on one of this device's workspaces has ever given up a wait (it never should): reads
-    a word per workspace back from the device, so call it outside the decode loop."""
+    a word per workspace back from the device, so call it outside the decode loop.  ``clear`` resets the words."""
     off = int(_lib.lib.hqq_attention_chain_error_offset())
     bad = False
     for (index, _stream), ws in list(_workspaces.items()):
         if index == device.index and ws.numel() >= off + 4:
-            bad = bad or bool(ws[off:off + 4].view(torch.int32).item())
+            word = ws[off:off + 4].view(torch.int32)
+            if bool(word.item()):
+                bad = True
+                if clear:
+                    word.zero_()
     return bad
 
 

@@ -10,6 +10,7 @@ HIP library's kernels; everything else here is plumbing, not the measured path."
 from __future__ import annotations
 
 import math
+import warnings
 from typing import Optional
 
 import torch
@@ -442,6 +443,8 @@ class MixtralForCausalLM(nn.Module):
     @torch.inference_mode()
     def generate(self, prompt_ids: torch.Tensor, max_new_tokens: int, cache=None):
         """Greedy decoding, batch 1; returns the generated ids (max_new_tokens,)."""
+        from . import hip_kernels
+        own_cache = cache is None
         cache = cache or self.new_cache(prompt_ids.numel() + max_new_tokens)
         logits = self.forward(prompt_ids, cache, 0)
         tok = logits[-1].argmax()
@@ -452,4 +455,13 @@ class MixtralForCausalLM(nn.Module):
             tok = logits[-1].argmax()
             out.append(tok)
             pos += 1
-        return torch.stack(out)
+        ids = torch.stack(out)
+        # The chained attention launch hands results from block to block inside one grid and assumes that workgroups
+        # start in index order; a block whose bounded wait ran out sets an error word and carries on with whatever it
+        # read.  That never happened in any run, but tokens and cache would be wrong if it did: check once per call,
+        # and if the word is set, clear it, stop chaining for this model and decode again with the three launches.
+        if getattr(self, "chain_attention", True) and hip_kernels.attention_chain_error(prompt_ids.device, clear=True):
+            warnings.warn("a chained attention launch gave up a wait; decoding again without chaining")
+            self.chain_attention = False
+            return self.generate(prompt_ids, max_new_tokens, None if own_cache else cache)
+        return ids

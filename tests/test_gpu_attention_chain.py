@@ -140,3 +140,31 @@ def test_chain_replayed_from_a_graph():
         assert torch.equal(y, want) and torch.equal(x_sum, want_sum)
         assert torch.equal(ck2[:, p], ck[:, p]) and torch.equal(cv2[:, p], cv[:, p])
     assert not hip_kernels.attention_chain_error(torch.device("cuda", torch.cuda.current_device()))
+
+
+def test_generate_notices_a_chain_that_gave_up_and_decodes_again_without_it():
+    """The error word of the chained launch is forced from the host (no kernel ever gives up a wait in a test):
+    generate() must notice it, clear it, stop chaining for the model and return the tokens of the three-launch path."""
+    import warnings
+    from mixtral_offloading_amd import _lib, build_model as bm, hip_kernels
+    cfg = bm.mixtral_config(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                            num_key_value_heads=2, vocab_size=128, num_local_experts=8)
+    off = bm.OffloadConfig(main_size=16, offload_size=0, buffer_size=1, offload_per_layer=0)
+    dev = torch.device("cuda:0")
+    model = bm.build_model(dev, bm.default_quant_config(), off, model_config=cfg, seed=5, max_positions=64)
+    prompt = torch.arange(7, device="cuda")
+    model.chain_attention = True
+    want = model.generate(prompt, 6)
+    assert not hip_kernels.attention_chain_error(dev)
+    word_at = int(_lib.lib.hqq_attention_chain_error_offset())
+    ws = hip_kernels.workspace(dev, word_at + 4)
+    ws[word_at:word_at + 4].view(torch.int32).fill_(1)
+    assert hip_kernels.attention_chain_error(dev)
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        got = model.generate(prompt, 6)
+    assert any("chained attention" in str(w.message) for w in caught)
+    assert torch.equal(got, want)
+    assert model.chain_attention is False and not hip_kernels.attention_chain_error(dev)
+    torch.cuda.synchronize()
+    assert not bool(ws[: 576 * 1024].any())  # the workspace head is at zero again for the launches that rely on it
