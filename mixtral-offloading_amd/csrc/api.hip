@@ -272,7 +272,7 @@ int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, i
     const bool alike = w1->nbits == w3->nbits && w1->group_size == w3->group_size;
     // one fused launch where a kernel family has one for the batch; the decode kernels need no more workspace than
     // they check for themselves
-    const bool prefer_tile = tile_supported(w1, M) && tile_supported(w3, M) && !strip_supported(w1, M) &&
+    const bool prefer_tile = tile_supported(w1, M) && tile_supported(w3, M) && !strip_gate_supported(w1, w3, M) &&
                              pick_family(w1, M) != FAM_LDS && pick_family(w3, M) != FAM_LDS;
     if (alike && !prefer_tile && smallbatch_supported(w1, M) && smallbatch_supported(w3, M))
         return launch_smallbatch_gate_up(w1, w3, x, M, h, workspace, workspace_bytes, s);
@@ -335,7 +335,7 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
         return launch_vec3_down(w2, a, b, M, y, mm, mm_bytes, ep, s);
     }
     // fused gate: decode batches always; wider ones only where the tile kernel does not take the shape
-    const bool prefer_tile = tile_supported(w1, M) && tile_supported(w3, M) && !strip_supported(w1, M) &&
+    const bool prefer_tile = tile_supported(w1, M) && tile_supported(w3, M) && !strip_gate_supported(w1, w3, M) &&
                              pick_family(w1, M) != FAM_LDS && pick_family(w3, M) != FAM_LDS;
     const bool fast13 = !prefer_tile && smallbatch_supported(w1, M) && smallbatch_supported(w3, M) && !w1->bias &&
                         !w3->bias && w1->nbits == w3->nbits && w1->group_size == w3->group_size;

@@ -1315,17 +1315,28 @@ int run_job(const StripJob &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t
 
 } // namespace
 
+// Batches of three rows and more go to the batch kernel (gemv_batch.hip) where it takes the shape.
+static bool use_batch(const hqq_linear *l, int64_t M) { return M >= 3 && !tuning_flag("HQQ_BATCH_OFF") && batch_supported(l, M); }
+
 bool strip_supported(const hqq_linear *l, int64_t M)
 {
     StripPlan pl;
-    return make_plan(l, M, 1, pl);
+    return make_plan(l, M, 1, pl) || use_batch(l, M);
+}
+
+bool strip_gate_supported(const hqq_linear *w1, const hqq_linear *w3, int64_t M)
+{
+    if (M >= 3 && !tuning_flag("HQQ_BATCH_OFF") && batch_gate_supported(w1, w3, M))
+        return true;
+    StripPlan a, b;
+    return make_plan(w1, M, 2, a) && make_plan(w3, M, 2, b) && same_family(w1, w3) && w1->N == w3->N;
 }
 
 size_t strip_workspace_bytes(const hqq_linear *l, int64_t M)
 {
     StripPlan pl;
     if (!make_plan(l, M, 1, pl))
-        return 0;
+        return use_batch(l, M) ? batch_workspace_bytes(l, M) : 0;
     // sized for the worst split the planner may choose for this shape (one slab per wave and block)
     return kHeadBytes + (size_t)pl.NS * (size_t)M * (size_t)l->N * sizeof(float);
 }
@@ -1333,6 +1344,8 @@ size_t strip_workspace_bytes(const hqq_linear *l, int64_t M)
 int launch_strip_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
                         const SmallBatchEpilogue &ep, hipStream_t s, const StripIndex *ix)
 {
+    if (use_batch(l, M))
+        return launch_batch_matmul(l, x, M, y, ws, ws_bytes, ep, s, ix);
     StripJob j = {};
     j.shape[0] = l, j.NG = 1, j.NL = 1, j.EPI = 0, j.ix = ix, j.first_lstride = 1;
     j.x = x, j.y[0] = y, j.row_scale = ep.row_scale, j.accumulate = ep.accumulate;
@@ -1346,6 +1359,8 @@ void strip_fill_record(void *dst, const hqq_linear *l) { fill_layer(*static_cast
 int launch_strip_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
                          size_t ws_bytes, hipStream_t s, const StripIndex *ix)
 {
+    if (M >= 3 && !tuning_flag("HQQ_BATCH_OFF") && batch_gate_supported(w1, w3, M))
+        return launch_batch_gate_up(w1, w3, x, M, h, ws, ws_bytes, s, ix);
     StripJob j = {};
     j.shape[0] = w1, j.shape[1] = w3, j.NG = 1, j.NL = 2, j.EPI = 1, j.ix = ix, j.first_lstride = 1;
     j.x = x, j.y[0] = h;

@@ -151,6 +151,15 @@ struct StripIndex {
     const int *sel;
     int stride, first;
 };
+bool strip_gate_supported(const hqq_linear *w1, const hqq_linear *w3, int64_t M); // the fused w1/w3 launch
+// decode batches of 3 to 16 rows (gemv_batch.hip): reached through the strip entry points
+bool batch_supported(const hqq_linear *l, int64_t M);
+bool batch_gate_supported(const hqq_linear *w1, const hqq_linear *w3, int64_t M);
+size_t batch_workspace_bytes(const hqq_linear *l, int64_t M);
+int launch_batch_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
+                        const SmallBatchEpilogue &ep, hipStream_t s, const StripIndex *ix = nullptr);
+int launch_batch_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
+                         size_t ws_bytes, hipStream_t s, const StripIndex *ix = nullptr);
 size_t strip_record_bytes();
 void strip_fill_record(void *dst, const hqq_linear *l);
 int launch_strip_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,

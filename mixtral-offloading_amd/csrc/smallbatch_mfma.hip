@@ -539,7 +539,7 @@ int launch_smallbatch_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *
 int launch_smallbatch_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,
                               size_t ws_bytes, hipStream_t s)
 {
-    if (strip_supported(w1, M) && strip_supported(w3, M))
+    if (strip_gate_supported(w1, w3, M))
         return launch_strip_gate_up(w1, w3, x, M, h, ws, ws_bytes, s);
     SBPlan pl, pl3;
     if (!make_plan(w1, M, pl) || !make_plan(w3, M, pl3) || w1->N != w3->N || w1->K != w3->K ||
