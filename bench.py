@@ -445,15 +445,19 @@ def decode_section(dev, tokens_resident=256, tokens_offload=256):
                 "tokens": tokens_offload, "hits": st["hits"] - before["hits"], "misses": st["misses"] - before["misses"],
                 "GB_copied_host_to_device": round((st["bytes_copied"] - before["bytes_copied"]) / 1e9, 2)}
             # the same with speculative loads: the next layer's router applied one layer early picks what to prefetch
+            # (a guess is only acted on while the host link is idle and never evicts the latest request's experts
+            # before guesses have proved the better bet: with this random router the link is busy all the time)
             model.speculate = True
             before = model.expert_cache.stats()
-            spec_tokens = 64
-            out[f"expert_cache_{per_layer}_per_layer_speculative_tok_s"] = round(timed_eager(model, spec_tokens), 2)
+            out[f"expert_cache_{per_layer}_per_layer_speculative_tok_s"] = round(timed_eager(model, tokens_offload), 2)
             st = model.expert_cache.stats()
             loads = st["prefetch_loads"] - before["prefetch_loads"]
             out[f"expert_cache_{per_layer}_per_layer_speculative_detail"] = {
-                "tokens": spec_tokens, "prefetch_loads": loads,
-                "guess_accuracy": round((st["prefetch_useful"] - before["prefetch_useful"]) / max(1, loads), 3),
+                "tokens": tokens_offload, "prefetch_loads": loads,
+                "guesses_dropped_link_busy": st["prefetch_skipped_busy"] - before["prefetch_skipped_busy"],
+                "guesses_dropped_protected": st["prefetch_skipped_protected"] - before["prefetch_skipped_protected"],
+                "guess_accuracy": round((st["guess_right"] - before["guess_right"]) / max(1, st["guess_scored"] - before["guess_scored"]), 3),
+                "repeat_rate": round((st["reuse_right"] - before["reuse_right"]) / max(1, st["reuse_scored"] - before["reuse_scored"]), 3),
                 "misses": st["misses"] - before["misses"],
                 "GB_copied_host_to_device": round((st["bytes_copied"] - before["bytes_copied"]) / 1e9, 2)}
             model.speculate = False

@@ -324,6 +324,14 @@ int hqq_lru_add_resident(hqq_lru *c, int32_t e);
  * order): order[i] = expert, slot[i] = device slot it will occupy, victim[i] = expert evicted to make room or -1 for a
  * hit.  Returns 0 or HQQ_E_CACHE (unknown expert, duplicates, more misses than slots).                               */
 int hqq_lru_plan(hqq_lru *c, const int32_t *experts, int32_t n, int32_t *order, int32_t *slot, int32_t *victim);
+/* Plan a speculative load (no counterpart in the reference, whose README.md:24-26 lists speculative loading as not
+ * yet available): of the `n` distinct guessed experts, those that are resident are left alone (their place in the
+ * eviction order does not change); each of the others takes the place of the least recently used resident that is
+ * not one of the `n_keep` experts in `keep` (the experts a guess must not evict), or is dropped when there is none.
+ * Hits and misses are not counted.  Outputs for the *count experts that are to be loaded, in request order: order[i]
+ * = expert, slot[i] = device slot, victim[i] = the expert evicted.  Returns 0 or HQQ_E_CACHE / HQQ_E_NULL.          */
+int hqq_lru_plan_guess(hqq_lru *c, const int32_t *experts, int32_t n, const int32_t *keep, int32_t n_keep,
+                       int32_t *order, int32_t *slot, int32_t *victim, int32_t *count);
 int64_t hqq_lru_hits(const hqq_lru *c);
 int64_t hqq_lru_misses(const hqq_lru *c);
 /* device slot of expert e, or -1 when it is not resident */

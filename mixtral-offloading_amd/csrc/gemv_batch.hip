@@ -69,12 +69,13 @@ __device__ __forceinline__ u32x4 to_b_order(u32x4 v)
     return o;
 }
 
-constexpr int kBatchWaves = 8;
-
 // EPI: 0 y = o (+ bias) (* row_scale) (+ y);  1 y = silu(o0) * o1 (two layers)
-template <int NBITS, int PH, int MS, int SKIND, int ZKIND, int EPI>
-__global__ __launch_bounds__(kBatchWaves * 64) void gemv_batch_kernel(BatchParams p)
+// WAVES: 16 for up to eight batch rows (the kernel then stays within the 128 registers that four waves to a SIMD
+// leave each), so that a block's whole share of K is requested at once; 8 for sixteen rows
+template <int NBITS, int PH, int MS, int SKIND, int ZKIND, int EPI, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemv_batch_kernel(BatchParams p)
 {
+    constexpr int kBatchWaves = WAVES;
     constexpr int F = 8 / NBITS;
     constexpr int LP = PH == 4 ? 2 : 1;
     constexpr int MB = 16 / PH;  // batch rows per set
@@ -413,7 +414,7 @@ __global__ __launch_bounds__(kBatchWaves * 64) void gemv_batch_kernel(BatchParam
 }
 
 struct BatchPlan {
-    int F, GP, RB, NS, PH, MS, KS, SPW, BK, SKIND, ZKIND;
+    int F, GP, RB, NS, PH, MS, WAVES, KS, SPW, BK, SKIND, ZKIND;
 };
 
 bool make_batch_plan(const hqq_linear *l, int64_t M, int NL, BatchPlan &pl)
@@ -442,12 +443,16 @@ bool make_batch_plan(const hqq_linear *l, int64_t M, int NL, BatchPlan &pl)
         return false;
     pl.PH = M <= 4 ? 4 : 2;
     pl.MS = M <= 8 ? 1 : 2;
-    pl.KS = kBatchWaves / NL;
     const int64_t tiles = (int64_t)pl.GP * pl.RB;
-    // K over as many blocks as it takes to cover the chip about once, a block holding at least one slab per wave
+    // K over as many blocks as it takes to cover the chip about once, a block holding at least a slab per wave of eight
     int BK = 1;
-    while (tiles * BK < 200 && (pl.NS + BK) / (BK + 1) >= pl.KS && BK < 8)
+    while (tiles * BK < 200 && (pl.NS + BK) / (BK + 1) >= 8 / NL && BK < 8)
         ++BK;
+    // Sixteen waves where they were measured ahead of eight: five to eight rows in blocks that hold all of K (the gate
+    // 17.7 -> 15.6 us, 14336x4096 10.2 -> 9.3 us; with K over four blocks the down projection loses, 10.8 -> 13.3 us,
+    // and so do batches of up to four rows)
+    pl.WAVES = pl.MS == 1 && pl.PH == 2 && BK == 1 ? tuning_int("HQQ_BATCH_WAVES", 16) : 8;
+    pl.KS = pl.WAVES / NL;
     if (NL == 2 && BK > 1)
         return false; // the gate's epilogue needs both projections whole
     pl.BK = BK;
@@ -458,23 +463,23 @@ bool make_batch_plan(const hqq_linear *l, int64_t M, int NL, BatchPlan &pl)
     return true;
 }
 
-template <int NBITS, int PH, int MS, int EPI>
+template <int NBITS, int PH, int MS, int EPI, int WAVES>
 void launch_batch_kinds(const BatchParams &p, const BatchPlan &pl, dim3 grid, hipStream_t s)
 {
     if (pl.SKIND == TK_F16)
-        gemv_batch_kernel<NBITS, PH, MS, TK_F16, TK_F16, EPI><<<grid, dim3(kBatchWaves * 64), 0, s>>>(p);
+        gemv_batch_kernel<NBITS, PH, MS, TK_F16, TK_F16, EPI, WAVES><<<grid, dim3(WAVES * 64), 0, s>>>(p);
     else
-        gemv_batch_kernel<NBITS, PH, MS, TK_U8_COLS, TK_U8_SCALAR, EPI><<<grid, dim3(kBatchWaves * 64), 0, s>>>(p);
+        gemv_batch_kernel<NBITS, PH, MS, TK_U8_COLS, TK_U8_SCALAR, EPI, WAVES><<<grid, dim3(WAVES * 64), 0, s>>>(p);
 }
 
 template <int NBITS, int EPI> void launch_batch_shape(const BatchParams &p, const BatchPlan &pl, dim3 grid, hipStream_t s)
 {
-    if (pl.PH == 4)
-        launch_batch_kinds<NBITS, 4, 1, EPI>(p, pl, grid, s);
-    else if (pl.MS == 1)
-        launch_batch_kinds<NBITS, 2, 1, EPI>(p, pl, grid, s);
+    if (pl.MS == 2)
+        launch_batch_kinds<NBITS, 2, 2, EPI, 8>(p, pl, grid, s);
+    else if (pl.PH == 4)
+        launch_batch_kinds<NBITS, 4, 1, EPI, 8>(p, pl, grid, s);
     else
-        launch_batch_kinds<NBITS, 2, 2, EPI>(p, pl, grid, s);
+        pl.WAVES == 16 ? launch_batch_kinds<NBITS, 2, 1, EPI, 16>(p, pl, grid, s) : launch_batch_kinds<NBITS, 2, 1, EPI, 8>(p, pl, grid, s);
 }
 
 int run_batch(const hqq_linear *l0, const hqq_linear *l1, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,

@@ -132,6 +132,53 @@ int hqq_lru_plan(hqq_lru *c, const int32_t *experts, int32_t n, int32_t *order, 
     return HQQ_OK;
 }
 
+int hqq_lru_plan_guess(hqq_lru *c, const int32_t *experts, int32_t n, const int32_t *keep, int32_t n_keep,
+                       int32_t *order, int32_t *slot, int32_t *victim, int32_t *count)
+{
+    if (!c || !experts || !order || !slot || !victim || !count || (n_keep > 0 && !keep))
+        return HQQ_E_NULL;
+    if (n < 0 || n_keep < 0)
+        return HQQ_E_CACHE;
+    for (int32_t i = 0; i < n; ++i) {
+        if (experts[i] < 0 || experts[i] >= c->n_experts)
+            return HQQ_E_CACHE;
+        for (int32_t k = 0; k < i; ++k)
+            if (experts[k] == experts[i])
+                return HQQ_E_CACHE; // duplicates
+    }
+    auto kept = [&](int32_t e) {
+        for (int32_t k = 0; k < n_keep; ++k)
+            if (keep[k] == e)
+                return true;
+        for (int32_t k = 0; k < n; ++k) // a guess does not evict another expert of the same guess either
+            if (experts[k] == e)
+                return true;
+        return false;
+    };
+    int32_t w = 0;
+    for (int32_t i = 0; i < n; ++i) {
+        const int32_t e = experts[i];
+        if (c->slot_of[e] >= 0)
+            continue;
+        auto it = c->order.begin(); // least recently used first
+        while (it != c->order.end() && kept(*it))
+            ++it;
+        if (it == c->order.end())
+            continue; // nothing it may evict: the guess is dropped
+        const int32_t v = *it;
+        c->order.erase(it);
+        const int32_t s = c->slot_of[v];
+        c->slot_of[v] = -1;
+        c->slot_of[e] = s;
+        c->expert_in[s] = e;
+        c->pos[e] = c->order.insert(c->order.end(), e);
+        order[w] = e, slot[w] = s, victim[w] = v;
+        ++w;
+    }
+    *count = w;
+    return HQQ_OK;
+}
+
 int64_t hqq_lru_hits(const hqq_lru *c) { return c ? c->hits : 0; }
 int64_t hqq_lru_misses(const hqq_lru *c) { return c ? c->misses : 0; }
 int hqq_lru_slot_of(const hqq_lru *c, int32_t e)

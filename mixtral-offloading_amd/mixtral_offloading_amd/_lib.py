@@ -100,6 +100,8 @@ _SIGNATURES = {
     "hqq_lru_destroy": (None, [c_void_p]),
     "hqq_lru_add_resident": (c_int, [c_void_p, c_int32]),
     "hqq_lru_plan": (c_int, [c_void_p, _P(c_int32), c_int32, _P(c_int32), _P(c_int32), _P(c_int32)]),
+    "hqq_lru_plan_guess": (c_int, [c_void_p, _P(c_int32), c_int32, _P(c_int32), c_int32, _P(c_int32), _P(c_int32), _P(c_int32),
+                                   _P(c_int32)]),
     "hqq_lru_hits": (c_int64, [c_void_p]),
     "hqq_lru_misses": (c_int64, [c_void_p]),
     "hqq_lru_slot_of": (c_int, [c_void_p, c_int32]),

@@ -59,9 +59,8 @@ class EvictionGroup:
         self.members: List[ExpertInfo] = []
         self.global_slot: List[int] = []  # local slot -> global device slot
         self.evictable = False  # true once an expert of the group is offloaded: residents can then be evicted
-        # requests made by speculative prefetches, kept apart so that hits / misses count real requests only
-        self.spec_hits = 0
-        self.spec_misses = 0
+        self.last_request: set = set()  # the experts of the group's latest real request
+        self.last_guess: set = set()    # the experts of the latest guess, until the next real request scores it
 
     def __del__(self):
         if getattr(self, "_lru", None):
@@ -70,11 +69,11 @@ class EvictionGroup:
 
     @property
     def hits(self) -> int:
-        return _lib.lib.hqq_lru_hits(self._lru) - self.spec_hits
+        return _lib.lib.hqq_lru_hits(self._lru)
 
     @property
     def misses(self) -> int:
-        return _lib.lib.hqq_lru_misses(self._lru) - self.spec_misses
+        return _lib.lib.hqq_lru_misses(self._lru)
 
     def slot_of(self, index: int) -> int:
         return _lib.lib.hqq_lru_slot_of(self._lru, index)
@@ -94,6 +93,19 @@ class EvictionGroup:
         if rc != 0:
             raise ValueError("No evictable experts" if not self.global_slot else "invalid expert request")
         return list(order), list(slot), list(victim)
+
+    def plan_guess(self, indices: List[int], keep: List[int]):
+        """The policy's part of a speculative load: which of the guessed experts are loaded, where, and whom they evict
+        (never an expert of `keep`); resident experts are left alone and nothing is counted."""
+        n, nk = len(indices), len(keep)
+        arr, kp = (ctypes.c_int32 * n)(*indices), (ctypes.c_int32 * max(nk, 1))(*keep)
+        order, slot, victim = (ctypes.c_int32 * n)(), (ctypes.c_int32 * n)(), (ctypes.c_int32 * n)()
+        count = ctypes.c_int32(0)
+        rc = _lib.lib.hqq_lru_plan_guess(self._lru, arr, n, kp, nk, order, slot, victim, ctypes.byref(count))
+        if rc != 0:
+            raise ValueError("invalid expert request")
+        k = count.value
+        return list(order[:k]), list(slot[:k]), list(victim[:k])
 
 
 class ExpertCache:
@@ -120,6 +132,19 @@ class ExpertCache:
         self._speculative = set()
         self.prefetch_loads = 0   # copies started on a guess
         self.prefetch_useful = 0  # of those, experts that a real request then found on the device
+        self.prefetch_skipped_busy = 0       # guesses dropped because the copy stream still had work (host link busy)
+        self.prefetch_skipped_protected = 0  # guesses dropped because only the latest request's experts could have made room
+        # how often a guessed expert is asked for next, and how often an expert of a request is asked for again by the
+        # next request of its group: every guess is scored, acted on or not
+        self.prefetch_backlog = 0  # unfinished copies a guess may queue behind (0: only on an idle link)
+        # Guesses are acted on only while the link is found busy in less than this share of the recent prefetch calls:
+        # when loads bound the step (measured: busy at 80 - 96 % of the calls with a random router), tokens per second
+        # go with the bytes copied and every wrong guess costs its slab, even one started on a momentarily idle link.
+        self.prefetch_busy_limit = 0.25
+        self._busy_share = 1.0  # running mean of "the link had unfinished copies" over prefetch calls
+        self._inflight: set = set()  # slots whose copy may still be running
+        self.guess_scored = self.guess_right = 0
+        self.reuse_scored = self.reuse_right = 0
         self.copy_trace = None    # a list: (uid, start event, end event, kind) of every copy, for tests that look at overlap
         self._copy_kind = "demand"
 
@@ -133,6 +158,11 @@ class ExpertCache:
     def _compute_stream(self):
         return torch.cuda.current_stream(self.device)
 
+    def _link_backlog(self) -> int:
+        """Copies given to the copy stream that have not finished yet (host-side event queries, no synchronisation)."""
+        self._inflight = {slot for slot in self._inflight if not self.ready[slot].query()}
+        return len(self._inflight)
+
     def _alloc_host(self, nbytes: int) -> torch.Tensor:
         return torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
 
@@ -145,6 +175,7 @@ class ExpertCache:
             _lib.check(_lib.lib.hqq_slab_h2d_async(dst.data_ptr(), info.host_slab.data_ptr(), self.module_size,
                                                    self.copy_stream.cuda_stream, None), "hqq_slab_h2d_async")
             self.ready[slot].record(self.copy_stream)
+            self._inflight.add(slot)
             if self.copy_trace is not None:
                 t1.record(self.copy_stream)
                 self.copy_trace.append((info.uid, t0, t1, self._copy_kind))
@@ -234,6 +265,15 @@ class ExpertCache:
         assert len(set(info.eviction_group for info in infos)) == 1, "experts must be in the same evicton group"
         group = self.group_infos[infos[0].eviction_group]
         order, local_slots, victims = group.plan([info.index for info in infos])
+        request = {info.index for info in infos}
+        if group.last_guess:
+            self.guess_scored += len(group.last_guess)
+            self.guess_right += len(group.last_guess & request)
+            group.last_guess = set()
+        if group.last_request:
+            self.reuse_scored += len(group.last_request)
+            self.reuse_right += len(group.last_request & request)
+        group.last_request = request
         compute = self._compute_stream()
         miss = {idx: victim >= 0 for idx, victim in zip(order, victims)}
         self._settle_speculation(group, order, victims, real=True)
@@ -338,20 +378,41 @@ class ExpertCache:
 
     def prefetch(self, *uids: ExpertUID) -> int:
         """Start loading the given experts of one eviction group on a guess (the reference lists speculative loading
-        as not yet available, README.md:24-26).  It is a request like any other to the LRU policy -- the experts become
-        most recently used, misses evict the least recently used residents -- except that nothing is handed out and
-        hits / misses are not counted: the copies run on the side stream and whoever asks for the expert later finds
-        it on the device.  Returns the number of copies started."""
+        as not yet available, README.md:24-26).  Nothing is handed out and hits / misses are not counted: the copies
+        run on the side stream, a loaded guess becomes the group's most recently used expert, and whoever asks for it
+        later finds it on the device.  Returns the number of copies started.
+
+        Two rules keep a guess from costing a real request anything.  A guess is only acted on while the host link
+        is idle (every copy given to the copy stream has finished; `prefetch_backlog` allows that many unfinished
+        ones) and has mostly been idle at the recent calls (`prefetch_busy_limit`): on a saturated link an early copy
+        only displaces a needed one and every wrong guess adds a slab to the queue.  And a guess does not evict an expert of the group's latest real request (the ones the current token
+        may ask for again) unless guesses have proved the better bet: every guess is scored against the next real
+        request of its group, every request against the one before it, and the latest request's experts are
+        protected until at least eight of each have been scored and guessed experts are asked for more often than
+        repeated ones.  Guesses that only protected experts could make room for are dropped.  Guessed experts that
+        are resident already are left alone (no change of their place in the eviction order)."""
         assert not self.active, "already loading experts; buffers are busy"
         infos = [self.registered_experts[uid] for uid in dict.fromkeys(uids)]
         if not infos:
             return 0
         assert len(set(info.eviction_group for info in infos)) == 1, "experts must be in the same evicton group"
         group = self.group_infos[infos[0].eviction_group]
-        before = (_lib.lib.hqq_lru_hits(group._lru), _lib.lib.hqq_lru_misses(group._lru))
-        order, local_slots, victims = group.plan([info.index for info in infos])
-        group.spec_hits += _lib.lib.hqq_lru_hits(group._lru) - before[0]
-        group.spec_misses += _lib.lib.hqq_lru_misses(group._lru) - before[1]
+        group.last_guess = {info.index for info in infos}
+        absent = sum(1 for info in infos if group.slot_of(info.index) < 0)
+        if not absent:
+            return 0
+        backlog = self._link_backlog()
+        self._busy_share = 0.9 * self._busy_share + 0.1 * (1.0 if backlog > 0 else 0.0)
+        if backlog > self.prefetch_backlog or self._busy_share > self.prefetch_busy_limit:
+            self.prefetch_skipped_busy += absent
+            return 0
+        guesses_win = (self.guess_scored >= 8 and self.reuse_scored >= 8 and
+                       self.guess_right * self.reuse_scored > self.reuse_right * self.guess_scored)
+        order, local_slots, victims = group.plan_guess([info.index for info in infos],
+                                                       [] if guesses_win else sorted(group.last_request))
+        self.prefetch_skipped_protected += absent - len(order)
+        if not order:
+            return 0
         self._settle_speculation(group, order, victims, real=False)
         started = 0
         for idx, local, victim in zip(order, local_slots, victims):
@@ -396,4 +457,8 @@ class ExpertCache:
     def stats(self) -> Dict[str, int]:
         return {"hits": sum(g.hits for g in self.group_infos.values()),
                 "misses": sum(g.misses for g in self.group_infos.values()), "bytes_copied": self.bytes_copied,
-                "prefetch_loads": self.prefetch_loads, "prefetch_useful": self.prefetch_useful}
+                "prefetch_loads": self.prefetch_loads, "prefetch_useful": self.prefetch_useful,
+                "prefetch_skipped_busy": self.prefetch_skipped_busy,
+                "prefetch_skipped_protected": self.prefetch_skipped_protected,
+                "guess_scored": self.guess_scored, "guess_right": self.guess_right,
+                "reuse_scored": self.reuse_scored, "reuse_right": self.reuse_right}

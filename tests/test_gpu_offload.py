@@ -283,6 +283,9 @@ def test_speculative_prefetch_overlaps_attention_and_keeps_the_tokens():
         model.model.embed_tokens.weight.data.mul_(2000.0)  # hidden states of size 40 against layer outputs of size 1
         model.speculate = speculate
         cache = model.expert_cache
+        # (with two places per layer nearly every request misses, so the link is hardly ever idle: let guesses queue
+        # behind demand copies here, the overlap is what this test is about)
+        cache.prefetch_backlog, cache.prefetch_busy_limit = 8, 1.0
         cache.copy_trace, model.attention_trace = [], []
         base = torch.cuda.Event(enable_timing=True)
         base.record()

@@ -19,8 +19,13 @@ class _Module:
 
 
 class _Event:
+    busy = False  # what query() reports: the tests of speculative loads set it on the class
+
     def record(self, stream=None):
         pass
+
+    def query(self):
+        return not _Event.busy
 
 
 class _Stream:
@@ -44,6 +49,7 @@ class HostOnlyCache(ExpertCache):
 
     def _copy_in(self, info, slot):
         torch.as_tensor(self.slots[slot].storage, dtype=torch.uint8).copy_(info.host_slab)
+        self._inflight.add(slot)
 
 
 def _slab_of(e):
@@ -54,6 +60,7 @@ def _slab_of(e):
 
 def _cache(main, buffers, n=8):
     c = HostOnlyCache(_Module, main_size=main, offload_size=n - main, buffer_size=buffers)
+    c._busy_share = 0.0  # (the tests of speculative loads start from a link that has been idle)
     for e in range(n):  # the last `main` experts are resident, as build_model places them
         c.add_expert_storage((0, e), _slab_of(e), eviction_group=0, offload=e < n - main)
     return c
@@ -143,3 +150,85 @@ def test_host_copies_are_pinned_only_for_experts_that_can_be_evicted():
     assert all(c.registered_experts[(0, e)].host_slab is None for e in range(2))
     for (g, e), module in c.load_experts((1, 1), (1, 0), unordered=True):
         assert _content(module) == 10 + e
+
+
+def _resident(c):
+    g = c.group_infos[0]
+    return sorted(m.index for m in g.members if g.slot_of(m.index) >= 0)
+
+
+def test_a_guess_is_dropped_while_the_host_link_is_busy():
+    c = _cache(main=4, buffers=2)  # resident: 4 5 6 7
+    for _ in c.load_experts((0, 6), (0, 7), (0, 3)):  # 3 evicts 4; its copy stays "unfinished" below
+        pass
+    assert _resident(c) == [3, 5, 6, 7]
+    _Event.busy = True
+    try:
+        assert c.prefetch((0, 0), (0, 1)) == 0
+        assert _resident(c) == [3, 5, 6, 7] and c.stats()["prefetch_skipped_busy"] == 2 and c.stats()["prefetch_loads"] == 0
+        c.prefetch_backlog = 1  # a caller may let guesses queue behind that many unfinished copies
+        assert c.prefetch((0, 0)) == 1 and _resident(c) == [0, 3, 6, 7]  # 5 went: 3, 6 and 7 are the latest request's
+        c.prefetch_backlog = 0
+    finally:
+        _Event.busy = False
+    # 0 is resident; 1 finds nobody it may evict (3, 6, 7 are protected, 0 belongs to the same guess)
+    assert c.prefetch((0, 0), (0, 1)) == 0 and _resident(c) == [0, 3, 6, 7]
+    st = c.stats()
+    assert st["prefetch_loads"] == 1 and st["prefetch_skipped_protected"] == 1
+    assert st["hits"] == 2 and st["misses"] == 1  # guesses are not counted as requests
+
+
+def test_a_guess_does_not_evict_the_latest_requests_experts_until_guesses_have_proved_better():
+    """Two places, top-2 requests: every resident expert belongs to the latest request, so guesses are dropped; once
+    enough guesses have been scored and they are right more often than experts repeat, they may evict."""
+    c = _cache(main=2, buffers=2)
+    for _ in c.load_experts((0, 6), (0, 7)):
+        pass
+    assert c.prefetch((0, 0), (0, 1)) == 0 and _resident(c) == [6, 7]
+    assert c.stats()["prefetch_skipped_protected"] == 2
+    # guesses that are always right, requests that never repeat an expert
+    seq = [(0, 1), (2, 3), (4, 5), (6, 7), (0, 1), (2, 3)]
+    for a, b in seq:
+        for (_, e), module in c.load_experts((0, a), (0, b)):
+            assert _content(module) == e
+        nxt = seq[(seq.index((a, b)) + 1) % len(seq)]
+        c.prefetch((0, nxt[0]), (0, nxt[1]))
+    st = c.stats()
+    assert st["guess_right"] == st["guess_scored"] >= 8 and st["reuse_right"] == 0
+    assert st["prefetch_loads"] > 0  # by now guesses evict
+    loads = st["prefetch_loads"]
+    for (_, e), module in c.load_experts((0, 4), (0, 5)):
+        assert _content(module) == e
+    assert c.stats()["prefetch_useful"] >= 2 and c.stats()["prefetch_loads"] == loads
+
+
+def test_a_guess_of_resident_experts_changes_nothing():
+    c = _cache(main=4, buffers=2)
+    for _ in c.load_experts((0, 4), (0, 5)):
+        pass
+    assert c.prefetch((0, 6), (0, 7)) == 0  # resident already
+    # 6 and 7 are still the least recently used: two misses evict exactly them
+    for _ in c.load_experts((0, 0), (0, 1)):
+        pass
+    assert _resident(c) == [0, 1, 4, 5]
+
+
+def test_guesses_stop_when_the_link_has_mostly_been_busy():
+    """The share of prefetch calls that found unfinished copies is tracked; above the limit no guess is acted on, even
+    at a call that finds the link idle, and guesses resume once the link has been idle for a while."""
+    c = _cache(main=4, buffers=2)
+    for _ in c.load_experts((0, 6), (0, 7), (0, 3)):
+        pass
+    _Event.busy = True
+    try:
+        for _ in range(6):
+            assert c.prefetch((0, 0)) == 0
+    finally:
+        _Event.busy = False
+    assert c._busy_share > c.prefetch_busy_limit
+    assert c.prefetch((0, 0)) == 0  # idle now, but busy at most of the recent calls
+    calls = 1
+    while c.prefetch((0, 0)) == 0:
+        calls += 1
+        assert calls < 40
+    assert calls > 3 and 0 in _resident(c)
