@@ -720,6 +720,17 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
         return p.accumulate ? (f16)((f16)(prev + t0) + t1) : (f16)(t0 + t1);
     };
 
+#ifdef HQQ_TUNING_BUILD
+    auto write_stamps = [&]() __attribute__((always_inline)) {
+        if (p.stamps && lane == 0) {
+            unsigned long long *d = p.stamps + ((size_t)((bzi * gridDim.y + by) * gridDim.x + bx) * 16 + wave) * 16;
+            for (int i = 0; i < 14; ++i)
+                d[i] = st[i];
+            d[14] = __builtin_amdgcn_s_getreg((31 << 11) | 4);  // HW_ID: wave, SIMD, CU, shader array and engine
+            d[15] = __builtin_amdgcn_s_getreg((31 << 11) | 20); // XCC_ID
+        }
+    };
+#endif
     // ---------------------------------------------------------------- a block that holds all of K finishes its tile
     // A thread per (tile row, batch row) adds the waves' sums in wave order and applies the epilogue.
     if (alone) {
@@ -774,13 +785,7 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
         }
 #ifdef HQQ_TUNING_BUILD
         STRIP_STAMP(13);
-        if (p.stamps && lane == 0) {
-            unsigned long long *d = p.stamps + ((size_t)((bzi * gridDim.y + by) * gridDim.x + bx) * 16 + wave) * 16;
-            for (int i = 0; i < 14; ++i)
-                d[i] = st[i];
-            d[14] = __builtin_amdgcn_s_getreg((31 << 11) | 4);  // HW_ID: wave, SIMD, CU, shader array and engine
-            d[15] = __builtin_amdgcn_s_getreg((31 << 11) | 20); // XCC_ID
-        }
+        write_stamps();
 #endif
         if (chain == CHAIN_FIRST) {
             CHAIN_STAMP(p.chain, 2);
@@ -860,6 +865,10 @@ __device__ __forceinline__ void strip_block(const StripParams &p, const int bx, 
                 f16 *dst = y_rows + (int64_t)m_t * N + n;
                 *dst = p.accumulate ? (f16)(*dst + val) : val;
             }
+#ifdef HQQ_TUNING_BUILD
+            STRIP_STAMP(13);
+            write_stamps();
+#endif
             return;
         }
     }

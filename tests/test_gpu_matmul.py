@@ -330,3 +330,55 @@ def test_split_k_keeps_nan_and_infinity(nbits, n, k, gs):
     ref = x.float() @ w.t()
     assert bool(torch.isfinite(y).all())
     assert float((y.float() - ref).abs().max()) <= 1e-2 * float(ref.abs().max()) + 1e-3 * float(x.float().norm() * w.norm(dim=1).max())
+
+
+# the decode-batch kernel (batches of 3 to 16 rows of 2- and 4-bit layers whose K is a multiple of 256): every batch
+# size, one slab and several, K that does not divide evenly over the waves, K split over blocks (few tiles),
+# 8-bit and fp16 tables, several row blocks per table row
+BATCH_SHAPES = [
+    (2, 1024, 256, 16, 128, True, True),
+    (2, 3584, 768, 16, 128, True, True),
+    (2, 256, 3840, 16, 128, True, True),
+    (2, 512, 1024, 32, 128, False, False),
+    (4, 1024, 512, 64, 128, True, True),
+    (4, 256, 4096, 64, 128, True, True),
+    (4, 512, 768, 16, 128, False, False),
+]
+
+
+@pytest.mark.parametrize("shape", BATCH_SHAPES, ids=lambda s: "w%d_%dx%d_g%d_%s" % (s[:4] + ("q" if s[5] else "f16",)))
+def test_decode_batch_kernel_every_batch_size(shape):
+    from mixtral_offloading_amd import _lib
+    nbits, n, k, gs, mgs, qs, qz = shape
+    rng = np.random.default_rng(5 * n + k)
+    layer, _ = o.random_layer(rng, n, k, nbits, gs, qs, qz, meta_group_size=mgs)
+    assert _lib.lib.hqq_matmul_kernel_family(desc_of(layer).ref, 8) == _lib.FAM_SMALLBATCH
+    for m in range(3, 17):
+        x = rng.standard_normal((m, k)).astype(np.float16)
+        bias = rng.standard_normal(n).astype(np.float16) if m % 3 == 0 else None
+        for rep in range(2):  # accumulation slots are left clean
+            _check(layer, x, bias=bias)
+
+
+@pytest.mark.parametrize("m", [4, 8, 16])
+def test_decode_batch_kernel_keeps_nan_and_infinity(m):
+    """A NaN activation in one batch row reaches every output of that row and no other row; an overflowing row sum
+    comes out as +-inf (K of the 2-bit layer is split over blocks, the 4-bit one's is not)."""
+    from mixtral_offloading_amd import hip_kernels
+    for nbits, n, k, gs in ((2, 4096, 14336, 16), (4, 4096, 4096, 64)):
+        desc = _signed_layer(nbits, n, k, gs, seed=nbits + m)
+        w = hip_kernels.dequantize(desc).float()
+        G = n // gs
+        x = torch.randn((m, k), device="cuda").half()
+        x[1] = (torch.sign(w[0]) * 65504.0).half()
+        x[2, k // 2 + 3] = float("nan")
+        ref = x.float() @ w.t()
+        for rep in range(2):
+            y = hip_kernels.matmul(desc, x)
+            assert bool(torch.isposinf(y[1, 0])) and bool(torch.isneginf(y[1, G]))
+            assert bool(torch.isnan(y[2]).all())
+            rest = [r for r in range(m) if r not in (1, 2)]
+            assert bool(torch.isfinite(y[rest]).all())
+            err = (y[rest].float() - ref[rest]).abs()
+            bound = 1e-2 * ref[rest].abs() + 1e-3 * x[rest].float().norm(dim=1)[:, None] * w.norm(dim=1)[None, :]
+            assert bool((err <= bound).all())
