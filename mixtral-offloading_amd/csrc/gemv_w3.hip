@@ -7,15 +7,31 @@
 // kernels the scale is folded into the activations once per tile,
 //     y[10w+i, m] = sum_k q_i[w, k] * xs[i, k, m]  -  sum_k z[i, k] * xs[i, k, m],     xs = 32 * s[i, k] * x[m, k]  (fp16).
 //
-// A wave takes one slab of 256 columns of a tile at a time.  Lane (t = lane >> 2, c = lane & 3) owns word row t,
+// A wave takes one slab of 256 columns of a tile at a time.
+//
+// One batch row (the decode step): the codes go to the matrix cores.  A word's ten fields are five sets of two, one
+// field in each 16-bit half of an operand register: two sets are plain masks of the word, the other three masks of
+// two byte gathers that move the fields straddling a 16-bit boundary into the low ten bits of a half (seven vector
+// instructions per word instead of thirty).  A field masked in place is the fp16 subnormal q * 2^(offset - 24), which
+// v_mfma_f32_16x16x32_f16 multiplies exactly.  The sixteen tile rows of the instruction are eight word rows times two
+// column phases: lane (word row, phase, k group) reads 16 bytes at column 32 * step + 8 * group + 4 * phase, so the
+// two lanes of a word row read 32 consecutive bytes; the sixteen columns are phase x half x set, the B operand of a
+// column holding xs of its own field in its own half (zeros in the other) at the columns of its own phase, and the
+// result is kept where the phases agree.  The fifth set has a B operand of its own.  The table phase works in three
+// rounds, a lane owning sixteen columns of one table row (coalesced 16-byte table reads), and leaves xs in LDS in
+// the order the B lanes read it; the zero term is a dot product per table row (8-bit tables: of the raw bytes as
+// subnormals and of xs, the zero table's own scale and zero applied to the sums).  The codes of the slab's second
+// half are requested after the table phase, see there.
+//
+// Two batch rows: lane (t = lane >> 2, c = lane & 3) owns word row t,
 // columns 16m + 4c .. +3 for m = 0..15: four consecutive lanes read 64 consecutive bytes, sixteen 128-bit loads per
 // lane, all in flight at once.  A pair of words gives, per field, one v_perm (the two bytes that hold the field, of
 // both words) and one v_and: the field masked in place is the fp16 subnormal q * 2^(rel - 24), which v_dot2_f32_f16
 // multiplies exactly and accumulates in fp32.  The table phase (lane l owns columns 4l .. 4l+3 of all ten rows)
 // leaves xs in LDS; the zero term is a dot product per table row, summed over the wave at the end.
 //
-// The waves of a block split K (one or two slabs each; with two, the second slab's loads are in flight while the
-// first slab's codes are worked on); when K needs several blocks (or the window count alone would leave
+// The waves of a block split K (one or two slabs each; with two batch rows the second slab's loads are in flight
+// while the first slab's codes are worked on); when K needs several blocks (or the window count alone would leave
 // most of the chip idle) the blocks of a tile add their results into one 64-bit fixed-point accumulation slot per
 // output with a returning device-scope atomic, and the block whose addition completes a slot writes that output
 // (launches with more outputs than there are slots store fp32 partial sums instead, and the block that arrives
@@ -38,6 +54,10 @@ constexpr int kW3Waves = 8;
 constexpr int kW3S = 2; // most slabs per wave
 
 constexpr int kW3MaxLayers = 4;
+#ifndef HQQ_W3_EARLY
+#define HQQ_W3_EARLY 4
+#endif
+constexpr int kW3Early = HQQ_W3_EARLY; // single rows: 32-column steps of a slab whose codes are requested before the table phase
 
 struct W3Params {
     LayerRecord layer[kW3MaxLayers];
@@ -64,7 +84,19 @@ struct W3Params {
     int S;  // slabs per wave
     int SB; // slabs per block
     int BK; // blocks along K per tile
+    int meta4; // the scale table's meta columns are a multiple of 4 but not of 16
+#ifdef HQQ_TUNING_BUILD
+    int skip; // timing experiments: 1 leaves out the code phase, 2 the table phase (their loads are still waited for)
+    unsigned long long *stamps; // per-wave time stamps, [block][16 waves][16], or null
+#endif
 };
+#ifdef HQQ_TUNING_BUILD
+#define HQQ_W3_SKIP(p, bit) (((p).skip & (bit)) != 0)
+#define W3_STAMP(i) do { if (p.stamps) st[i] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define HQQ_W3_SKIP(p, bit) false
+#define W3_STAMP(i)
+#endif
 
 // field i of a word: bit offset 3*(9-i); the two bytes B, B+1 that hold it, its offset inside them
 __host__ __device__ constexpr int w3_bit(int i) { return 3 * (9 - i); }
@@ -76,6 +108,36 @@ __host__ __device__ constexpr uint32_t w3_sel(int i)
 }
 __host__ __device__ constexpr uint32_t w3_mask(int i) { return (7u << (w3_bit(i) & 7)) * 0x00010001u; }
 __host__ __device__ constexpr float w3_unscale(int i) { return (float)(1u << (24 - (w3_bit(i) & 7))) / kXsScale; }
+
+// One batch row: a word's ten fields go to the matrix cores as five sets of two, one field in each 16-bit half of an
+// operand register (so a register is one column, and the B operand keeps the halves apart with zeros).  Sets 0 and 1
+// are the word itself; the others are two byte gathers, which put the fields that straddle a 16-bit boundary into
+// the low ten bits of a half:
+//   set 0: field 9 (offset 0) | field 3 (offset 2)      the word, halves at bits 0 and 16
+//   set 1: field 8 (offset 3) | field 2 (offset 5)
+//   set 2: field 7 (offset 6) | field 4 (offset 7)      gather B: bytes (0,1) | (1,2)
+//   set 3: field 6 (offset 1) | field 1 (offset 0)      gather A: bytes (1,2) | (3,zero)
+//   set 4: field 5 (offset 4) | field 0 (offset 3)
+constexpr uint32_t kW3GatherA = 0x0c030201u, kW3GatherB = 0x02010100u;
+__host__ __device__ constexpr int w3_set_offset(int set, int half)
+{
+    return half ? (set == 0 ? 2 : set == 1 ? 5 : set == 2 ? 7 : set == 3 ? 0 : 3)
+                : (set == 0 ? 0 : set == 1 ? 3 : set == 2 ? 6 : set == 3 ? 1 : 4);
+}
+__host__ __device__ constexpr uint32_t w3_set_mask(int set)
+{
+    return (7u << w3_set_offset(set, 0)) | (7u << (16 + w3_set_offset(set, 1)));
+}
+__device__ __forceinline__ int w3_set_field(int set, int half)
+{
+    return half ? (0x01423 >> (4 * set)) & 15 : 9 - set;
+}
+// a field masked at offset o of a half is the fp16 subnormal q * 2^(o - 24)
+__device__ __forceinline__ float w3_set_unscale(int set, int half)
+{
+    const int o = half ? (0x30752 >> (4 * set)) & 15 : (0x41630 >> (4 * set)) & 15;
+    return __builtin_bit_cast(float, (uint32_t)(127 + 24 - 5 - o) << 23); // 2^(24 - o) / 32
+}
 
 __device__ __forceinline__ float quad_sum(float v)
 {
@@ -97,11 +159,27 @@ template <int MT, bool Q8, int XMODE, int S>
 __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
 {
     constexpr int NT = kW3Waves * 64;
-    // xs of the slab: [4-column group q][batch row][field][4 halves]
-    __shared__ __attribute__((aligned(16))) f16 xs_lds[kW3Waves][64][MT][10][4];
+#ifdef HQQ_TUNING_BUILD
+    unsigned long long st[16] = {};
+#endif
+    W3_STAMP(0);
+#ifdef HQQ_TUNING_BUILD
+    if (p.stamps)
+        st[9] = __builtin_readcyclecounter();
+#endif
+    // xs of each wave's slab.  Two batch rows: [4-column group][batch row][table row][4 halves]; one batch row:
+    // [16-column step][4-column piece][table row][4 halves]
+    __shared__ __attribute__((aligned(16))) f16 xs_raw[kW3Waves * 64 * MT * 10 * 4];
+    __shared__ __attribute__((aligned(16))) f16 h_lds[MT == 1 && XMODE ? kW3Waves : 1][kSlab]; // silu(xa) * xb of the slab
+    __shared__ float zt_lds[kW3Waves][10];
     __shared__ float red_lds[kW3Waves][16][10][MT];
     __shared__ int ticket_lds;
 
+    // Every kernel argument the prologue reads is fetched here, in one batch: read where they are used, they come in
+    // five or six scalar loads one after the other, each waiting for the branch before it.
+    asm volatile("" ::"s"(p.table), "s"(p.sel), "s"(p.stride), "s"(p.first), "s"(p.lper), "s"(p.x), "s"(p.xa), "s"(p.xb),
+                 "s"(p.x_lstride), "s"(p.P), "s"(p.G), "s"(p.K), "s"(p.NW), "s"(p.KS), "s"(p.SB), "s"(p.NS), "s"(p.pair),
+                 "s"(p.y), "s"(p.y_lstride), "s"(p.part), "s"(p.part_lstride));
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kb = blockIdx.x, rb = blockIdx.y;
@@ -121,28 +199,298 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
         __builtin_memcpy(&R, rec, sizeof(R));
     } else {
         R = p.layer[__builtin_amdgcn_readfirstlane(layer)];
+        asm volatile("" ::"s"(R.codes), "s"(R.sq), "s"(R.zq), "s"(R.s_ms), "s"(R.s_mz), "s"(R.z_ms), "s"(R.z_mz), "s"(R.s_cols),
+                     "s"(R.s_inv)); // the whole record in one batch as well
     }
     f16 *const yl = p.y + (int64_t)(p.pair ? 0 : layer) * p.y_lstride;
     float *const partl = p.part + (int64_t)layer * p.part_lstride;
     const int M = MT == 1 ? 1 : p.M;
     const int K = p.K;
+    const uint32_t j0 = (uint32_t)(10 * w0) % (uint32_t)p.G;
+
+    const int slab_lo = kb * p.SB + wave * S;
+    int slab_hi = (kb + 1) * p.SB;
+    if (slab_hi > p.NS)
+        slab_hi = p.NS;
+    auto wave_sync = [&]() __attribute__((always_inline)) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+
+    if constexpr (MT == 1) {
+        // ------------------------------------------------------------ one batch row: the codes on the matrix cores
+        constexpr int SK = Q8 ? TK_U8_COLS : TK_F16, ZK = Q8 ? TK_U8_SCALAR : TK_F16;
+        f16 *const xs_w = xs_raw + wave * (16 * 4 * 10 * 4); // [step][piece][table row][4 halves]
+        // code role: tile row lane & 15 = 2 * (word row within its group of eight) + phase, k group lane >> 4; the
+        // tile's sixteen word rows are two such groups
+        const int rho = (lane & 15) >> 1, phi = lane & 1, gk = lane >> 4;
+        uint32_t code_at[2];
+#pragma unroll
+        for (int g8 = 0; g8 < 2; ++g8) {
+            const int wr = w0 + p.P * (16 * rb + 8 * g8 + rho);
+            code_at[g8] = (uint32_t)(wr < p.NW ? wr : w0) * (uint32_t)K * 4u + (uint32_t)(32 * gk + 16 * phi);
+        }
+        // column role: column lane & 15 = phase + 2 * half + 4 * set for the sets 0..3; the fifth set has a B operand
+        // of its own, of which the columns 0..3 are kept
+        const int set = (lane & 15) >> 2, half = (lane >> 1) & 1;
+        const int fcol = w3_set_field(set, half), fcol4 = w3_set_field(4, half);
+        const uint32_t b_at = (uint32_t)(((2 * gk + phi) * 10 + fcol) * 8), b4_at = (uint32_t)(((2 * gk + phi) * 10 + fcol4) * 8);
+        const uint32_t sel_a = half ? 0x01000c0cu : 0x0c0c0100u, sel_b = half ? 0x03020c0cu : 0x0c0c0302u;
+        // table role: round r, lane (row = lane >> 4, chunk = lane & 15); the third round has two rows only
+        const int qT = lane & 15;
+        const bool third_ok = lane < 32;
+        uint32_t trow_at[3];
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            const int f = r < 2 ? 4 * r + (lane >> 4) : 8 + ((lane >> 4) & 1);
+            uint32_t j = j0 + (uint32_t)f; // (10*w0 + f) mod G; G >= 10
+            j -= j >= (uint32_t)p.G ? (uint32_t)p.G : 0u;
+            trow_at[r] = j * (uint32_t)K + (uint32_t)(16 * qT);
+        }
+
+        f32x4 acc[2][5];
+#pragma unroll
+        for (int g8 = 0; g8 < 2; ++g8)
+#pragma unroll
+            for (int i = 0; i < 5; ++i)
+                acc[g8][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        if (lane < 10)
+            zt_lds[wave][lane] = 0.f;
+        // the masks in scalar registers: as literals they double the size of the instructions that use them
+        uint32_t mk[5] = {w3_set_mask(0), w3_set_mask(1), w3_set_mask(2), w3_set_mask(3), w3_set_mask(4)};
+        asm volatile("" : "+s"(mk[0]), "+s"(mk[1]), "+s"(mk[2]), "+s"(mk[3]), "+s"(mk[4]));
+
+        if (wave < p.KS) {
+            for (int slab = slab_lo; slab < slab_lo + S && slab < slab_hi; ++slab) {
+                const uint32_t k0 = (uint32_t)slab * kSlab;
+                W3_STAMP(1);
+                // every load of the slab, in the order the arithmetic needs them.  The whole-tensor meta of the zero
+                // table has the same address in every lane, written so that the compiler does not see it (lane >> 6
+                // is zero): a load it knows to be uniform moves to scalar registers and is waited for at once.
+                uint32_t zms_raw = 0, zmz_raw = 0;
+                // the zero term of the lane's table row and columns: fp16 tables sum z * xs; 8-bit tables sum zq * xs
+                // (the bytes as fp16 subnormals, zq * 2^-24) and xs, and z = (zq - mz) * ms is applied to the sums
+                float zacc[3] = {0.f, 0.f, 0.f}, zxs[3] = {0.f, 0.f, 0.f};
+                if constexpr (Q8) {
+                    zms_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_ms) + (lane >> 6));
+                    zmz_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_mz) + (lane >> 6));
+                }
+                Raw16<SK> rs[3];
+                Raw16<ZK> rz[3];
+#pragma unroll
+                for (int r = 0; r < 3; ++r) {
+                    const uint32_t ce = trow_at[r] + k0;
+                    uint32_t cm = 0;
+                    if constexpr (Q8) {
+                        cm = ce - __umulhi(ce, R.s_inv) * R.s_cols; // ce mod cols; the quotient estimate is at most 2 short
+                        cm -= cm >= R.s_cols ? R.s_cols : 0;
+                        cm -= cm >= R.s_cols ? R.s_cols : 0;
+                    }
+                    if (Q8 && p.meta4) {
+                        // the meta columns are a multiple of 4 only: the lane's sixteen entries may wrap inside, four
+                        // pieces each with its own column
+                        rs[r].q = gload<u32x4>(R.sq + ce);
+#pragma unroll
+                        for (int pc = 0; pc < 4; ++pc) {
+                            uint32_t c4 = cm + 4u * pc;
+                            c4 -= c4 >= R.s_cols ? R.s_cols : 0;
+                            const u32x2 a = gload<u32x2>(R.s_ms + c4), b = gload<u32x2>(R.s_mz + c4);
+                            rs[r].ms[pc >> 1][2 * (pc & 1)] = a.x, rs[r].ms[pc >> 1][2 * (pc & 1) + 1] = a.y;
+                            rs[r].mz[pc >> 1][2 * (pc & 1)] = b.x, rs[r].mz[pc >> 1][2 * (pc & 1) + 1] = b.y;
+                        }
+                    } else {
+                        load16<SK>(rs[r], R.sq, R.s_ms, R.s_mz, ce, cm);
+                    }
+                    load16<ZK>(rz[r], R.zq, nullptr, nullptr, ce, 0);
+                }
+                u32x4 xr[2];
+                u32x2 xg = {0, 0}, xh = {0, 0};
+                if constexpr (XMODE) {
+                    xg = gload<u32x2>(p.xa + (int64_t)layer * p.x_lstride + k0 + (uint32_t)(4 * lane));
+                    xh = gload<u32x2>(p.xb + (int64_t)layer * p.x_lstride + k0 + (uint32_t)(4 * lane));
+                } else {
+                    xr[0] = gload<u32x4>(p.x + k0 + (uint32_t)(16 * qT));
+                    xr[1] = gload<u32x4>(p.x + k0 + (uint32_t)(16 * qT + 8));
+                }
+                // A step is 32 columns: four words of both row groups.  The codes of the slab's second half are requested
+                // after the table phase: a wave that has issued its loads waits there, which lets the other wave of the
+                // SIMD issue its own (the older wave is served first), so that both have the first half of their data
+                // early and neither is left with a whole slab of arithmetic after the last byte has arrived.
+                u32x4 cw[8][2];
+#pragma unroll
+                for (int s = 0; s < kW3Early; ++s)
+#pragma unroll
+                    for (int g8 = 0; g8 < 2; ++g8)
+                        cw[s][g8] = gload<u32x4>(R.codes + (code_at[g8] + 4u * k0 + (uint32_t)(128 * s)));
+                __builtin_amdgcn_sched_barrier(0); // nothing below moves above the loads, no load sinks into the arithmetic
+                W3_STAMP(2);
+
+                // table phase: xs = 32 * s * x of the ten table rows into LDS, the zero term accumulated
+                if constexpr (Q8) // the meta values become opaque here, so no use of them is hoisted above the loads
+                    asm volatile("" : "+v"(zms_raw), "+v"(zmz_raw));
+                if constexpr (XMODE) {
+                    const f16x2 a01 = as_h2(xg.x), a23 = as_h2(xg.y), b01 = as_h2(xh.x), b23 = as_h2(xh.y);
+                    u32x2 hv;
+                    hv.x = as_u32((f16x2){silu_mul(a01.x, b01.x), silu_mul(a01.y, b01.y)});
+                    hv.y = as_u32((f16x2){silu_mul(a23.x, b23.x), silu_mul(a23.y, b23.y)});
+                    *reinterpret_cast<u32x2 *>(&h_lds[wave][4 * lane]) = hv;
+                    wave_sync();
+                    xr[0] = *reinterpret_cast<const u32x4 *>(&h_lds[wave][16 * qT]);
+                    xr[1] = *reinterpret_cast<const u32x4 *>(&h_lds[wave][16 * qT + 8]);
+                }
+                const f16x2 k32 = {(f16)kXsScale, (f16)kXsScale};
+                const f16x2 ones = {(f16)1.0f, (f16)1.0f};
+#pragma unroll
+                for (int r = 0; r < 3; ++r) {
+                    if (HQQ_W3_SKIP(p, 2)) {
+                        asm volatile("" ::"v"(rs[r].q), "v"(rs[r].q_hi), "v"(rs[r].ms[0]), "v"(rs[r].ms[1]), "v"(rs[r].mz[0]),
+                                     "v"(rs[r].mz[1]), "v"(rz[r].q), "v"(rz[r].q_hi), "v"(xr[0]), "v"(xr[1]));
+                        continue;
+                    }
+                    const int f = r < 2 ? 4 * r + (lane >> 4) : 8 + ((lane >> 4) & 1);
+                    f16x2 sv[8], zv[8];
+                    decode16<SK>(rs[r], k32, k32, sv);
+                    if constexpr (!Q8)
+                        decode16<ZK>(rz[r], k32, k32, zv);
+                    uint32_t a[8];
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) {
+                        const f16x2 v = (sv[t] * k32) * as_h2(xr[t >> 2][t & 3]);
+                        if constexpr (Q8) {
+                            // bytes 2 * (t & 1), 2 * (t & 1) + 1 of the word into the low bytes of the two halves
+                            const uint32_t zq = __builtin_amdgcn_perm(0u, rz[r].q[t >> 1], (t & 1) ? 0x0c030c02u : 0x0c010c00u);
+                            zacc[r] = __builtin_amdgcn_fdot2(as_h2(zq), v, zacc[r], false);
+                            zxs[r] = __builtin_amdgcn_fdot2(ones, v, zxs[r], false);
+                        } else {
+                            zacc[r] = __builtin_amdgcn_fdot2(zv[t], v, zacc[r], false);
+                        }
+                        a[t] = as_u32(v);
+                    }
+                    if (r < 2 || third_ok) {
+#pragma unroll
+                        for (int pi = 0; pi < 4; ++pi)
+                            *reinterpret_cast<u32x2 *>(xs_w + ((qT * 4 + pi) * 10 + f) * 4) = (u32x2){a[2 * pi], a[2 * pi + 1]};
+                    }
+                }
+                // the zero terms of the slab: summed over the sixteen chunk lanes of a table row and added up in LDS,
+                // here rather than after the last code step, where every instruction delays the block's result
+#pragma unroll
+                for (int r = 0; r < 3; ++r) {
+                    const int f = r < 2 ? 4 * r + (lane >> 4) : 8 + ((lane >> 4) & 1);
+                    float z = zacc[r];
+                    if constexpr (Q8) {
+                        const float ms = (float)__builtin_bit_cast(f16, (uint16_t)zms_raw), mz = (float)__builtin_bit_cast(f16, (uint16_t)zmz_raw);
+                        z = ms * (z * 16777216.0f - mz * zxs[r]);
+                    }
+                    z = row16_sum(z);
+                    if (qT == 0 && (r < 2 || third_ok))
+                        zt_lds[wave][f] += z;
+                }
+                wave_sync();
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int s = kW3Early; s < 8; ++s)
+#pragma unroll
+                    for (int g8 = 0; g8 < 2; ++g8)
+                        cw[s][g8] = gload<u32x4>(R.codes + (code_at[g8] + 4u * k0 + (uint32_t)(128 * s)));
+                __builtin_amdgcn_sched_barrier(0);
+                W3_STAMP(3);
+
+                // code phase: per word two plain masks and two byte gathers with three masks.  The B operands of a step
+                // are read from LDS a step ahead.
+                auto read_b = [&](u32x2 &bx, u32x2 &by, int s) __attribute__((always_inline)) {
+                    bx = *reinterpret_cast<const u32x2 *>(reinterpret_cast<const char *>(xs_w) + b_at + s * 640);
+                    by = *reinterpret_cast<const u32x2 *>(reinterpret_cast<const char *>(xs_w) + b4_at + s * 640);
+                };
+                u32x2 bx, by;
+                read_b(bx, by, 0);
+#pragma unroll
+                for (int s = 0; s < 8; ++s) {
+                    const u32x4 bu = {__builtin_amdgcn_perm(0u, bx.x, sel_a), __builtin_amdgcn_perm(0u, bx.x, sel_b),
+                                      __builtin_amdgcn_perm(0u, bx.y, sel_a), __builtin_amdgcn_perm(0u, bx.y, sel_b)};
+                    const u32x4 bv = {__builtin_amdgcn_perm(0u, by.x, sel_a), __builtin_amdgcn_perm(0u, by.x, sel_b),
+                                      __builtin_amdgcn_perm(0u, by.y, sel_a), __builtin_amdgcn_perm(0u, by.y, sel_b)};
+                    const f16x8 B = __builtin_bit_cast(f16x8, bu), B4 = __builtin_bit_cast(f16x8, bv);
+                    if (s + 1 < 8)
+                        read_b(bx, by, s + 1);
+#ifdef HQQ_TUNING_BUILD
+                    if (s == 1 || s == 2 || s == 4 || s == 6) {
+                        asm volatile("" ::"v"(cw[s][0]));
+                        W3_STAMP(s == 1 ? 4 : s == 2 ? 5 : s == 4 ? 6 : 7);
+                    }
+#endif
+#pragma unroll
+                    for (int g8 = 0; g8 < 2; ++g8) {
+                        const u32x4 w = cw[s][g8];
+                        if (HQQ_W3_SKIP(p, 1)) {
+                            asm volatile("" ::"v"(w));
+                            continue;
+                        }
+                        u32x4 wa, wb;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            wa[j] = __builtin_amdgcn_perm(w[j], w[j], kW3GatherA);
+                            wb[j] = __builtin_amdgcn_perm(w[j], w[j], kW3GatherB);
+                        }
+                        acc[g8][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, w & mk[0]), B, acc[g8][0], 0, 0, 0);
+                        acc[g8][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, w & mk[1]), B, acc[g8][1], 0, 0, 0);
+                        acc[g8][2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, wb & mk[2]), B, acc[g8][2], 0, 0, 0);
+                        acc[g8][3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, wa & mk[3]), B, acc[g8][3], 0, 0, 0);
+                        acc[g8][4] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, wa & mk[4]), B4, acc[g8][4], 0, 0, 0);
+                    }
+                }
+                wave_sync();
+                W3_STAMP(8);
+            }
+        }
+
+        // wave result
+        wave_sync();
+        const float zt = zt_lds[wave][fcol] * (1.0f / kXsScale), zt4 = zt_lds[wave][fcol4] * (1.0f / kXsScale);
+        const float un = w3_set_unscale(set, half), un4 = w3_set_unscale(4, half);
+        // Accumulator element v of a lane is tile row 4 * (lane >> 4) + v = 2 * word row + phase; a column keeps the
+        // rows of its own phase, and the two phases of a word row are lanes one apart.
+        const uint32_t odd = phi ? ~0u : 0u;
+#pragma unroll
+        for (int g8 = 0; g8 < 2; ++g8) {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                // a bitwise select: written as a conditional the compiler turns it into an indexed read of the vector
+                auto pick = [&](const f32x4 &c) __attribute__((always_inline)) {
+                    return __builtin_bit_cast(float, (__builtin_bit_cast(uint32_t, (float)c[2 * e + 1]) & odd) |
+                                                         (__builtin_bit_cast(uint32_t, (float)c[2 * e]) & ~odd));
+                };
+                float v = pick(acc[g8][0]);
+#pragma unroll
+                for (int i = 1; i < 4; ++i) {
+                    const float c = pick(acc[g8][i]);
+                    v = set == i ? c : v;
+                }
+                float v4 = pick(acc[g8][4]);
+                v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+                v4 += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v4), 0xB1, 0xF, 0xF, true));
+                const int row = 8 * g8 + 2 * gk + e;
+                if (phi == 0) {
+                    red_lds[wave][row][fcol][0] = fmaf(v, un, -zt);
+                    if (set == 0)
+                        red_lds[wave][row][fcol4][0] = fmaf(v4, un4, -zt4);
+                }
+            }
+        }
+    } else {
+    // ---------------------------------------------------------------- two batch rows: dot products on the vector units
+    auto xs_lds = reinterpret_cast<f16(*)[64][MT][10][4]>(xs_raw);
     const int t = lane >> 2, c = lane & 3;
     const int wr = w0 + p.P * (16 * rb + t); // this lane's word row
     const bool row_ok = wr < p.NW;
-    const uint32_t j0 = (uint32_t)(10 * w0) % (uint32_t)p.G;
     const uint32_t code_base = (uint32_t)(row_ok ? wr : w0) * (uint32_t)K * 4u + (uint32_t)(16 * c);
-
     float acc[10][MT], zacc[10][MT];
 #pragma unroll
     for (int i = 0; i < 10; ++i)
 #pragma unroll
         for (int m = 0; m < MT; ++m)
             acc[i][m] = zacc[i][m] = 0.f;
-
-    const int slab_lo = kb * p.SB + wave * S;
-    int slab_hi = (kb + 1) * p.SB;
-    if (slab_hi > p.NS)
-        slab_hi = p.NS;
 
     // What a slab's table phase reads: tables, their per-column meta, the zero table's whole-tensor meta, x.
     struct Tab {
@@ -196,11 +544,6 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
 #pragma unroll
         for (int m = 0; m < 16; ++m)
             cw[m] = gload<u32x4>(R.codes + (code_base + 4u * ((uint32_t)slab * kSlab) + (uint32_t)(64 * m)));
-    };
-    auto wave_sync = [&]() __attribute__((always_inline)) {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     };
     // table phase: xs into LDS, zero term accumulated
     auto table_phase = [&](Tab &T) __attribute__((always_inline)) {
@@ -325,7 +668,26 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
                 red_lds[wave][t][i][m] = a - z;
         }
     }
+    }
+#ifdef HQQ_TUNING_BUILD
+    if (p.stamps)
+        st[10] = __builtin_readcyclecounter();
+#endif
+    W3_STAMP(11);
     __syncthreads();
+    W3_STAMP(12);
+#ifdef HQQ_TUNING_BUILD
+    auto write_stamps = [&]() __attribute__((always_inline)) {
+        if (p.stamps && lane == 0) {
+            st[13] = __builtin_amdgcn_s_memrealtime();
+            unsigned long long *d = p.stamps + ((size_t)((blockIdx.z * gridDim.y + rb) * gridDim.x + kb) * 16 + wave) * 16;
+            for (int i = 0; i < 14; ++i)
+                d[i] = st[i];
+            d[14] = __builtin_amdgcn_s_getreg((31 << 11) | 4);  // HW_ID
+            d[15] = __builtin_amdgcn_s_getreg((31 << 11) | 20); // XCC_ID
+        }
+    };
+#endif
 
     // ---------------------------------------------------------------- block result
     const bool alone = p.BK == 1;
@@ -365,6 +727,9 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
             __hip_atomic_store(partl + ((int64_t)kb * M + m_t) * p.N + n, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
+#ifdef HQQ_TUNING_BUILD
+    write_stamps();
+#endif
     if (alone || p.slots)
         return;
 
@@ -392,6 +757,10 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
         finish(m_t, n, v);
     }
 }
+
+#ifdef HQQ_TUNING_BUILD
+unsigned long long *g_w3_stamps = nullptr; // device buffer the launches write their waves' time stamps to
+#endif
 
 struct W3Plan {
     int G, P, NW, RB, NS, KS, S, SB, BK;
@@ -422,10 +791,11 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, W3Plan &pl)
     pl.q8 = sk == TK_U8_COLS && zk == TK_U8_SCALAR;
     if (!pl.q8 && !(sk == TK_F16 && zk == TK_F16))
         return false;
-    if (!aligned16(l->codes) || (reinterpret_cast<uintptr_t>(l->scale.data) & 7u) || (reinterpret_cast<uintptr_t>(l->zero.data) & 7u))
+    // a lane of the table phase reads sixteen consecutive entries of a table row and of its per-column meta
+    if (!aligned16(l->codes) || !aligned16(l->scale.data) || !aligned16(l->zero.data))
         return false;
-    if (pl.q8 && (l->scale.meta_cols % 4 != 0 || (reinterpret_cast<uintptr_t>(l->scale.meta_scale) & 7u) ||
-                  (reinterpret_cast<uintptr_t>(l->scale.meta_zero) & 7u)))
+    if (pl.q8 && (l->scale.meta_cols % 4 != 0 || l->scale.meta_cols < 16 || !aligned16(l->scale.meta_scale) ||
+                  !aligned16(l->scale.meta_zero)))
         return false;
     pl.G = (int)G;
     pl.P = (int)(G / gcd_int(10, (int)G));
@@ -515,7 +885,7 @@ int run_job(const W3Job &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
     if (pl.BK > 1 && (!ws || ws_bytes < job_workspace_bytes(pl, l, j.NL)))
         return HQQ_E_WORKSPACE;
     if (fused ? ((reinterpret_cast<uintptr_t>(j.xa) | reinterpret_cast<uintptr_t>(j.xb)) & 7u) != 0
-              : (reinterpret_cast<uintptr_t>(j.x) & 7u) != 0)
+              : (reinterpret_cast<uintptr_t>(j.x) & 15u) != 0)
         return HQQ_E_ALIGN;
     W3Params p = {};
     if (j.ix) {
@@ -539,6 +909,11 @@ int run_job(const W3Job &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
     p.part_lstride = (int64_t)pl.BK * 2 * l->N;
     p.y_lstride = j.y_lstride;
     p.accumulate = j.ep.accumulate;
+    p.meta4 = pl.q8 && l->scale.meta_cols % 16 != 0;
+#ifdef HQQ_TUNING_BUILD
+    p.skip = tuning_int("HQQ_W3_SKIP", 0);
+    p.stamps = g_w3_stamps;
+#endif
     p.N = (int)l->N, p.K = (int)l->K, p.G = pl.G, p.P = pl.P, p.NW = pl.NW, p.RB = pl.RB;
     p.NS = pl.NS, p.KS = pl.KS, p.S = pl.S, p.SB = pl.SB, p.BK = pl.BK;
     const dim3 grid((unsigned)pl.BK, (unsigned)pl.RB, (unsigned)(pl.P * j.NL));
@@ -665,3 +1040,7 @@ int launch_vec3_down_pair(const hqq_linear *w2, const f16 *ab, int64_t ab_lstrid
 }
 
 } // namespace hqq
+
+#ifdef HQQ_TUNING_BUILD
+extern "C" void hqq_tuning_w3_stamps(void *buf) { hqq::g_w3_stamps = static_cast<unsigned long long *>(buf); }
+#endif
