@@ -261,188 +261,219 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
         uint32_t mk[5] = {w3_set_mask(0), w3_set_mask(1), w3_set_mask(2), w3_set_mask(3), w3_set_mask(4)};
         asm volatile("" : "+s"(mk[0]), "+s"(mk[1]), "+s"(mk[2]), "+s"(mk[3]), "+s"(mk[4]));
 
-        if (wave < p.KS) {
-            for (int slab = slab_lo; slab < slab_lo + S && slab < slab_hi; ++slab) {
-                const uint32_t k0 = (uint32_t)slab * kSlab;
-                W3_STAMP(1);
-                // every load of the slab, in the order the arithmetic needs them.  The whole-tensor meta of the zero
-                // table has the same address in every lane, written so that the compiler does not see it (lane >> 6
-                // is zero): a load it knows to be uniform moves to scalar registers and is waited for at once.
-                uint32_t zms_raw = 0, zmz_raw = 0;
-                // the zero term of the lane's table row and columns: fp16 tables sum z * xs; 8-bit tables sum zq * xs
-                // (the bytes as fp16 subnormals, zq * 2^-24) and xs, and z = (zq - mz) * ms is applied to the sums
-                float zacc[3] = {0.f, 0.f, 0.f}, zxs[3] = {0.f, 0.f, 0.f};
+        // What a slab has in flight or in registers.
+        struct Slab {
+            uint32_t k0;
+            uint32_t zms_raw, zmz_raw;
+            Raw16<SK> rs[3];
+            Raw16<ZK> rz[3];
+            u32x4 xr[2];
+            u32x2 xg, xh;
+            u32x4 cw[8][2]; // a step is 32 columns: four words of both row groups
+        };
+        // The loads of a slab's tables, activations and first code steps, in the order the arithmetic needs them.  The
+        // whole-tensor meta of the zero table has the same address in every lane, written so that the compiler does not
+        // see it (lane >> 6 is zero): a load it knows to be uniform moves to scalar registers and is waited for at once.
+        auto issue_first = [&](Slab &L, int slab) __attribute__((always_inline)) {
+            const uint32_t k0 = L.k0 = (uint32_t)slab * kSlab;
+            L.zms_raw = L.zmz_raw = 0;
+            if constexpr (Q8) {
+                L.zms_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_ms) + (lane >> 6));
+                L.zmz_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_mz) + (lane >> 6));
+            }
+#pragma unroll
+            for (int r = 0; r < 3; ++r) {
+                const uint32_t ce = trow_at[r] + k0;
+                uint32_t cm = 0;
                 if constexpr (Q8) {
-                    zms_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_ms) + (lane >> 6));
-                    zmz_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_mz) + (lane >> 6));
+                    cm = ce - __umulhi(ce, R.s_inv) * R.s_cols; // ce mod cols; the quotient estimate is at most 2 short
+                    cm -= cm >= R.s_cols ? R.s_cols : 0;
+                    cm -= cm >= R.s_cols ? R.s_cols : 0;
                 }
-                Raw16<SK> rs[3];
-                Raw16<ZK> rz[3];
+                if (Q8 && p.meta4) {
+                    // the meta columns are a multiple of 4 only: the lane's sixteen entries may wrap inside, four
+                    // pieces each with its own column
+                    L.rs[r].q = gload<u32x4>(R.sq + ce);
 #pragma unroll
-                for (int r = 0; r < 3; ++r) {
-                    const uint32_t ce = trow_at[r] + k0;
-                    uint32_t cm = 0;
-                    if constexpr (Q8) {
-                        cm = ce - __umulhi(ce, R.s_inv) * R.s_cols; // ce mod cols; the quotient estimate is at most 2 short
-                        cm -= cm >= R.s_cols ? R.s_cols : 0;
-                        cm -= cm >= R.s_cols ? R.s_cols : 0;
+                    for (int pc = 0; pc < 4; ++pc) {
+                        uint32_t c4 = cm + 4u * pc;
+                        c4 -= c4 >= R.s_cols ? R.s_cols : 0;
+                        const u32x2 a = gload<u32x2>(R.s_ms + c4), b = gload<u32x2>(R.s_mz + c4);
+                        L.rs[r].ms[pc >> 1][2 * (pc & 1)] = a.x, L.rs[r].ms[pc >> 1][2 * (pc & 1) + 1] = a.y;
+                        L.rs[r].mz[pc >> 1][2 * (pc & 1)] = b.x, L.rs[r].mz[pc >> 1][2 * (pc & 1) + 1] = b.y;
                     }
-                    if (Q8 && p.meta4) {
-                        // the meta columns are a multiple of 4 only: the lane's sixteen entries may wrap inside, four
-                        // pieces each with its own column
-                        rs[r].q = gload<u32x4>(R.sq + ce);
-#pragma unroll
-                        for (int pc = 0; pc < 4; ++pc) {
-                            uint32_t c4 = cm + 4u * pc;
-                            c4 -= c4 >= R.s_cols ? R.s_cols : 0;
-                            const u32x2 a = gload<u32x2>(R.s_ms + c4), b = gload<u32x2>(R.s_mz + c4);
-                            rs[r].ms[pc >> 1][2 * (pc & 1)] = a.x, rs[r].ms[pc >> 1][2 * (pc & 1) + 1] = a.y;
-                            rs[r].mz[pc >> 1][2 * (pc & 1)] = b.x, rs[r].mz[pc >> 1][2 * (pc & 1) + 1] = b.y;
-                        }
-                    } else {
-                        load16<SK>(rs[r], R.sq, R.s_ms, R.s_mz, ce, cm);
-                    }
-                    load16<ZK>(rz[r], R.zq, nullptr, nullptr, ce, 0);
-                }
-                u32x4 xr[2];
-                u32x2 xg = {0, 0}, xh = {0, 0};
-                if constexpr (XMODE) {
-                    xg = gload<u32x2>(p.xa + (int64_t)layer * p.x_lstride + k0 + (uint32_t)(4 * lane));
-                    xh = gload<u32x2>(p.xb + (int64_t)layer * p.x_lstride + k0 + (uint32_t)(4 * lane));
                 } else {
-                    xr[0] = gload<u32x4>(p.x + k0 + (uint32_t)(16 * qT));
-                    xr[1] = gload<u32x4>(p.x + k0 + (uint32_t)(16 * qT + 8));
+                    load16<SK>(L.rs[r], R.sq, R.s_ms, R.s_mz, ce, cm);
                 }
-                // A step is 32 columns: four words of both row groups.  The codes of the slab's second half are requested
-                // after the table phase: a wave that has issued its loads waits there, which lets the other wave of the
-                // SIMD issue its own (the older wave is served first), so that both have the first half of their data
-                // early and neither is left with a whole slab of arithmetic after the last byte has arrived.
-                u32x4 cw[8][2];
+                load16<ZK>(L.rz[r], R.zq, nullptr, nullptr, ce, 0);
+            }
+            L.xg = L.xh = (u32x2){0, 0};
+            if constexpr (XMODE) {
+                L.xg = gload<u32x2>(p.xa + (int64_t)layer * p.x_lstride + k0 + (uint32_t)(4 * lane));
+                L.xh = gload<u32x2>(p.xb + (int64_t)layer * p.x_lstride + k0 + (uint32_t)(4 * lane));
+            } else {
+                L.xr[0] = gload<u32x4>(p.x + k0 + (uint32_t)(16 * qT));
+                L.xr[1] = gload<u32x4>(p.x + k0 + (uint32_t)(16 * qT + 8));
+            }
 #pragma unroll
-                for (int s = 0; s < kW3Early; ++s)
+            for (int s = 0; s < kW3Early; ++s)
 #pragma unroll
-                    for (int g8 = 0; g8 < 2; ++g8)
-                        cw[s][g8] = gload<u32x4>(R.codes + (code_at[g8] + 4u * k0 + (uint32_t)(128 * s)));
-                __builtin_amdgcn_sched_barrier(0); // nothing below moves above the loads, no load sinks into the arithmetic
-                W3_STAMP(2);
-
-                // table phase: xs = 32 * s * x of the ten table rows into LDS, the zero term accumulated
-                if constexpr (Q8) // the meta values become opaque here, so no use of them is hoisted above the loads
-                    asm volatile("" : "+v"(zms_raw), "+v"(zmz_raw));
-                if constexpr (XMODE) {
-                    const f16x2 a01 = as_h2(xg.x), a23 = as_h2(xg.y), b01 = as_h2(xh.x), b23 = as_h2(xh.y);
-                    u32x2 hv;
-                    hv.x = as_u32((f16x2){silu_mul(a01.x, b01.x), silu_mul(a01.y, b01.y)});
-                    hv.y = as_u32((f16x2){silu_mul(a23.x, b23.x), silu_mul(a23.y, b23.y)});
-                    *reinterpret_cast<u32x2 *>(&h_lds[wave][4 * lane]) = hv;
-                    wave_sync();
-                    xr[0] = *reinterpret_cast<const u32x4 *>(&h_lds[wave][16 * qT]);
-                    xr[1] = *reinterpret_cast<const u32x4 *>(&h_lds[wave][16 * qT + 8]);
-                }
-                const f16x2 k32 = {(f16)kXsScale, (f16)kXsScale};
-                const f16x2 ones = {(f16)1.0f, (f16)1.0f};
+                for (int g8 = 0; g8 < 2; ++g8)
+                    L.cw[s][g8] = gload<u32x4>(R.codes + (code_at[g8] + 4u * k0 + (uint32_t)(128 * s)));
+            __builtin_amdgcn_sched_barrier(0); // nothing below moves above the loads, no load sinks into the arithmetic
+        };
+        // The codes of the slab's second half are requested after the table phase: a wave that has issued its loads
+        // waits there, which lets the other wave of the SIMD issue its own (the older wave is served first), so that
+        // both have the first half of their data early and neither is left with a whole slab of arithmetic after the
+        // last byte has arrived.
+        auto issue_second = [&](Slab &L) __attribute__((always_inline)) {
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int r = 0; r < 3; ++r) {
-                    if (HQQ_W3_SKIP(p, 2)) {
-                        asm volatile("" ::"v"(rs[r].q), "v"(rs[r].q_hi), "v"(rs[r].ms[0]), "v"(rs[r].ms[1]), "v"(rs[r].mz[0]),
-                                     "v"(rs[r].mz[1]), "v"(rz[r].q), "v"(rz[r].q_hi), "v"(xr[0]), "v"(xr[1]));
-                        continue;
-                    }
-                    const int f = r < 2 ? 4 * r + (lane >> 4) : 8 + ((lane >> 4) & 1);
-                    f16x2 sv[8], zv[8];
-                    decode16<SK>(rs[r], k32, k32, sv);
-                    if constexpr (!Q8)
-                        decode16<ZK>(rz[r], k32, k32, zv);
-                    uint32_t a[8];
+            for (int s = kW3Early; s < 8; ++s)
 #pragma unroll
-                    for (int t = 0; t < 8; ++t) {
-                        const f16x2 v = (sv[t] * k32) * as_h2(xr[t >> 2][t & 3]);
-                        if constexpr (Q8) {
-                            // bytes 2 * (t & 1), 2 * (t & 1) + 1 of the word into the low bytes of the two halves
-                            const uint32_t zq = __builtin_amdgcn_perm(0u, rz[r].q[t >> 1], (t & 1) ? 0x0c030c02u : 0x0c010c00u);
-                            zacc[r] = __builtin_amdgcn_fdot2(as_h2(zq), v, zacc[r], false);
-                            zxs[r] = __builtin_amdgcn_fdot2(ones, v, zxs[r], false);
-                        } else {
-                            zacc[r] = __builtin_amdgcn_fdot2(zv[t], v, zacc[r], false);
-                        }
-                        a[t] = as_u32(v);
-                    }
-                    if (r < 2 || third_ok) {
-#pragma unroll
-                        for (int pi = 0; pi < 4; ++pi)
-                            *reinterpret_cast<u32x2 *>(xs_w + ((qT * 4 + pi) * 10 + f) * 4) = (u32x2){a[2 * pi], a[2 * pi + 1]};
-                    }
-                }
-                // the zero terms of the slab: summed over the sixteen chunk lanes of a table row and added up in LDS,
-                // here rather than after the last code step, where every instruction delays the block's result
-#pragma unroll
-                for (int r = 0; r < 3; ++r) {
-                    const int f = r < 2 ? 4 * r + (lane >> 4) : 8 + ((lane >> 4) & 1);
-                    float z = zacc[r];
-                    if constexpr (Q8) {
-                        const float ms = (float)__builtin_bit_cast(f16, (uint16_t)zms_raw), mz = (float)__builtin_bit_cast(f16, (uint16_t)zmz_raw);
-                        z = ms * (z * 16777216.0f - mz * zxs[r]);
-                    }
-                    z = row16_sum(z);
-                    if (qT == 0 && (r < 2 || third_ok))
-                        zt_lds[wave][f] += z;
-                }
+                for (int g8 = 0; g8 < 2; ++g8)
+                    L.cw[s][g8] = gload<u32x4>(R.codes + (code_at[g8] + 4u * L.k0 + (uint32_t)(128 * s)));
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        // table phase: xs = 32 * s * x of the ten table rows into LDS, and the zero terms
+        auto table_phase = [&](Slab &L) __attribute__((always_inline)) {
+            if constexpr (Q8) // the meta values become opaque here, so no use of them is hoisted above the loads
+                asm volatile("" : "+v"(L.zms_raw), "+v"(L.zmz_raw));
+            if constexpr (XMODE) {
+                const f16x2 a01 = as_h2(L.xg.x), a23 = as_h2(L.xg.y), b01 = as_h2(L.xh.x), b23 = as_h2(L.xh.y);
+                u32x2 hv;
+                hv.x = as_u32((f16x2){silu_mul(a01.x, b01.x), silu_mul(a01.y, b01.y)});
+                hv.y = as_u32((f16x2){silu_mul(a23.x, b23.x), silu_mul(a23.y, b23.y)});
+                *reinterpret_cast<u32x2 *>(&h_lds[wave][4 * lane]) = hv;
                 wave_sync();
-                __builtin_amdgcn_sched_barrier(0);
+                L.xr[0] = *reinterpret_cast<const u32x4 *>(&h_lds[wave][16 * qT]);
+                L.xr[1] = *reinterpret_cast<const u32x4 *>(&h_lds[wave][16 * qT + 8]);
+            }
+            const f16x2 k32 = {(f16)kXsScale, (f16)kXsScale};
+            const f16x2 ones = {(f16)1.0f, (f16)1.0f};
+            // the zero term of the lane's table row and columns: fp16 tables sum z * xs; 8-bit tables sum zq * xs (the
+            // bytes as fp16 subnormals, zq * 2^-24) and xs, and z = (zq - mz) * ms is applied to the sums
+            float zacc[3] = {0.f, 0.f, 0.f}, zxs[3] = {0.f, 0.f, 0.f};
 #pragma unroll
-                for (int s = kW3Early; s < 8; ++s)
+            for (int r = 0; r < 3; ++r) {
+                if (HQQ_W3_SKIP(p, 2)) {
+                    asm volatile("" ::"v"(L.rs[r].q), "v"(L.rs[r].q_hi), "v"(L.rs[r].ms[0]), "v"(L.rs[r].ms[1]), "v"(L.rs[r].mz[0]),
+                                 "v"(L.rs[r].mz[1]), "v"(L.rz[r].q), "v"(L.rz[r].q_hi), "v"(L.xr[0]), "v"(L.xr[1]));
+                    continue;
+                }
+                const int f = r < 2 ? 4 * r + (lane >> 4) : 8 + ((lane >> 4) & 1);
+                f16x2 sv[8], zv[8];
+                decode16<SK>(L.rs[r], k32, k32, sv);
+                if constexpr (!Q8)
+                    decode16<ZK>(L.rz[r], k32, k32, zv);
+                uint32_t a[8];
 #pragma unroll
-                    for (int g8 = 0; g8 < 2; ++g8)
-                        cw[s][g8] = gload<u32x4>(R.codes + (code_at[g8] + 4u * k0 + (uint32_t)(128 * s)));
-                __builtin_amdgcn_sched_barrier(0);
-                W3_STAMP(3);
-
-                // code phase: per word two plain masks and two byte gathers with three masks.  The B operands of a step
-                // are read from LDS a step ahead.
-                auto read_b = [&](u32x2 &bx, u32x2 &by, int s) __attribute__((always_inline)) {
-                    bx = *reinterpret_cast<const u32x2 *>(reinterpret_cast<const char *>(xs_w) + b_at + s * 640);
-                    by = *reinterpret_cast<const u32x2 *>(reinterpret_cast<const char *>(xs_w) + b4_at + s * 640);
-                };
-                u32x2 bx, by;
-                read_b(bx, by, 0);
-#pragma unroll
-                for (int s = 0; s < 8; ++s) {
-                    const u32x4 bu = {__builtin_amdgcn_perm(0u, bx.x, sel_a), __builtin_amdgcn_perm(0u, bx.x, sel_b),
-                                      __builtin_amdgcn_perm(0u, bx.y, sel_a), __builtin_amdgcn_perm(0u, bx.y, sel_b)};
-                    const u32x4 bv = {__builtin_amdgcn_perm(0u, by.x, sel_a), __builtin_amdgcn_perm(0u, by.x, sel_b),
-                                      __builtin_amdgcn_perm(0u, by.y, sel_a), __builtin_amdgcn_perm(0u, by.y, sel_b)};
-                    const f16x8 B = __builtin_bit_cast(f16x8, bu), B4 = __builtin_bit_cast(f16x8, bv);
-                    if (s + 1 < 8)
-                        read_b(bx, by, s + 1);
-#ifdef HQQ_TUNING_BUILD
-                    if (s == 1 || s == 2 || s == 4 || s == 6) {
-                        asm volatile("" ::"v"(cw[s][0]));
-                        W3_STAMP(s == 1 ? 4 : s == 2 ? 5 : s == 4 ? 6 : 7);
+                for (int t = 0; t < 8; ++t) {
+                    const f16x2 v = (sv[t] * k32) * as_h2(L.xr[t >> 2][t & 3]);
+                    if constexpr (Q8) {
+                        // bytes 2 * (t & 1), 2 * (t & 1) + 1 of the word into the low bytes of the two halves
+                        const uint32_t zq = __builtin_amdgcn_perm(0u, L.rz[r].q[t >> 1], (t & 1) ? 0x0c030c02u : 0x0c010c00u);
+                        zacc[r] = __builtin_amdgcn_fdot2(as_h2(zq), v, zacc[r], false);
+                        zxs[r] = __builtin_amdgcn_fdot2(ones, v, zxs[r], false);
+                    } else {
+                        zacc[r] = __builtin_amdgcn_fdot2(zv[t], v, zacc[r], false);
                     }
+                    a[t] = as_u32(v);
+                }
+                if (r < 2 || third_ok) {
+#pragma unroll
+                    for (int pi = 0; pi < 4; ++pi)
+                        *reinterpret_cast<u32x2 *>(xs_w + ((qT * 4 + pi) * 10 + f) * 4) = (u32x2){a[2 * pi], a[2 * pi + 1]};
+                }
+            }
+            // the zero terms of the slab: summed over the sixteen chunk lanes of a table row and added up in LDS, here
+            // rather than after the last code step, where every instruction delays the block's result
+#pragma unroll
+            for (int r = 0; r < 3; ++r) {
+                const int f = r < 2 ? 4 * r + (lane >> 4) : 8 + ((lane >> 4) & 1);
+                float z = zacc[r];
+                if constexpr (Q8) {
+                    const float ms = (float)__builtin_bit_cast(f16, (uint16_t)L.zms_raw), mz = (float)__builtin_bit_cast(f16, (uint16_t)L.zmz_raw);
+                    z = ms * (z * 16777216.0f - mz * zxs[r]);
+                }
+                z = row16_sum(z);
+                if (qT == 0 && (r < 2 || third_ok))
+                    zt_lds[wave][f] += z;
+            }
+            wave_sync();
+        };
+        // code phase: per word two plain masks and two byte gathers with three masks.  The B operands of a step are read
+        // from LDS a step ahead.
+        auto code_phase = [&](const Slab &L) __attribute__((always_inline)) {
+            auto read_b = [&](u32x2 &bx, u32x2 &by, int s) __attribute__((always_inline)) {
+                bx = *reinterpret_cast<const u32x2 *>(reinterpret_cast<const char *>(xs_w) + b_at + s * 640);
+                by = *reinterpret_cast<const u32x2 *>(reinterpret_cast<const char *>(xs_w) + b4_at + s * 640);
+            };
+            u32x2 bx, by;
+            read_b(bx, by, 0);
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                const u32x4 bu = {__builtin_amdgcn_perm(0u, bx.x, sel_a), __builtin_amdgcn_perm(0u, bx.x, sel_b),
+                                  __builtin_amdgcn_perm(0u, bx.y, sel_a), __builtin_amdgcn_perm(0u, bx.y, sel_b)};
+                const u32x4 bv = {__builtin_amdgcn_perm(0u, by.x, sel_a), __builtin_amdgcn_perm(0u, by.x, sel_b),
+                                  __builtin_amdgcn_perm(0u, by.y, sel_a), __builtin_amdgcn_perm(0u, by.y, sel_b)};
+                const f16x8 B = __builtin_bit_cast(f16x8, bu), B4 = __builtin_bit_cast(f16x8, bv);
+                if (s + 1 < 8)
+                    read_b(bx, by, s + 1);
+#ifdef HQQ_TUNING_BUILD
+                if (s == 1 || s == 2 || s == 4 || s == 6) {
+                    asm volatile("" ::"v"(L.cw[s][0]));
+                    W3_STAMP(s == 1 ? 4 : s == 2 ? 5 : s == 4 ? 6 : 7);
+                }
 #endif
 #pragma unroll
-                    for (int g8 = 0; g8 < 2; ++g8) {
-                        const u32x4 w = cw[s][g8];
-                        if (HQQ_W3_SKIP(p, 1)) {
-                            asm volatile("" ::"v"(w));
-                            continue;
-                        }
-                        u32x4 wa, wb;
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            wa[j] = __builtin_amdgcn_perm(w[j], w[j], kW3GatherA);
-                            wb[j] = __builtin_amdgcn_perm(w[j], w[j], kW3GatherB);
-                        }
-                        acc[g8][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, w & mk[0]), B, acc[g8][0], 0, 0, 0);
-                        acc[g8][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, w & mk[1]), B, acc[g8][1], 0, 0, 0);
-                        acc[g8][2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, wb & mk[2]), B, acc[g8][2], 0, 0, 0);
-                        acc[g8][3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, wa & mk[3]), B, acc[g8][3], 0, 0, 0);
-                        acc[g8][4] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, wa & mk[4]), B4, acc[g8][4], 0, 0, 0);
+                for (int g8 = 0; g8 < 2; ++g8) {
+                    const u32x4 w = L.cw[s][g8];
+                    if (HQQ_W3_SKIP(p, 1)) {
+                        asm volatile("" ::"v"(w));
+                        continue;
                     }
+                    u32x4 wa, wb;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        wa[j] = __builtin_amdgcn_perm(w[j], w[j], kW3GatherA);
+                        wb[j] = __builtin_amdgcn_perm(w[j], w[j], kW3GatherB);
+                    }
+                    acc[g8][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, w & mk[0]), B, acc[g8][0], 0, 0, 0);
+                    acc[g8][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, w & mk[1]), B, acc[g8][1], 0, 0, 0);
+                    acc[g8][2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, wb & mk[2]), B, acc[g8][2], 0, 0, 0);
+                    acc[g8][3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, wa & mk[3]), B, acc[g8][3], 0, 0, 0);
+                    acc[g8][4] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, wa & mk[4]), B4, acc[g8][4], 0, 0, 0);
                 }
-                wave_sync();
-                W3_STAMP(8);
             }
+            wave_sync(); // the next table phase writes where these steps have read
+        };
+
+        if (wave < p.KS && slab_lo < slab_hi) {
+            Slab A;
+            W3_STAMP(1);
+            issue_first(A, slab_lo);
+            W3_STAMP(2);
+            table_phase(A);
+            issue_second(A);
+            W3_STAMP(3);
+            if constexpr (S == 2) {
+                // The second slab's tables and first code steps are requested before the first slab's codes are worked
+                // on (unconditionally: a wave whose second slab lies past its range reads the first again and leaves
+                // out the arithmetic).
+                const bool two = slab_lo + 1 < slab_hi;
+                Slab B;
+                issue_first(B, two ? slab_lo + 1 : slab_lo);
+                code_phase(A);
+                if (two) {
+                    table_phase(B);
+                    issue_second(B);
+                    code_phase(B);
+                }
+            } else {
+                code_phase(A);
+            }
+            W3_STAMP(8);
         }
 
         // wave result
