@@ -285,7 +285,8 @@ int hqq_attention_chain(const hqq_linear *q, const hqq_linear *k, const hqq_line
  *      (rows, cols) matrix whose columns are the groups (axis 0; rows = group size 8, 16, 32, 64 or 128).  w is fp16
  *      (w_is_fp32 = 0) or fp32.  scale = min((2^nbits - 1) / (max - min), 2e4), zero = -min * scale (rounded when
  *      round_zero), refined by `iters` iterations at most of hqq's half-quadratic solver when iters > 0 (lp_norm 0.7,
- *      beta 10, kappa 1.01, 20 iterations are hqq's defaults; the solver stops for the whole tensor when the mean
+ *      beta 10, kappa 1.01, 20 iterations are hqq's defaults; beta and kappa are doubles, as in the reference's host
+ *      loop, so that beta takes the same sequence of values; the solver stops for the whole tensor when the mean
  *      absolute error no longer falls), then q = clamp(round(w * scale + zero), 0, 2^nbits - 1).  Outputs: codes
  *      uint8 (rows, cols), unpacked; inv_scale fp32 (cols) = 1 / scale; zero fp32 (cols).  The workspace (8-byte
  *      aligned, hqq_quantize_workspace_bytes()) is only needed when iters > 0.  hqq_quantize_whole is the one-group
@@ -293,7 +294,7 @@ int hqq_attention_chain(const hqq_linear *q, const hqq_linear *k, const hqq_line
  *      the workspace.                                                                                              */
 size_t hqq_quantize_workspace_bytes(void);
 int hqq_quantize_groups(const void *w, int32_t w_is_fp32, int64_t rows, int64_t cols, int32_t nbits, int32_t round_zero,
-                        int32_t iters, float lp_norm, float beta, float kappa, void *codes_u8, void *inv_scale_f32,
+                        int32_t iters, float lp_norm, double beta, double kappa, void *codes_u8, void *inv_scale_f32,
                         void *zero_f32, void *workspace, size_t workspace_bytes, void *stream);
 int hqq_quantize_whole(const void *x_f32, int64_t n, int32_t nbits, void *codes_u8, void *inv_scale_f32, void *zero_f32,
                        void *workspace, size_t workspace_bytes, void *stream);

@@ -739,7 +739,7 @@ int hqq_attention_decode(const void *q_f16, const void *k_f16, const void *v_f16
 size_t hqq_quantize_workspace_bytes(void) { return quantize_workspace_bytes(); }
 
 int hqq_quantize_groups(const void *w, int32_t w_is_fp32, int64_t rows, int64_t cols, int32_t nbits, int32_t round_zero,
-                        int32_t iters, float lp_norm, float beta, float kappa, void *codes_u8, void *inv_scale_f32,
+                        int32_t iters, float lp_norm, double beta, double kappa, void *codes_u8, void *inv_scale_f32,
                         void *zero_f32, void *workspace, size_t workspace_bytes, void *stream)
 {
     if (!w || !codes_u8 || !inv_scale_f32 || !zero_f32)

@@ -205,7 +205,7 @@ int launch_zero_workspace_head(void *ws, size_t ws_bytes, hipStream_t s);
 // the quantiser (quantize_kernels.hip)
 size_t quantize_workspace_bytes();
 int launch_quantize_groups(const void *w, int fp32_in, int64_t rows, int64_t cols, int nbits, int round_zero, int iters,
-                           float lp, float beta, float kappa, uint8_t *codes, float *inv_scale, float *zero, void *ws,
+                           float lp, double beta, double kappa, uint8_t *codes, float *inv_scale, float *zero, void *ws,
                            size_t ws_bytes, hipStream_t s);
 int launch_quantize_whole(const float *x, int64_t n, int nbits, uint8_t *codes, float *inv_scale, float *zero, void *ws,
                           size_t ws_bytes, hipStream_t s);

@@ -31,7 +31,8 @@ struct QuantParams {
     float max_v;
     int round_zero;
     int iters;
-    float lp, beta, kappa;
+    float lp;
+    double beta, kappa; // doubles, as in the host loop they restate
     uint8_t *codes;   // (rows, cols)
     float *inv_scale; // (cols)
     float *zero;      // (cols)
@@ -95,7 +96,7 @@ template <int GS, int CP, int PASS> __global__ __launch_bounds__(kQThreads) void
     if constexpr (PASS != 0) {
         const int iters = PASS == 1 ? p.iters : *p.stop;
         __shared__ double red[kQThreads / 64];
-        double beta = (double)p.beta; // the host loop keeps beta as a double and hands 1 / beta to fp32 tensor ops
+        double beta = p.beta; // the host loop keeps beta as a double and hands 1 / beta to fp32 tensor ops
         const float pm1 = p.lp - 1.0f;
         for (int it = 0; it < iters; ++it) {
             const float inv_beta = (float)(1.0 / beta);
@@ -116,7 +117,7 @@ template <int GS, int CP, int PASS> __global__ __launch_bounds__(kQThreads) void
                 zero[j] = acc / (float)GS;
                 e += ej;
             }
-            beta *= (double)p.kappa;
+            beta *= p.kappa;
             if constexpr (PASS == 1) {
                 double s = on ? (double)e : 0.0;
 #pragma unroll
@@ -292,7 +293,7 @@ template <int GS> int run_groups(const QuantParams &p, hipStream_t s)
 size_t quantize_workspace_bytes() { return kQMaxIters * sizeof(double) + 64; }
 
 int launch_quantize_groups(const void *w, int fp32_in, int64_t rows, int64_t cols, int nbits, int round_zero, int iters,
-                           float lp, float beta, float kappa, uint8_t *codes, float *inv_scale, float *zero, void *ws,
+                           float lp, double beta, double kappa, uint8_t *codes, float *inv_scale, float *zero, void *ws,
                            size_t ws_bytes, hipStream_t s)
 {
     if (rows < 1 || cols < 1 || nbits < 1 || nbits > 8 || iters < 0 || iters > kQMaxIters)

@@ -89,7 +89,7 @@ _SIGNATURES = {
                                c_void_p, c_size_t, c_void_p]),
     "hqq_quantize_workspace_bytes": (c_size_t, []),
     "hqq_quantize_groups": (c_int, [c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, ctypes.c_float,
-                                    ctypes.c_float, ctypes.c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+                                    ctypes.c_double, ctypes.c_double, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hqq_quantize_whole": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hqq_attention_decode_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32]),
     "hqq_attention_decode_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,

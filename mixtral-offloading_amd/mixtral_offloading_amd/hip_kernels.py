@@ -584,7 +584,7 @@ def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: tor
                      pos: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, out: torch.Tensor,
                      split: bool = True) -> torch.Tensor:
     """Rope, cache append and attention of one new token; ``pos`` is an int64 device tensor with the position.
-    Caches longer than 512 positions are split over several blocks per head unless ``split`` is False."""
+    Caches longer than 1024 positions are split over several blocks per head unless ``split`` is False."""
     n_kv, max_len, hd = cache_k.shape
     n_heads = q.numel() // hd
     assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous() and cache_k.is_contiguous() and cache_v.is_contiguous()

@@ -52,7 +52,8 @@ class Rotary:
 
     def causal_bias(self, T, start, g):
         """fp32 (g * T, start + T): 0 where row r (token r % T at position start + r % T) may attend, -inf elsewhere.
-        The last one made is kept: the layers of a pass all ask for the same one."""
+        The last one made is kept while a pass runs (its layers all ask for the same one); forward_tokens drops it
+        at the end of the pass, a long prompt's bias being hundreds of megabytes."""
         key = (T, start, g)
         if getattr(self, "_bias_key", None) != key:
             dev = self.cos.device
@@ -61,6 +62,9 @@ class Rotary:
             self._bias = torch.zeros(allowed.shape, dtype=torch.float32, device=dev).masked_fill_(~allowed, float("-inf"))
             self._bias_key = key
         return self._bias
+
+    def drop_causal_bias(self):
+        self._bias, self._bias_key = None, None
 
     def apply(self, q, k, positions):
         cos, sin = self.cos[positions][:, None, :], self.sin[positions][:, None, :]  # (T, 1, hd)
@@ -424,6 +428,7 @@ class MixtralForCausalLM(nn.Module):
         x = self.model.embed_tokens(input_ids)  # a new tensor: the layers update it in place
         for layer, (ck, cv) in zip(self.model.layers, cache):
             x = layer(x, self.rotary, ck, cv, start, inplace=True)
+        self.rotary.drop_causal_bias()
         return self.lm_head(self.model.norm(x))
 
     @torch.inference_mode()

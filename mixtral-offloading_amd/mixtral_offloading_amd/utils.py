@@ -45,24 +45,6 @@ def nested_pack(flat, structure):
     return build(structure)
 
 
-def nested_compare(t, u) -> bool:
-    """Do the two structures have the same shape (containers and keys)?"""
-    if isinstance(t, (list, tuple)):
-        return isinstance(u, type(t)) and len(t) == len(u) and all(nested_compare(a, b) for a, b in zip(t, u))
-    if isinstance(t, dict):
-        return isinstance(u, dict) and set(t) == set(u) and all(nested_compare(t[k], u[k]) for k in t)
-    return True
-
-
-def nested_map(fn, *t):
-    if not t:
-        raise ValueError("Expected 2+ arguments, got 1")
-    for other in t[1:]:
-        if not nested_compare(t[0], other):
-            raise ValueError("Nested structure of %r and %r differs" % (t[0], other))
-    return nested_pack(map(fn, *map(nested_flatten, t)), t[0])
-
-
 @contextmanager
 def with_default_dtype(dtype):
     saved = torch.get_default_dtype()
