@@ -37,7 +37,8 @@
 // (launches with more outputs than there are slots store fp32 partial sums instead, and the block that arrives
 // last at the tile's counter adds them in a fixed order).  Batches above two rows run as passes of two.
 //
-// A launch may hold up to four layers of one shape (blockIdx.z = layer * P + window): the two projections of an
+// A launch may hold up to four layers of one shape (a one-dimensional grid over layer, window, row block and K
+// block, see the kernel): the two projections of an
 // expert's gate, or those of two experts.  Their records come from the kernel arguments or from a device table
 // (record sel[layer / lper] * stride + first + layer % lper), so that the expert can be chosen on the device.
 // XMODE 1 builds the activations on the fly as silu(xa) * xb, which is how the down projection reads the two
@@ -85,7 +86,11 @@ struct W3Params {
     int SB; // slabs per block
     int BK; // blocks along K per tile
     int meta4; // the scale table's meta columns are a multiple of 4 but not of 16
+    // the work list (see the kernel): blocks per XCD, XCDs with one more, magic multipliers ceil(2^32 / d) of the
+    // divisions, and the window of list position n: (n * win_mul) mod P
+    uint32_t per_xcd, xcd_more, bk_magic, rb_magic, p_magic, win_mul;
 #ifdef HQQ_TUNING_BUILD
+    int plain_order; // timing experiments: blocks take the work list in launch order
     int skip; // timing experiments: 1 leaves out the code phase, 2 the table phase (their loads are still waited for)
     unsigned long long *stamps; // per-wave time stamps, [block][16 waves][16], or null
 #endif
@@ -182,9 +187,25 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
                  "s"(p.y), "s"(p.y_lstride), "s"(p.part), "s"(p.part_lstride));
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int kb = blockIdx.x, rb = blockIdx.y;
-    const int layer = (int)(blockIdx.z >= (unsigned)p.P) + (int)(blockIdx.z >= 2u * p.P) + (int)(blockIdx.z >= 3u * p.P);
-    const int w0 = (int)blockIdx.z - layer * p.P;
+    // Which tile this block works on.  Consecutive blocks of a launch go to the eight XCDs in turn, each with an L2 of
+    // its own, and a table row is needed by several windows (ten rows per window, G / gcd(10, G) windows): block b is
+    // the (b / 8)-th block of XCD b % 8, every XCD takes a contiguous range of the work list, and the list runs over
+    // the windows in the order of their first table row, so that windows which share table rows meet in one L2.
+    uint32_t v;
+    {
+        const uint32_t xcd = blockIdx.x & 7u, nth = blockIdx.x >> 3;
+        v = xcd * p.per_xcd + (xcd < p.xcd_more ? xcd : p.xcd_more) + nth;
+#ifdef HQQ_TUNING_BUILD
+        if (p.plain_order)
+            v = blockIdx.x;
+#endif
+    }
+    auto div = [](uint32_t a, uint32_t d, uint32_t magic) { return d == 1 ? a : __umulhi(a, magic); }; // a * d < 2^32
+    const uint32_t v1 = div(v, (uint32_t)p.BK, p.bk_magic), v2 = div(v1, (uint32_t)p.RB, p.rb_magic);
+    const int kb = (int)(v - v1 * (uint32_t)p.BK), rb = (int)(v1 - v2 * (uint32_t)p.RB);
+    const int layer = (int)div(v2, (uint32_t)p.P, p.p_magic);
+    const uint32_t nthw = v2 - (uint32_t)layer * (uint32_t)p.P, step = nthw * p.win_mul; // below 2^20 each way
+    const int w0 = (int)(step - div(step, (uint32_t)p.P, p.p_magic) * (uint32_t)p.P);
     // The layer's record.  From a table it is read one word per lane and broadcast; every load through it below is
     // an explicit device-memory load (a pointer out of a record has lost its address space).
     LayerRecord R;
@@ -711,7 +732,7 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
     auto write_stamps = [&]() __attribute__((always_inline)) {
         if (p.stamps && lane == 0) {
             st[13] = __builtin_amdgcn_s_memrealtime();
-            unsigned long long *d = p.stamps + ((size_t)((blockIdx.z * gridDim.y + rb) * gridDim.x + kb) * 16 + wave) * 16;
+            unsigned long long *d = p.stamps + ((size_t)blockIdx.x * 16 + wave) * 16;
             for (int i = 0; i < 14; ++i)
                 d[i] = st[i];
             d[14] = __builtin_amdgcn_s_getreg((31 << 11) | 4);  // HW_ID
@@ -851,6 +872,8 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, W3Plan &pl)
     pl.KS = (pl.SB + pl.S - 1) / pl.S;
     if ((int64_t)pl.P * NL > 65535 || pl.RB > 65535 || (int64_t)pl.P * pl.RB * NL * sizeof(int) > kTileCounterBytes)
         return false;
+    if ((int64_t)pl.P * NL * pl.RB * pl.BK * (pl.RB > pl.BK ? pl.RB : pl.BK) >= (1ll << 32))
+        return false; // the kernel's block-to-tile divisions are exact below this
     return true;
 }
 
@@ -943,11 +966,27 @@ int run_job(const W3Job &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
     p.meta4 = pl.q8 && l->scale.meta_cols % 16 != 0;
 #ifdef HQQ_TUNING_BUILD
     p.skip = tuning_int("HQQ_W3_SKIP", 0);
+    p.plain_order = tuning_int("HQQ_W3_ORDER", 0) & 1;
     p.stamps = g_w3_stamps;
 #endif
     p.N = (int)l->N, p.K = (int)l->K, p.G = pl.G, p.P = pl.P, p.NW = pl.NW, p.RB = pl.RB;
     p.NS = pl.NS, p.KS = pl.KS, p.S = pl.S, p.SB = pl.SB, p.BK = pl.BK;
-    const dim3 grid((unsigned)pl.BK, (unsigned)pl.RB, (unsigned)(pl.P * j.NL));
+    const uint32_t blocks = (uint32_t)pl.BK * (uint32_t)pl.RB * (uint32_t)(pl.P * j.NL);
+    const dim3 grid(blocks);
+    auto magic = [](int d) { return (uint32_t)((1ull << 32) / (uint32_t)d + 1); };
+    p.per_xcd = blocks / 8, p.xcd_more = blocks % 8;
+    p.bk_magic = magic(pl.BK), p.rb_magic = magic(pl.RB), p.p_magic = magic(pl.P);
+    // Windows in the order of their first table row: window w starts at row 10 w mod G = g * ((10 / g) w mod P) with
+    // g = gcd(10, G), so list position n holds the window with (10 / g) w = n (mod P).
+    p.win_mul = 1;
+    if (pl.P <= 1024 && !(tuning_int("HQQ_W3_ORDER", 0) & 2)) {
+        const int t = 10 / gcd_int(10, pl.G);
+        for (int w = 1; w < pl.P; ++w)
+            if ((int64_t)t * w % pl.P == 1) {
+                p.win_mul = (uint32_t)w;
+                break;
+            }
+    }
     for (int64_t m0 = 0; m0 < M; m0 += 2) { // passes of two batch rows; later passes find the weights in the caches
         const int mb = M - m0 >= 2 ? 2 : 1;
         if (fused)
