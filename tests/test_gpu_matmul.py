@@ -382,3 +382,38 @@ def test_decode_batch_kernel_keeps_nan_and_infinity(m):
             err = (y[rest].float() - ref[rest]).abs()
             bound = 1e-2 * ref[rest].abs() + 1e-3 * x[rest].float().norm(dim=1)[:, None] * w.norm(dim=1)[None, :]
             assert bool((err <= bound).all())
+
+
+# (N, K, group size, meta group size, 8-bit tables): 3-bit layers the single-row kernel takes (K a multiple of 256).
+# Table-row counts G = N / group size of 20, 10, 80, 24, 12 and 40 give windows of word rows P = G / gcd(10, G) of
+# 2, 1, 8, 12, 6 and 4; 768x1280 has 120 meta columns (a multiple of 4 only: a lane's sixteen table entries wrap
+# inside); 1280x4608 and 400x8192 split K over waves with two slabs each and over several blocks; the block counts
+# include ones that are not a multiple of the eight XCDs the work list is dealt to.
+W3_SHAPES = [
+    (1280, 512, 64, 128, True),
+    (640, 1024, 64, 128, False),
+    (2960, 256, 37, 128, True),
+    (1296, 512, 54, 128, True),
+    (768, 1280, 64, 128, True),
+    (1280, 4608, 32, 128, True),
+    (400, 8192, 40, 128, False),
+    (130, 256, 13, 128, True),
+]
+
+
+@pytest.mark.parametrize("shape", W3_SHAPES, ids=lambda s: "%dx%d_g%d_%s" % (s[:3] + ("q" if s[4] else "f16",)))
+def test_three_bit_single_row_kernel(shape):
+    """One batch row (the codes on the matrix cores), three rows (a pass of two and a pass of one) and two rows, with
+    and without bias, twice over so that the accumulation slots are found clean."""
+    from mixtral_offloading_amd import _lib
+    n, k, gs, mgs, q8 = shape
+    rng = np.random.default_rng(n + 11 * k)
+    layer, _ = o.random_layer(rng, n, k, 3, gs, q8, q8, meta_group_size=mgs)
+    assert _lib.lib.hqq_matmul_kernel_family(desc_of(layer).ref, 1) == _lib.FAM_VEC3
+    for m in (1, 3, 2, 1):
+        x = rng.standard_normal((m, k)).astype(np.float16)
+        bias = rng.standard_normal(n).astype(np.float16) if m == 3 else None
+        _check(layer, x, bias=bias)
+    # activations forty times larger: nothing overflows on the way
+    x = (rng.standard_normal((1, k)) * 40).astype(np.float16)
+    _check(layer, x)
