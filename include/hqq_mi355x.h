@@ -103,8 +103,9 @@ int hqq_dequantize(const hqq_linear *l, void *w_out_f16, void *stream);
 size_t hqq_matmul_workspace_bytes(const hqq_linear *l, int64_t M);
 /* zero the head (counters and slots) of a workspace with a small fill kernel (safe under stream capture)            */
 int hqq_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
-/* same, with the kernel family forced (-1 = automatic choice, else 0..4 as hqq_matmul_kernel_family reports):
- * HQQ_E_UNSUPPORTED when that family does not take the configuration.  For tests and profiling.                    */
+/* same, with the kernel family forced (-1 = automatic choice, else 0..5 as hqq_matmul_kernel_family reports):
+ * HQQ_E_UNSUPPORTED when that family does not take the configuration.  For tests and profiling.  (Family 5 forced
+ * on a batch smaller than it is chosen from needs 576 KiB + 2 * N * K bytes of workspace.)                          */
 int hqq_matmul_transpose_ex(const hqq_linear *l, const void *x_f16, int64_t M, void *y_f16, void *workspace,
                             size_t workspace_bytes, int family, void *stream);
 int hqq_matmul_transpose(const hqq_linear *l, const void *x_f16, int64_t M, void *y_f16, void *workspace,
@@ -300,8 +301,11 @@ int hqq_quantize_whole(const void *x_f32, int64_t n, int32_t nbits, void *codes_
                        void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- which kernel family a call would use (for tests and profiles): 0 general, 1 MFMA small-batch, 2 MFMA tile,
- *      3 three-bit vector kernel, 4 MFMA kernel with weights dequantised into shared memory (reads 3-bit words as
- *      they are stored).                                                                                              */
+ *      3 three-bit decode kernel, 4 MFMA kernel with weights dequantised into shared memory (reads 3-bit words as
+ *      they are stored), 5 batches of hundreds of rows: hqq_dequantize into the workspace, then one fp16 GEMM of the
+ *      vendor's library (rocBLAS) with fp32 accumulation, which is the reference's PyTorch path
+ *      (src/custom_layers.py:95-116 and torch.matmul); hqq_matmul_workspace_bytes grows by 2 * N * K bytes there.
+ *      The first such call on a device creates the library's handle (it allocates: not under stream capture).      */
 int hqq_matmul_kernel_family(const hqq_linear *l, int64_t M);
 
 /* ---- expert offload: replaces the two copies of ExpertCache._swap (src/expert_cache.py:186-189).

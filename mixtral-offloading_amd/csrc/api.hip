@@ -41,7 +41,7 @@ int validate_linear(const hqq_linear *l)
 
 static inline size_t align256(size_t v) { return (v + 255u) & ~(size_t)255u; }
 
-enum { FAM_GENERAL = 0, FAM_SMALLBATCH = 1, FAM_TILE = 2, FAM_VEC3 = 3, FAM_LDS = 4 };
+enum { FAM_GENERAL = 0, FAM_SMALLBATCH = 1, FAM_TILE = 2, FAM_VEC3 = 3, FAM_LDS = 4, FAM_DQGEMM = 5 };
 constexpr int64_t kSmallBatchMax = 16;
 
 // a batch wider than the small-batch kernels take, run as slices of 16 rows (the weights of the later slices come
@@ -50,6 +50,8 @@ static bool sliced_supported(const hqq_linear *l, int64_t M) { return M > kSmall
 
 static int pick_family(const hqq_linear *l, int64_t M)
 {
+    if (dqgemm_preferred(l, M)) // hundreds of rows: de-quantise once, then a library GEMM
+        return FAM_DQGEMM;
     if (strip_supported(l, M)) // decode batches: part of the small-batch family
         return FAM_SMALLBATCH;
     if (l->nbits == 3 && M >= 5 && M <= kSmallBatchMax && ldsgemm_supported(l, M)) // 3-bit words read as they are stored
@@ -79,6 +81,8 @@ static size_t family_workspace(const hqq_linear *l, int64_t M, int fam)
         return tile_workspace_bytes(l, M);
     if (fam == FAM_LDS)
         return ldsgemm_workspace_bytes(l, M);
+    if (fam == FAM_DQGEMM)
+        return dqgemm_workspace_bytes(l, M);
     return 0;
 }
 
@@ -105,6 +109,8 @@ static int run_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void
         return launch_tile_matmul(l, x, M, y, ws, ws_bytes, s);
     case FAM_LDS:
         return launch_ldsgemm_matmul(l, x, M, y, ws, ws_bytes, s);
+    case FAM_DQGEMM:
+        return launch_dqgemm_matmul(l, x, M, y, ws, ws_bytes, s);
     default:
         return launch_general_matmul(l, x, M, y, s);
     }
@@ -158,6 +164,9 @@ size_t hqq_matmul_workspace_bytes(const hqq_linear *l, int64_t M)
     const size_t d = ldsgemm_supported(l, M) ? ldsgemm_workspace_bytes(l, M) : 0;
     if (d > b)
         b = d;
+    const size_t e = dqgemm_preferred(l, M) ? dqgemm_workspace_bytes(l, M) : 0; // (forced on fewer rows it needs 2 * N * K bytes)
+    if (e > b)
+        b = e;
     return align256(a > b ? a : b);
 }
 
@@ -191,7 +200,9 @@ int hqq_matmul_transpose_ex(const hqq_linear *l, const void *x_f16, int64_t M, v
         return HQQ_E_UNSUPPORTED;
     if (fam == FAM_LDS && !ldsgemm_supported(l, M))
         return HQQ_E_UNSUPPORTED;
-    if (fam < 0 || fam > FAM_LDS)
+    if (fam == FAM_DQGEMM && !dqgemm_supported(l, M))
+        return HQQ_E_UNSUPPORTED;
+    if (fam < 0 || fam > FAM_DQGEMM)
         return HQQ_E_UNSUPPORTED;
     const size_t need = family_workspace(l, M, fam);
     if (need > 0 && (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)))
@@ -272,9 +283,10 @@ int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, i
     const bool alike = w1->nbits == w3->nbits && w1->group_size == w3->group_size;
     // one fused launch where a kernel family has one for the batch; the decode kernels need no more workspace than
     // they check for themselves
-    const bool prefer_tile = tile_supported(w1, M) && tile_supported(w3, M) && !strip_gate_supported(w1, w3, M) &&
+    const bool wide = pick_family(w1, M) == FAM_DQGEMM || pick_family(w3, M) == FAM_DQGEMM; // two plain projections
+    const bool prefer_tile = !wide && tile_supported(w1, M) && tile_supported(w3, M) && !strip_gate_supported(w1, w3, M) &&
                              pick_family(w1, M) != FAM_LDS && pick_family(w3, M) != FAM_LDS;
-    if (alike && !prefer_tile && smallbatch_supported(w1, M) && smallbatch_supported(w3, M))
+    if (alike && !wide && !prefer_tile && smallbatch_supported(w1, M) && smallbatch_supported(w3, M))
         return launch_smallbatch_gate_up(w1, w3, x, M, h, workspace, workspace_bytes, s);
     if (prefer_tile && tile_gate_supported(w1, w3, M))
         return launch_tile_gate_up(w1, w3, x, M, h, workspace, workspace_bytes, s);
@@ -335,9 +347,10 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
         return launch_vec3_down(w2, a, b, M, y, mm, mm_bytes, ep, s);
     }
     // fused gate: decode batches always; wider ones only where the tile kernel does not take the shape
-    const bool prefer_tile = tile_supported(w1, M) && tile_supported(w3, M) && !strip_gate_supported(w1, w3, M) &&
+    const bool wide = pick_family(w1, M) == FAM_DQGEMM || pick_family(w3, M) == FAM_DQGEMM; // two plain projections
+    const bool prefer_tile = !wide && tile_supported(w1, M) && tile_supported(w3, M) && !strip_gate_supported(w1, w3, M) &&
                              pick_family(w1, M) != FAM_LDS && pick_family(w3, M) != FAM_LDS;
-    const bool fast13 = !prefer_tile && smallbatch_supported(w1, M) && smallbatch_supported(w3, M) && !w1->bias &&
+    const bool fast13 = !wide && !prefer_tile && smallbatch_supported(w1, M) && smallbatch_supported(w3, M) && !w1->bias &&
                         !w3->bias && w1->nbits == w3->nbits && w1->group_size == w3->group_size;
     if (fast13) {
         rc = launch_smallbatch_gate_up(w1, w3, x, M, h, mm, mm_bytes, s);

@@ -253,6 +253,11 @@ int launch_attention_decode(const f16 *q, const f16 *k, const f16 *v, const f16 
                             hipStream_t s, void *ws = nullptr, size_t ws_bytes = 0);
 int attention_parts(int64_t max_len); // blocks per head of the attention launch
 size_t attention_workspace_bytes(int64_t max_len, int n_heads, int head_dim);
+// dequant_gemm.hip: wide batches as hqq_dequantize into the workspace + one library GEMM
+bool dqgemm_supported(const hqq_linear *l, int64_t M);
+bool dqgemm_preferred(const hqq_linear *l, int64_t M);
+size_t dqgemm_workspace_bytes(const hqq_linear *l, int64_t M);
+int launch_dqgemm_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s);
 int launch_silu_mul(const f16 *a, const f16 *b, f16 *h, int64_t count, hipStream_t s);
 int launch_scale_store(const f16 *src, f16 *dst, const f16 *row_scale, int accumulate, int64_t M, int64_t N,
                        hipStream_t s);

@@ -20,7 +20,7 @@ if not os.path.exists(LIB_PATH):
 lib = ctypes.CDLL(LIB_PATH)
 
 HQQ_TABLE_F16, HQQ_TABLE_U8 = 0, 1
-FAM_GENERAL, FAM_SMALLBATCH, FAM_TILE, FAM_VEC3, FAM_LDS = 0, 1, 2, 3, 4
+FAM_GENERAL, FAM_SMALLBATCH, FAM_TILE, FAM_VEC3, FAM_LDS, FAM_DQGEMM = 0, 1, 2, 3, 4, 5
 HQQ_E_UNSUPPORTED = -6  # the library does not take the configuration (include/hqq_mi355x.h)
 
 

@@ -127,6 +127,8 @@ def matmul(desc: LinearDesc, a: torch.Tensor, family: int = -1) -> torch.Tensor:
     if M > 0:
         with _on(a.device):
             need = _lib.lib.hqq_matmul_workspace_bytes(desc.ref, M)
+            if family == _lib.FAM_DQGEMM:  # forced below the batch size it is chosen from: room for the fp16 weights
+                need = max(need, 2 * desc.N * desc.K + (1 << 20))
             ws = workspace(a.device, need)
             _lib.check(_lib.lib.hqq_matmul_transpose_ex(desc.ref, x.data_ptr(), M, c.data_ptr(), ws.data_ptr(),
                                                         ws.numel(), family, _lib.current_stream_ptr(a.device)),

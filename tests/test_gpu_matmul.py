@@ -51,7 +51,7 @@ def test_matmul_auto_family(shape, m):
     _check(layer, x)
 
 
-@pytest.mark.parametrize("family", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("family", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "w%d_%dx%d_g%d" % s[:4])
 def test_matmul_forced_family(shape, family):
     """Every family that accepts a configuration must meet the same tolerance."""
@@ -67,7 +67,7 @@ def test_matmul_forced_family(shape, family):
             ran += 1
         except _lib.HqqError as e:
             assert e.code == -6  # HQQ_E_UNSUPPORTED is the only acceptable refusal
-    if family == 0:
+    if family in (0, 5):  # the general kernel and de-quantise + library GEMM take every configuration
         assert ran == 4
     if shape[1:3] in ((1024, 1024), (512, 1024), (512, 512)) and family in (1, 2):
         # the tuned kernels must really have run here, not refused (the tile family only takes batches above 16)
@@ -417,3 +417,31 @@ def test_three_bit_single_row_kernel(shape):
     # activations forty times larger: nothing overflows on the way
     x = (rng.standard_normal((1, k)) * 40).astype(np.float16)
     _check(layer, x)
+
+
+@pytest.mark.parametrize("nbits,n,k,gs,m", [(2, 14336, 4096, 16, 512), (2, 4096, 14336, 16, 1024), (4, 4096, 4096, 64, 640),
+                                            (3, 14336, 4096, 64, 300), (2, 14336, 4096, 16, 2048)])
+def test_wide_batches_dequantize_then_library_gemm(nbits, n, k, gs, m):
+    """Hundreds of rows: the weights are de-quantised into the workspace and multiplied by the vendor library's fp16
+    GEMM (the reference's PyTorch path).  Against fp32 sums over the same de-quantised weights; with a bias; and a
+    decode-sized call on the same workspace afterwards finds its counters and slots at zero."""
+    from mixtral_offloading_amd import _lib, hip_kernels
+    desc = _full_size_layer(nbits, n, k, gs, seed=n + k + nbits + m)
+    assert _lib.lib.hqq_matmul_kernel_family(desc.ref, m) == _lib.FAM_DQGEMM
+    assert _lib.lib.hqq_matmul_kernel_family(desc.ref, 128) != _lib.FAM_DQGEMM
+    g = torch.Generator(device="cuda").manual_seed(m)
+    x = torch.randn((m, k), device="cuda", generator=g).half()
+    w = hip_kernels.dequantize(desc).float()
+    ref = x.float() @ w.t()
+    atol = 1e-3 * x.float().norm(dim=1)[:, None] * w.norm(dim=1)[None, :]
+    bound = 1e-2 * ref.abs() + atol + ref.abs() * 2.0 ** -11
+    for _ in range(2):
+        y = hip_kernels.matmul(desc, x)
+        err = (y.float() - ref).abs()
+        worst = float((err / bound).max())
+        assert worst <= 0.1, worst
+        one = hip_kernels.matmul(desc, x[:1].contiguous())  # the decode kernel, same workspace
+        assert float(((one.float() - ref[:1]).abs() / bound[:1]).max()) <= 0.1
+    # the same rows through the tile kernel: both are fp16 roundings of nearly the same fp32 sums
+    tile = hip_kernels.matmul(desc, x, family=_lib.FAM_TILE)
+    assert float(((tile.float() - y.float()).abs() / bound).max()) <= 0.1
