@@ -287,8 +287,8 @@ def survey_section(dev):
               + (f"  stream read of the same bytes {r['stream_read_same_bytes_us']:.2f} us ({r['frac_of_stream_read']:.2f})" if ceiling else ""),
               file=sys.stderr, flush=True)
 
-    shapes = [(4, 4096, 4096, 64, (1, 4, 16, 128, 512)), (4, 1024, 4096, 64, (1,)), (2, 14336, 4096, 16, (1, 4, 16, 128, 512)),
-              (2, 4096, 14336, 16, (1, 4, 16, 128, 512)), (3, 14336, 4096, 64, (1, 8, 128)), (3, 4096, 14336, 64, (1, 8, 128))]
+    shapes = [(4, 4096, 4096, 64, (1, 4, 16, 128, 512, 4096)), (4, 1024, 4096, 64, (1,)), (2, 14336, 4096, 16, (1, 4, 16, 128, 512, 4096)),
+              (2, 4096, 14336, 16, (1, 4, 16, 128, 512, 4096)), (3, 14336, 4096, 64, (1, 8, 128, 4096)), (3, 4096, 14336, 64, (1, 8, 128))]
     for nbits, n, k, gs, batches in shapes:
         wbytes = (n * k * nbits // 8 if nbits != 3 else ((n + 9) // 10) * k * 4) + 2 * (n * k // gs) + 4 * (n * k // gs // META_GROUP) + 4
         nl = max(2, min(16, (320 << 20) // wbytes + 1))
@@ -331,6 +331,16 @@ def survey_section(dev):
             fam = lib.hqq_matmul_kernel_family(layers[0].ref, m)
             add(f"matmul {tag} M={m} (family {fam})", timed(f, 48 if m <= 16 else 16), wbytes + 2 * m * (n + k), 2.0 * m * n * k,
                 ceiling=m <= 16)
+            if fam == _lib.FAM_DQGEMM:
+                # the matrix-core tile kernel, forced, beside the de-quantise + library GEMM form chosen for wide batches
+
+                def t(i):
+                    rc = lib.hqq_matmul_transpose_ex(layers[i % nl].ref, x.data_ptr(), m, y.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                     _lib.FAM_TILE, stream.cuda_stream)
+                    if rc != 0:
+                        raise _lib.HqqError(rc, "hqq_matmul_transpose_ex")
+
+                add(f"matmul {tag} M={m} (family {_lib.FAM_TILE}, forced)", timed(t, 8), wbytes + 2 * m * (n + k), 2.0 * m * n * k)
             if (nbits, n, m) in ((2, 14336, 128), (2, 14336, 512)) and fam != _lib.FAM_LDS:
                 # the other prefill kernel (weights de-quantised into LDS), forced, beside the one the library picks
 

@@ -37,14 +37,15 @@ bool dqgemm_supported(const hqq_linear *l, int64_t M)
     return M >= 1 && M < (1ll << 31) && l->N < (1ll << 31) && l->K < (1ll << 31);
 }
 
-// From how many rows on the de-quantise-then-GEMM form is the faster one (measured at Mixtral shapes: 2- and 4-bit
-// layers with N >= K from 512 rows, with K > N from 1024, 3-bit layers, whose tile kernel pays for a rewrite of the
-// codes as well, from 256); small layers stay with the matrix-core kernels, whose launch is cheaper than two.
+// From how many rows on the de-quantise-then-GEMM form is the faster one (measured at Mixtral shapes, cache-cold: 2-
+// and 4-bit layers with N >= K break even near 512 rows, with K > N near 1024, 3-bit layers, whose tile kernel pays
+// for a rewrite of the codes as well, near 256; the thresholds sit a little above); small layers stay with the
+// matrix-core kernels, whose launch is cheaper than two.
 bool dqgemm_preferred(const hqq_linear *l, int64_t M)
 {
     if (!dqgemm_supported(l, M) || l->N * l->K < (1ll << 22))
         return false;
-    const int64_t from = l->nbits == 3 ? 256 : (l->N >= l->K ? 512 : 1024);
+    const int64_t from = l->nbits == 3 ? 320 : (l->N >= l->K ? 640 : 1280);
     return M >= from;
 }
 

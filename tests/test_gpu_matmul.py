@@ -419,8 +419,8 @@ def test_three_bit_single_row_kernel(shape):
     _check(layer, x)
 
 
-@pytest.mark.parametrize("nbits,n,k,gs,m", [(2, 14336, 4096, 16, 512), (2, 4096, 14336, 16, 1024), (4, 4096, 4096, 64, 640),
-                                            (3, 14336, 4096, 64, 300), (2, 14336, 4096, 16, 2048)])
+@pytest.mark.parametrize("nbits,n,k,gs,m", [(2, 14336, 4096, 16, 640), (2, 4096, 14336, 16, 1280), (4, 4096, 4096, 64, 700),
+                                            (3, 14336, 4096, 64, 320), (2, 14336, 4096, 16, 2048)])
 def test_wide_batches_dequantize_then_library_gemm(nbits, n, k, gs, m):
     """Hundreds of rows: the weights are de-quantised into the workspace and multiplied by the vendor library's fp16
     GEMM (the reference's PyTorch path).  Against fp32 sums over the same de-quantised weights; with a bias; and a
