@@ -364,7 +364,7 @@ def prefill_section(dev, tokens=128, repeats=3):
 
     cfg = bm.mixtral_config()
     off = bm.OffloadConfig(main_size=32 * 8, offload_size=0, buffer_size=4, offload_per_layer=0)
-    model = bm.build_model(dev, bm.default_quant_config(), off, model_config=cfg, seed=0, max_positions=1024)
+    model = bm.build_model(dev, bm.default_quant_config(), off, model_config=cfg, seed=0, max_positions=max(1024, tokens + 2))
     gen = torch.Generator(device=dev).manual_seed(1)
     prompt = torch.randint(0, cfg.vocab_size, (tokens,), device=dev, generator=gen)
     cache = model.new_cache(tokens + 2)
