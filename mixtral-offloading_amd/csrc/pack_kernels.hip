@@ -3,6 +3,7 @@
 // These are streaming byte kernels, bounded by HBM: every thread moves whole
 // 32-bit or 128-bit words and does its bit work on four codes per lane-op.
 // Layouts follow the reference packers (src/packing.py:10-97).
+#include "gemv_parts.hpp"
 #include "hqq_common.hpp"
 #include "table_reader.hpp"
 
@@ -344,9 +345,113 @@ void dequantize_words_s(int sk, int zk, int grid, const hqq_linear *l, const Tab
         dequantize_words_z<NBITS, 3>(zk, grid, l, sc, zr, si, zi, G, w, s);
 }
 
+// The same values again for HQQ's two table layouts (8-bit scale with per-column meta and 8-bit zero with one meta
+// pair, or both fp16) when K and the meta columns are multiples of 16: one thread owns sixteen columns of one packed
+// row, so every access is 128 bits wide (codes, tables, meta, and two stores per weight row) and a wave writes 2 KB
+// of a weight row at a time.
+template <int NBITS, int SKIND, int ZKIND>
+__global__ __launch_bounds__(kThreads) void dequantize_chunks_kernel(const uint8_t *__restrict__ codes, const uint8_t *__restrict__ sq,
+                                                                     const uint8_t *__restrict__ zq, const f16 *__restrict__ s_ms,
+                                                                     const f16 *__restrict__ s_mz, const f16 *__restrict__ z_ms,
+                                                                     const f16 *__restrict__ z_mz, uint32_t s_cols, uint32_t s_inv,
+                                                                     uint32_t N, uint32_t K, uint32_t G, f16 *__restrict__ w)
+{
+    using namespace gemv;
+    constexpr uint32_t F = NBITS == 3 ? 10 : 8 / NBITS;
+    const uint32_t prows = (N + F - 1) / F, kchunks = K / 16;
+    const uint32_t idx = blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= prows * kchunks)
+        return;
+    const uint32_t p = idx / kchunks, k0 = (idx - p * kchunks) * 16;
+    u32x4 cw[NBITS == 3 ? 4 : 1];
+    if constexpr (NBITS == 3) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            cw[q] = gload<u32x4>(reinterpret_cast<const uint32_t *>(codes) + (size_t)p * K + k0 + 4 * q);
+    } else {
+        cw[0] = gload<u32x4>(codes + (size_t)p * K + k0);
+    }
+    f16x2 zms = {(f16)1.0f, (f16)1.0f}, zmz = {(f16)0.0f, (f16)0.0f};
+    if constexpr (ZKIND == TK_U8_SCALAR)
+        zms = (f16x2){z_ms[0], z_ms[0]}, zmz = (f16x2){z_mz[0], z_mz[0]};
+    const f16x2 k1024 = {(f16)1024.0f, (f16)1024.0f};
+    uint32_t j = (F * p) % G;
+#pragma unroll
+    for (uint32_t i = 0; i < F; ++i) {
+        const uint32_t n = F * p + i;
+        if (n >= N)
+            break;
+        const uint32_t ce = j * K + k0;
+        uint32_t cm = 0;
+        if constexpr (SKIND == TK_U8_COLS) {
+            cm = ce - __umulhi(ce, s_inv) * s_cols; // ce mod cols; the quotient estimate is at most 2 short
+            cm -= cm >= s_cols ? s_cols : 0;
+            cm -= cm >= s_cols ? s_cols : 0;
+        }
+        Raw16<SKIND> rs;
+        Raw16<ZKIND> rz;
+        load16<SKIND>(rs, sq, s_ms, s_mz, ce, cm);
+        load16<ZKIND>(rz, zq, nullptr, nullptr, ce, 0);
+        f16x2 sv[8], zv[8];
+        decode16<SKIND>(rs, zms, zmz, sv);
+        decode16<ZKIND>(rz, zms, zmz, zv);
+        u32x4 o[2];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint32_t b; // the codes of row n at columns 4q .. 4q+3, one per byte
+            if constexpr (NBITS == 3) {
+                const uint32_t sh = 3 * (9 - i);
+                b = ((cw[q].x >> sh) & 7u) | (((cw[q].y >> sh) & 7u) << 8) | (((cw[q].z >> sh) & 7u) << 16) |
+                    (((cw[q].w >> sh) & 7u) << 24);
+            } else {
+                b = (cw[0][q] >> (NBITS * (F - 1 - i))) & ((1u << NBITS) - 1) * 0x01010101u;
+            }
+            const f16x2 q01 = as_h2(__builtin_amdgcn_perm(0x64646464u, b, 0x04010400u)) - k1024;
+            const f16x2 q23 = as_h2(__builtin_amdgcn_perm(0x64646464u, b, 0x04030402u)) - k1024;
+            const f16x2 d01 = q01 - zv[2 * q], d23 = q23 - zv[2 * q + 1]; // first rounding
+            o[q >> 1][2 * (q & 1)] = as_u32(d01 * sv[2 * q]);             // second rounding
+            o[q >> 1][2 * (q & 1) + 1] = as_u32(d23 * sv[2 * q + 1]);
+        }
+        u32x4 *dst = reinterpret_cast<u32x4 *>(w + (size_t)n * K + k0);
+        dst[0] = o[0], dst[1] = o[1]; // plain stores: the GEMM that follows finds much of the layer in the last-level cache
+        if (++j == G)
+            j = 0;
+    }
+}
+
+template <int NBITS> bool dequantize_chunks(const hqq_linear *l, f16 *w, hipStream_t s)
+{
+    const int sk = gemv::table_kind(l->scale), zk = gemv::table_kind(l->zero);
+    const bool q8 = sk == gemv::TK_U8_COLS && zk == gemv::TK_U8_SCALAR, f16t = sk == gemv::TK_F16 && zk == gemv::TK_F16;
+    const int64_t G = l->N / l->group_size;
+    constexpr int F = NBITS == 3 ? 10 : 8 / NBITS;
+    const int64_t prows = (l->N + F - 1) / F, threads = prows * (l->K / 16);
+    if ((!q8 && !f16t) || l->K % 16 != 0 || G * l->K >= (1ll << 32) || threads >= (1ll << 31) ||
+        !aligned16(w) || !aligned16(l->codes) || !aligned16(l->scale.data) || !aligned16(l->zero.data))
+        return false;
+    if (q8 && (l->scale.meta_cols % 16 != 0 || !aligned16(l->scale.meta_scale) || !aligned16(l->scale.meta_zero)))
+        return false;
+    const uint32_t s_cols = q8 ? (uint32_t)l->scale.meta_cols : 1;
+    const uint32_t s_inv = (uint32_t)(0xFFFFFFFFull / (uint64_t)s_cols);
+    const unsigned grid = (unsigned)((threads + kThreads - 1) / kThreads);
+    const uint8_t *codes = static_cast<const uint8_t *>(l->codes), *sq = static_cast<const uint8_t *>(l->scale.data),
+                  *zq = static_cast<const uint8_t *>(l->zero.data);
+    const f16 *sms = static_cast<const f16 *>(l->scale.meta_scale), *smz = static_cast<const f16 *>(l->scale.meta_zero),
+              *zms = static_cast<const f16 *>(l->zero.meta_scale), *zmz = static_cast<const f16 *>(l->zero.meta_zero);
+    if (q8)
+        dequantize_chunks_kernel<NBITS, gemv::TK_U8_COLS, gemv::TK_U8_SCALAR><<<grid, kThreads, 0, s>>>(
+            codes, sq, zq, sms, smz, zms, zmz, s_cols, s_inv, (uint32_t)l->N, (uint32_t)l->K, (uint32_t)G, w);
+    else
+        dequantize_chunks_kernel<NBITS, gemv::TK_F16, gemv::TK_F16><<<grid, kThreads, 0, s>>>(
+            codes, sq, zq, sms, smz, zms, zmz, s_cols, s_inv, (uint32_t)l->N, (uint32_t)l->K, (uint32_t)G, w);
+    return true;
+}
+
 // launches the word-path de-quantiser when the layer fits it; false = the caller takes the per-element kernel
 bool dequantize_words(const hqq_linear *l, const Table &sc, const Table &zr, f16 *w, hipStream_t s)
 {
+    if (l->nbits == 4 ? dequantize_chunks<4>(l, w, s) : l->nbits == 2 ? dequantize_chunks<2>(l, w, s) : dequantize_chunks<3>(l, w, s))
+        return true;
     const int sk = words_table_kind(l->scale), zk = words_table_kind(l->zero);
     const int64_t G = l->N / l->group_size;
     const int F = l->nbits == 3 ? 10 : 8 / l->nbits;
