@@ -68,6 +68,42 @@ def test_argument_errors_without_touching_the_gpu():
                                       None) == -3  # more than 16 experts
 
 
+def test_kernel_family_by_batch_size_is_host_logic():
+    """Which family a call would use is decided on the host from the descriptor alone (fake, aligned addresses): the
+    decode kernels up to 16 rows, the tile kernel above, de-quantise + library GEMM from a few hundred rows on, and
+    the workspace query grows by the fp16 weights exactly there."""
+    from mixtral_offloading_amd import _lib
+    lib = _lib.lib
+
+    def layer(nbits, n, k, gs):
+        lin = _lib.HqqLinear()
+        lin.nbits, lin.group_size, lin.N, lin.K, lin.codes = nbits, gs, n, k, 1 << 30
+        g = n // gs
+        for t, at in ((lin.scale, 2 << 30), (lin.zero, 3 << 30)):
+            t.data, t.kind = at, _lib.HQQ_TABLE_U8
+        lin.scale.meta_cols, lin.scale.meta_scale, lin.scale.meta_zero = g * k // 128, 4 << 30, 5 << 30
+        lin.zero.meta_cols, lin.zero.meta_scale, lin.zero.meta_zero = 1, 6 << 30, 7 << 30
+        return lin
+
+    def fam(lin, m):
+        return lib.hqq_matmul_kernel_family(ctypes.byref(lin), m)
+
+    up, down, q, up3 = layer(2, 14336, 4096, 16), layer(2, 4096, 14336, 16), layer(4, 4096, 4096, 64), layer(3, 14336, 4096, 64)
+    for lin in (up, down, q):
+        assert [fam(lin, m) for m in (1, 2, 3, 16)] == [_lib.FAM_SMALLBATCH] * 4
+        assert [fam(lin, m) for m in (17, 128, 512)] == [_lib.FAM_TILE] * 3
+        assert fam(lin, 4096) == _lib.FAM_DQGEMM
+    assert [fam(up, 639), fam(up, 640)] == [_lib.FAM_TILE, _lib.FAM_DQGEMM]
+    assert [fam(down, 1279), fam(down, 1280)] == [_lib.FAM_TILE, _lib.FAM_DQGEMM]
+    assert [fam(up3, m) for m in (1, 4, 8, 128, 319, 320)] == [_lib.FAM_VEC3, _lib.FAM_VEC3, _lib.FAM_LDS, _lib.FAM_TILE,
+                                                               _lib.FAM_TILE, _lib.FAM_DQGEMM]
+    small = layer(4, 1024, 1024, 64)  # a million weights: never worth two launches
+    assert fam(small, 4096) == _lib.FAM_TILE
+    fp16_weights = 2 * 14336 * 4096
+    assert lib.hqq_matmul_workspace_bytes(ctypes.byref(up), 639) < fp16_weights
+    assert lib.hqq_matmul_workspace_bytes(ctypes.byref(up), 640) >= fp16_weights
+
+
 def _plan(lib, c, experts):
     n = len(experts)
     arr = (ctypes.c_int32 * n)(*experts)
