@@ -54,6 +54,8 @@ static int pick_family(const hqq_linear *l, int64_t M)
         return FAM_DQGEMM;
     if (strip_supported(l, M)) // decode batches: part of the small-batch family
         return FAM_SMALLBATCH;
+    if (l->nbits == 3 && M <= 8 && vec3_supported(l, M)) // up to eight rows in one pass over the 3-bit words
+        return FAM_VEC3;
     if (l->nbits == 3 && M >= 5 && M <= kSmallBatchMax && ldsgemm_supported(l, M)) // 3-bit words read as they are stored
         return FAM_LDS;
     if (l->nbits == 3 && tile_supported(l, M)) // wider batches: 3-bit codes rewritten as 4-bit ones, then the tile kernel
@@ -285,7 +287,8 @@ int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, i
     // they check for themselves
     const bool wide = pick_family(w1, M) == FAM_DQGEMM || pick_family(w3, M) == FAM_DQGEMM; // two plain projections
     const bool prefer_tile = !wide && tile_supported(w1, M) && tile_supported(w3, M) && !strip_gate_supported(w1, w3, M) &&
-                             pick_family(w1, M) != FAM_LDS && pick_family(w3, M) != FAM_LDS;
+                             pick_family(w1, M) != FAM_LDS && pick_family(w3, M) != FAM_LDS && pick_family(w1, M) != FAM_VEC3 &&
+                             pick_family(w3, M) != FAM_VEC3;
     if (alike && !wide && !prefer_tile && smallbatch_supported(w1, M) && smallbatch_supported(w3, M))
         return launch_smallbatch_gate_up(w1, w3, x, M, h, workspace, workspace_bytes, s);
     if (prefer_tile && tile_gate_supported(w1, w3, M))
@@ -344,12 +347,13 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
         SmallBatchEpilogue ep;
         ep.row_scale = (const f16 *)row_scale_f16;
         ep.accumulate = accumulate;
-        return launch_vec3_down(w2, a, b, M, y, mm, mm_bytes, ep, s);
+        return launch_vec3_down(w2, a, b, M, y, mm, mm_bytes, ep, s, h);
     }
     // fused gate: decode batches always; wider ones only where the tile kernel does not take the shape
     const bool wide = pick_family(w1, M) == FAM_DQGEMM || pick_family(w3, M) == FAM_DQGEMM; // two plain projections
     const bool prefer_tile = !wide && tile_supported(w1, M) && tile_supported(w3, M) && !strip_gate_supported(w1, w3, M) &&
-                             pick_family(w1, M) != FAM_LDS && pick_family(w3, M) != FAM_LDS;
+                             pick_family(w1, M) != FAM_LDS && pick_family(w3, M) != FAM_LDS && pick_family(w1, M) != FAM_VEC3 &&
+                             pick_family(w3, M) != FAM_VEC3;
     const bool fast13 = !wide && !prefer_tile && smallbatch_supported(w1, M) && smallbatch_supported(w3, M) && !w1->bias &&
                         !w3->bias && w1->nbits == w3->nbits && w1->group_size == w3->group_size;
     if (fast13) {
@@ -495,7 +499,7 @@ int hqq_expert_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, const hqq
         SmallBatchEpilogue ep3;
         ep3.row_scale = (const f16 *)row_scale_f16;
         ep3.accumulate = accumulate;
-        return launch_vec3_down(w2, a, b, M, (f16 *)y_f16, p, mm_bytes, ep3, s, &down3);
+        return launch_vec3_down(w2, a, b, M, (f16 *)y_f16, p, mm_bytes, ep3, s, h, &down3);
     }
     const StripIndex gate = {device_table, expert_index, 3, 0}, down = {device_table, expert_index, 3, 2};
     if ((rc = launch_strip_gate_up(w1, w3, (const f16 *)x_f16, M, h, p, mm_bytes, s, &gate)) != HQQ_OK)
@@ -565,11 +569,11 @@ int hqq_expert_pair_ffn_indexed(const hqq_linear *w1, const hqq_linear *w2, cons
         SmallBatchEpilogue ep;
         ep.row_scale = (const f16 *)row_scale_f16;
         ep.accumulate = accumulate;
-        if ((rc = launch_vec3_down(w2, h0, h0 + ls, 1, (f16 *)y_f16, p, mm_bytes, ep, s, &down)) != HQQ_OK)
+        if ((rc = launch_vec3_down(w2, h0, h0 + ls, 1, (f16 *)y_f16, p, mm_bytes, ep, s, nullptr, &down)) != HQQ_OK)
             return rc;
         ep.row_scale = (const f16 *)row_scale_f16 + 1;
         ep.accumulate = 1;
-        return launch_vec3_down(w2, h0 + 2 * ls, h0 + 3 * ls, 1, (f16 *)y_f16, p, mm_bytes, ep, s, &down1);
+        return launch_vec3_down(w2, h0 + 2 * ls, h0 + 3 * ls, 1, (f16 *)y_f16, p, mm_bytes, ep, s, nullptr, &down1);
     }
     if ((rc = launch_strip_gate_up_pair(w1, w3, (const f16 *)x_f16, h0, h1, p, mm_bytes, s, gate)) != HQQ_OK)
         return rc;

@@ -23,19 +23,19 @@
 // subnormals and of xs, the zero table's own scale and zero applied to the sums).  The codes of the slab's second
 // half are requested after the table phase, see there.
 //
-// Two batch rows: lane (t = lane >> 2, c = lane & 3) owns word row t,
-// columns 16m + 4c .. +3 for m = 0..15: four consecutive lanes read 64 consecutive bytes, sixteen 128-bit loads per
-// lane, all in flight at once.  A pair of words gives, per field, one v_perm (the two bytes that hold the field, of
-// both words) and one v_and: the field masked in place is the fp16 subnormal q * 2^(rel - 24), which v_dot2_f32_f16
-// multiplies exactly and accumulates in fp32.  The table phase (lane l owns columns 4l .. 4l+3 of all ten rows)
-// leaves xs in LDS; the zero term is a dot product per table row, summed over the wave at the end.
+// Two to eight batch rows: the same layout with the batch rows in the instruction's columns, column = phase + 2 *
+// half + 4 * (batch row within its group of four), one or two such groups.  Every set of fields then has a B operand
+// of its own per group: 32 * s of the lane's field from LDS times the lane's own x[m, k] read straight from memory,
+// placed in the lane's half.  The zero term is two more matrix instructions per step and group, 32 * s * z of the
+// ten table rows (from LDS) against x.  One pass over the words serves all rows; the accumulators of eight rows fill
+// the register file, so a wave of such a pass takes a single slab.  Wider batches run as passes of eight.
 //
-// The waves of a block split K (one or two slabs each; with two batch rows the second slab's loads are in flight
+// The waves of a block split K (one or two slabs each; with one batch row the second slab's loads are in flight
 // while the first slab's codes are worked on); when K needs several blocks (or the window count alone would leave
 // most of the chip idle) the blocks of a tile add their results into one 64-bit fixed-point accumulation slot per
 // output with a returning device-scope atomic, and the block whose addition completes a slot writes that output
 // (launches with more outputs than there are slots store fp32 partial sums instead, and the block that arrives
-// last at the tile's counter adds them in a fixed order).  Batches above two rows run as passes of two.
+// last at the tile's counter adds them in a fixed order).
 //
 // A launch may hold up to four layers of one shape (a one-dimensional grid over layer, window, row block and K
 // block, see the kernel): the two projections of an
@@ -46,6 +46,7 @@
 // and add into y.
 #include "gemv_parts.hpp"
 #include "hqq_common.hpp"
+#include <type_traits>
 
 namespace hqq {
 using namespace gemv;
@@ -103,17 +104,7 @@ struct W3Params {
 #define W3_STAMP(i)
 #endif
 
-// field i of a word: bit offset 3*(9-i); the two bytes B, B+1 that hold it, its offset inside them
-__host__ __device__ constexpr int w3_bit(int i) { return 3 * (9 - i); }
-__host__ __device__ constexpr uint32_t w3_sel(int i)
-{
-    const uint32_t B = (uint32_t)w3_bit(i) >> 3;
-    const uint32_t lo0 = B, hi0 = B < 3 ? B + 1 : 0x0cu, lo1 = 4 + B, hi1 = B < 3 ? 4 + B + 1 : 0x0cu;
-    return (hi1 << 24) | (lo1 << 16) | (hi0 << 8) | lo0;
-}
-__host__ __device__ constexpr uint32_t w3_mask(int i) { return (7u << (w3_bit(i) & 7)) * 0x00010001u; }
-__host__ __device__ constexpr float w3_unscale(int i) { return (float)(1u << (24 - (w3_bit(i) & 7))) / kXsScale; }
-
+// Field i of a word lies at bit 3 * (9 - i).
 // One batch row: a word's ten fields go to the matrix cores as five sets of two, one field in each 16-bit half of an
 // operand register (so a register is one column, and the B operand keeps the halves apart with zeros).  Sets 0 and 1
 // are the word itself; the others are two byte gathers, which put the fields that straddle a 16-bit boundary into
@@ -144,13 +135,6 @@ __device__ __forceinline__ float w3_set_unscale(int set, int half)
     return __builtin_bit_cast(float, (uint32_t)(127 + 24 - 5 - o) << 23); // 2^(24 - o) / 32
 }
 
-__device__ __forceinline__ float quad_sum(float v)
-{
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
-    return v;
-}
-
 // silu in fp32 with one rounding, then the fp16 product: the two roundings of the elementwise kernel
 __device__ __forceinline__ f16 silu_mul(f16 a, f16 b)
 {
@@ -172,12 +156,21 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
     if (p.stamps)
         st[9] = __builtin_readcyclecounter();
 #endif
-    // xs of each wave's slab.  Two batch rows: [4-column group][batch row][table row][4 halves]; one batch row:
-    // [16-column step][4-column piece][table row][4 halves]
-    __shared__ __attribute__((aligned(16))) f16 xs_raw[kW3Waves * 64 * MT * 10 * 4];
-    __shared__ __attribute__((aligned(16))) f16 h_lds[MT == 1 && XMODE ? kW3Waves : 1][kSlab]; // silu(xa) * xb of the slab
-    __shared__ float zt_lds[kW3Waves][10];
-    __shared__ float red_lds[kW3Waves][16][10][MT];
+    // xs of each wave's slab: [32-column step][4-column piece][table row][4 halves].  (A batch: 32 * s in that layout,
+    // 32 * s * z beside it, and a wave's results in the place of its own tables once it has read them for the last
+    // time.)
+    static_assert(MT == 1 || MT == 4 || MT == 8, "one row, or one or two column groups of four rows");
+    constexpr bool kBatch = MT >= 4;
+    __shared__ __attribute__((aligned(16))) f16 xs_raw[kW3Waves * 64 * 10 * 4];
+    __shared__ __attribute__((aligned(16))) f16 zs_raw[kBatch ? kW3Waves * 64 * 10 * 4 : 8];
+    __shared__ __attribute__((aligned(16))) f16 h_lds[XMODE ? kW3Waves : 1][kSlab]; // silu(xa) * xb of the slab
+    __shared__ float zt_lds[kW3Waves][10][kBatch ? MT : 1];
+    __shared__ float red_raw[kBatch ? 1 : kW3Waves * 16 * 10 * MT];
+    // the results of wave w: [word row 16][field 10][batch row MT]; a batch wave puts them where its own tables were
+    constexpr int kRedStride = kBatch ? 64 * 10 * 4 / 2 : 16 * 10 * MT; // floats
+    static_assert(kRedStride >= 16 * 10 * MT, "the results fit where the tables were");
+    float *const red_base = kBatch ? reinterpret_cast<float *>(xs_raw) : red_raw;
+    auto red_lds = [&](int w) __attribute__((always_inline)) { return reinterpret_cast<float(*)[10][MT]>(red_base + w * kRedStride); };
     __shared__ int ticket_lds;
 
     // Every kernel argument the prologue reads is fetched here, in one batch: read where they are used, they come in
@@ -277,7 +270,7 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
             for (int i = 0; i < 5; ++i)
                 acc[g8][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
         if (lane < 10)
-            zt_lds[wave][lane] = 0.f;
+            zt_lds[wave][lane][0] = 0.f;
         // the masks in scalar registers: as literals they double the size of the instructions that use them
         uint32_t mk[5] = {w3_set_mask(0), w3_set_mask(1), w3_set_mask(2), w3_set_mask(3), w3_set_mask(4)};
         asm volatile("" : "+s"(mk[0]), "+s"(mk[1]), "+s"(mk[2]), "+s"(mk[3]), "+s"(mk[4]));
@@ -419,7 +412,7 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
                 }
                 z = row16_sum(z);
                 if (qT == 0 && (r < 2 || third_ok))
-                    zt_lds[wave][f] += z;
+                    zt_lds[wave][f][0] += z;
             }
             wave_sync();
         };
@@ -499,7 +492,7 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
 
         // wave result
         wave_sync();
-        const float zt = zt_lds[wave][fcol] * (1.0f / kXsScale), zt4 = zt_lds[wave][fcol4] * (1.0f / kXsScale);
+        const float zt = zt_lds[wave][fcol][0] * (1.0f / kXsScale), zt4 = zt_lds[wave][fcol4][0] * (1.0f / kXsScale);
         const float un = w3_set_unscale(set, half), un4 = w3_set_unscale(4, half);
         // Accumulator element v of a lane is tile row 4 * (lane >> 4) + v = 2 * word row + phase; a column keeps the
         // rows of its own phase, and the two phases of a word row are lanes one apart.
@@ -524,202 +517,264 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
                 v4 += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v4), 0xB1, 0xF, 0xF, true));
                 const int row = 8 * g8 + 2 * gk + e;
                 if (phi == 0) {
-                    red_lds[wave][row][fcol][0] = fmaf(v, un, -zt);
+                    red_lds(wave)[row][fcol][0] = fmaf(v, un, -zt);
                     if (set == 0)
-                        red_lds[wave][row][fcol4][0] = fmaf(v4, un4, -zt4);
+                        red_lds(wave)[row][fcol4][0] = fmaf(v4, un4, -zt4);
                 }
             }
         }
     } else {
-    // ---------------------------------------------------------------- two batch rows: dot products on the vector units
-    auto xs_lds = reinterpret_cast<f16(*)[64][MT][10][4]>(xs_raw);
-    const int t = lane >> 2, c = lane & 3;
-    const int wr = w0 + p.P * (16 * rb + t); // this lane's word row
-    const bool row_ok = wr < p.NW;
-    const uint32_t code_base = (uint32_t)(row_ok ? wr : w0) * (uint32_t)K * 4u + (uint32_t)(16 * c);
-    float acc[10][MT], zacc[10][MT];
+        // ------------------------------------------------------------ three to eight batch rows on the matrix cores
+        // The single row's layout with the batch rows in the columns: column = phase + 2 * half + 4 * (batch row within
+        // its group of four), so every set of fields has a B operand of its own per group, 32 * s[k] (from LDS) times
+        // the lane's own x[m, k] (read straight from memory) placed in the lane's half.  The zero term is two more
+        // matrix instructions per step and group: A = 32 * s * z of table rows 0..7, then 8 and 9 (rows = table row x
+        // phase, two columns per register as they lie in LDS), B = x as loaded.
+        static_assert(XMODE == 0, "batches take their activations as they are");
+        constexpr int BG = MT / 4;
+        constexpr int SK = Q8 ? TK_U8_COLS : TK_F16, ZK = Q8 ? TK_U8_SCALAR : TK_F16;
+        f16 *const s_w = xs_raw + wave * (16 * 4 * 10 * 4); // [step][piece][table row][4 halves]
+        f16 *const z_w = zs_raw + wave * (16 * 4 * 10 * 4);
+        const int rho = (lane & 15) >> 1, phi = lane & 1, gk = lane >> 4;
+        uint32_t code_at[2];
 #pragma unroll
-    for (int i = 0; i < 10; ++i)
-#pragma unroll
-        for (int m = 0; m < MT; ++m)
-            acc[i][m] = zacc[i][m] = 0.f;
-
-    // What a slab's table phase reads: tables, their per-column meta, the zero table's whole-tensor meta, x.
-    struct Tab {
-        uint32_t sraw[10][2], zraw[10][2];
-        u32x2 msr[10], mzr[10];
-        u32x2 xr[MT], xg[XMODE ? MT : 1];
-        uint32_t zms_raw, zmz_raw;
-    };
-    // Every load of a slab is issued in the order the arithmetic needs them (loads retire in issue order): zero meta,
-    // tables, x, then the codes.  Whole-tensor meta of the zero table: the address is the same in every lane but
-    // written so that the compiler does not see it (lane >> 6 is zero): a load it knows to be uniform is moved to
-    // scalar registers at once, which waits for it before any weight load has been issued.
-    auto load_tab = [&](Tab &T, int slab) __attribute__((always_inline)) {
-        const uint32_t k0 = (uint32_t)slab * kSlab;
-        T.zms_raw = T.zmz_raw = 0;
-        if constexpr (Q8) {
-            T.zms_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_ms) + (lane >> 6));
-            T.zmz_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_mz) + (lane >> 6));
+        for (int g8 = 0; g8 < 2; ++g8) {
+            const int wr = w0 + p.P * (16 * rb + 8 * g8 + rho);
+            code_at[g8] = (uint32_t)(wr < p.NW ? wr : w0) * (uint32_t)K * 4u + (uint32_t)(32 * gk + 16 * phi);
         }
+        const int half = (lane >> 1) & 1, mrow = (lane & 15) >> 2;
+        const uint32_t piece_at = (uint32_t)((2 * gk + phi) * 10 * 8);
+        const uint32_t sel_a = half ? 0x01000c0cu : 0x0c0c0100u, sel_b = half ? 0x03020c0cu : 0x0c0c0302u;
+        const uint32_t z_at0 = piece_at + (uint32_t)(rho * 8), z_at1 = piece_at + (uint32_t)((8 + (rho & 1)) * 8);
+        uint32_t x_at[BG]; // halves
 #pragma unroll
-        for (int i = 0; i < 10; ++i) {
-            uint32_t j = j0 + (uint32_t)i; // (10*w0 + i) mod G; G >= 10
+        for (int bg = 0; bg < BG; ++bg) {
+            const int m = 4 * bg + mrow;
+            x_at[bg] = (uint32_t)(m < M ? m : 0) * (uint32_t)K + (uint32_t)(8 * gk + 4 * phi);
+        }
+        const int qT = lane & 15;
+        const bool third_ok = lane < 32;
+        uint32_t trow_at[3];
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            const int f = r < 2 ? 4 * r + (lane >> 4) : 8 + ((lane >> 4) & 1);
+            uint32_t j = j0 + (uint32_t)f;
             j -= j >= (uint32_t)p.G ? (uint32_t)p.G : 0u;
-            const uint32_t ce = j * (uint32_t)K + k0 + (uint32_t)(4 * lane);
-            if constexpr (Q8) {
-                T.sraw[i][0] = gload<uint32_t>(R.sq + ce);
-                T.zraw[i][0] = gload<uint32_t>(R.zq + ce);
-                uint32_t cm = ce - __umulhi(ce, R.s_inv) * R.s_cols; // ce mod cols; the quotient estimate is at most 2 short
-                cm -= cm >= R.s_cols ? R.s_cols : 0;
-                cm -= cm >= R.s_cols ? R.s_cols : 0;
-                T.msr[i] = gload<u32x2>(R.s_ms + cm);
-                T.mzr[i] = gload<u32x2>(R.s_mz + cm);
-            } else {
-                const u32x2 a = gload<u32x2>(reinterpret_cast<const f16 *>(R.sq) + ce);
-                const u32x2 b = gload<u32x2>(reinterpret_cast<const f16 *>(R.zq) + ce);
-                T.sraw[i][0] = a.x, T.sraw[i][1] = a.y, T.zraw[i][0] = b.x, T.zraw[i][1] = b.y;
+            trow_at[r] = j * (uint32_t)K + (uint32_t)(16 * qT);
+        }
+        f32x4 acc[2][5][BG], accz[2][BG];
+#pragma unroll
+        for (int bg = 0; bg < BG; ++bg) {
+#pragma unroll
+            for (int g8 = 0; g8 < 2; ++g8) {
+                accz[g8][bg] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int i = 0; i < 5; ++i)
+                    acc[g8][i][bg] = (f32x4){0.f, 0.f, 0.f, 0.f};
             }
         }
+        uint32_t mk[5] = {w3_set_mask(0), w3_set_mask(1), w3_set_mask(2), w3_set_mask(3), w3_set_mask(4)};
+        asm volatile("" : "+s"(mk[0]), "+s"(mk[1]), "+s"(mk[2]), "+s"(mk[3]), "+s"(mk[4]));
+
+        if (wave < p.KS) {
+#pragma clang loop unroll(disable)
+            for (int slab = slab_lo; slab < slab_lo + S && slab < slab_hi; ++slab) {
+                const uint32_t k0 = (uint32_t)slab * kSlab;
+                W3_STAMP(1);
+                // every load of the slab in the order of use: tables, activations, codes
+                uint32_t zms_raw = 0, zmz_raw = 0;
+                if constexpr (Q8) {
+                    zms_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_ms) + (lane >> 6));
+                    zmz_raw = gload<uint16_t>(reinterpret_cast<const uint16_t *>(R.z_mz) + (lane >> 6));
+                }
+                Raw16<SK> rs[3];
+                Raw16<ZK> rz[3];
 #pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            const uint32_t at = (uint32_t)((m < M ? m : 0) * K) + k0 + (uint32_t)(4 * lane);
-            if constexpr (XMODE) {
-                T.xg[m] = gload<u32x2>(p.xa + (int64_t)layer * p.x_lstride + at);
-                T.xr[m] = gload<u32x2>(p.xb + (int64_t)layer * p.x_lstride + at);
-            } else {
-                T.xr[m] = gload<u32x2>(p.x + at);
+                for (int r = 0; r < 3; ++r) {
+                    const uint32_t ce = trow_at[r] + k0;
+                    uint32_t cm = 0;
+                    if constexpr (Q8) {
+                        cm = ce - __umulhi(ce, R.s_inv) * R.s_cols;
+                        cm -= cm >= R.s_cols ? R.s_cols : 0;
+                        cm -= cm >= R.s_cols ? R.s_cols : 0;
+                    }
+                    if (Q8 && p.meta4) {
+                        rs[r].q = gload<u32x4>(R.sq + ce);
+#pragma unroll
+                        for (int pc = 0; pc < 4; ++pc) {
+                            uint32_t c4 = cm + 4u * pc;
+                            c4 -= c4 >= R.s_cols ? R.s_cols : 0;
+                            const u32x2 a = gload<u32x2>(R.s_ms + c4), b = gload<u32x2>(R.s_mz + c4);
+                            rs[r].ms[pc >> 1][2 * (pc & 1)] = a.x, rs[r].ms[pc >> 1][2 * (pc & 1) + 1] = a.y;
+                            rs[r].mz[pc >> 1][2 * (pc & 1)] = b.x, rs[r].mz[pc >> 1][2 * (pc & 1) + 1] = b.y;
+                        }
+                    } else {
+                        load16<SK>(rs[r], R.sq, R.s_ms, R.s_mz, ce, cm);
+                    }
+                    load16<ZK>(rz[r], R.zq, nullptr, nullptr, ce, 0);
+                }
+                u32x2 xw[BG][8];
+#pragma unroll
+                for (int bg = 0; bg < BG; ++bg)
+#pragma unroll
+                    for (int s = 0; s < kW3Early; ++s)
+                        xw[bg][s] = gload<u32x2>(p.x + (x_at[bg] + k0 + (uint32_t)(32 * s)));
+                u32x4 cw[8][2];
+#pragma unroll
+                for (int s = 0; s < kW3Early; ++s)
+#pragma unroll
+                    for (int g8 = 0; g8 < 2; ++g8)
+                        cw[s][g8] = gload<u32x4>(R.codes + (code_at[g8] + 4u * k0 + (uint32_t)(128 * s)));
+                __builtin_amdgcn_sched_barrier(0);
+                W3_STAMP(2);
+
+                // table phase: 32 * s and 32 * s * z of the ten table rows into LDS
+                if constexpr (Q8)
+                    asm volatile("" : "+v"(zms_raw), "+v"(zmz_raw));
+                const f16x2 k32 = {(f16)kXsScale, (f16)kXsScale};
+                const f16x2 zms = as_h2(zms_raw * 0x10001u), zmz = as_h2(zmz_raw * 0x10001u);
+#pragma unroll
+                for (int r = 0; r < 3; ++r) {
+                    const int f = r < 2 ? 4 * r + (lane >> 4) : 8 + ((lane >> 4) & 1);
+                    f16x2 sv[8], zv[8];
+                    decode16<SK>(rs[r], k32, k32, sv);
+                    decode16<ZK>(rz[r], zms, zmz, zv);
+                    uint32_t a[8], b[8];
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) {
+                        const f16x2 v = sv[t] * k32;
+                        a[t] = as_u32(v), b[t] = as_u32(zv[t] * v);
+                    }
+                    if (r < 2 || third_ok) {
+#pragma unroll
+                        for (int pi = 0; pi < 4; ++pi) {
+                            *reinterpret_cast<u32x2 *>(s_w + ((qT * 4 + pi) * 10 + f) * 4) = (u32x2){a[2 * pi], a[2 * pi + 1]};
+                            *reinterpret_cast<u32x2 *>(z_w + ((qT * 4 + pi) * 10 + f) * 4) = (u32x2){b[2 * pi], b[2 * pi + 1]};
+                        }
+                    }
+                }
+                wave_sync();
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int bg = 0; bg < BG; ++bg) // the second half of the activations and codes, into the registers the tables have left
+#pragma unroll
+                    for (int s = kW3Early; s < 8; ++s)
+                        xw[bg][s] = gload<u32x2>(p.x + (x_at[bg] + k0 + (uint32_t)(32 * s)));
+#pragma unroll
+                for (int s = kW3Early; s < 8; ++s)
+#pragma unroll
+                    for (int g8 = 0; g8 < 2; ++g8)
+                        cw[s][g8] = gload<u32x4>(R.codes + (code_at[g8] + 4u * k0 + (uint32_t)(128 * s)));
+                __builtin_amdgcn_sched_barrier(0);
+                W3_STAMP(3);
+
+                // code phase, a step is 32 columns
+#pragma unroll
+                for (int s = 0; s < 8; ++s) {
+#ifdef HQQ_TUNING_BUILD
+                    if (s == 1 || s == 2 || s == 4 || s == 6) {
+                        asm volatile("" ::"v"(cw[s][0]));
+                        W3_STAMP(s == 1 ? 4 : s == 2 ? 5 : s == 4 ? 6 : 7);
+                    }
+#endif
+                    const char *s_step = reinterpret_cast<const char *>(s_w) + s * 640, *z_step = reinterpret_cast<const char *>(z_w) + s * 640;
+                    const u32x2 za = *reinterpret_cast<const u32x2 *>(z_step + z_at0), zb = *reinterpret_cast<const u32x2 *>(z_step + z_at1);
+                    const f16x8 Az0 = __builtin_bit_cast(f16x8, (u32x4){za.x, za.y, 0u, 0u});
+                    const f16x8 Az1 = __builtin_bit_cast(f16x8, (u32x4){zb.x, zb.y, 0u, 0u});
+#pragma unroll
+                    for (int bg = 0; bg < BG; ++bg) {
+                        const f16x8 Bx = __builtin_bit_cast(f16x8, (u32x4){xw[bg][s].x, xw[bg][s].y, 0u, 0u});
+                        accz[0][bg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Az0, Bx, accz[0][bg], 0, 0, 0);
+                        accz[1][bg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Az1, Bx, accz[1][bg], 0, 0, 0);
+                    }
+                    u32x4 wa[2];
+#pragma unroll
+                    for (int set = 0; set < 5; ++set) {
+                        const u32x2 sb = *reinterpret_cast<const u32x2 *>(s_step + piece_at + w3_set_field(set, half) * 8);
+                        f16x8 B[BG];
+#pragma unroll
+                        for (int bg = 0; bg < BG; ++bg) {
+                            const uint32_t p01 = as_u32(as_h2(sb.x) * as_h2(xw[bg][s].x)), p23 = as_u32(as_h2(sb.y) * as_h2(xw[bg][s].y));
+                            B[bg] = __builtin_bit_cast(f16x8, (u32x4){__builtin_amdgcn_perm(0u, p01, sel_a), __builtin_amdgcn_perm(0u, p01, sel_b),
+                                                                     __builtin_amdgcn_perm(0u, p23, sel_a), __builtin_amdgcn_perm(0u, p23, sel_b)});
+                        }
+#pragma unroll
+                        for (int g8 = 0; g8 < 2; ++g8) {
+                            const u32x4 w = cw[s][g8];
+                            u32x4 src = w;
+                            if (set == 2) {
+#pragma unroll
+                                for (int j = 0; j < 4; ++j)
+                                    src[j] = __builtin_amdgcn_perm(w[j], w[j], kW3GatherB);
+                            } else if (set == 3) {
+#pragma unroll
+                                for (int j = 0; j < 4; ++j)
+                                    wa[g8][j] = __builtin_amdgcn_perm(w[j], w[j], kW3GatherA);
+                                src = wa[g8];
+                            } else if (set == 4) {
+                                src = wa[g8];
+                            }
+                            const f16x8 A = __builtin_bit_cast(f16x8, src & mk[set]);
+#pragma unroll
+                            for (int bg = 0; bg < BG; ++bg)
+                                acc[g8][set][bg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B[bg], acc[g8][set][bg], 0, 0, 0);
+                        }
+                    }
+                }
+                wave_sync();
+                W3_STAMP(8);
             }
         }
-    };
-    auto load_codes = [&](u32x4(&cw)[16], int slab) __attribute__((always_inline)) {
+
+        // wave result.  Element v of an accumulator is tile row 4 * (lane >> 4) + v = 2 * (row of the group) + phase; a
+        // column keeps the rows of its own phase, and the two phases are lanes one apart: the lanes of phase 0 add
+        // their neighbour's odd element to their own even one.  First the zero terms, through LDS to the columns of
+        // their table row; then the results, in the place of the wave's own tables.
+        auto both = [&](const f32x4 &c, int e) __attribute__((always_inline)) {
+            return c[2 * e] + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, (float)c[2 * e + 1]), 0xB1, 0xF, 0xF, true));
+        };
+        float zv[BG][2][2];
 #pragma unroll
-        for (int m = 0; m < 16; ++m)
-            cw[m] = gload<u32x4>(R.codes + (code_base + 4u * ((uint32_t)slab * kSlab) + (uint32_t)(64 * m)));
-    };
-    // table phase: xs into LDS, zero term accumulated
-    auto table_phase = [&](Tab &T) __attribute__((always_inline)) {
-        if constexpr (Q8) // the meta values become opaque here, so no use of them is hoisted above the loads
-            asm volatile("" : "+v"(T.zms_raw), "+v"(T.zmz_raw));
-        if constexpr (XMODE) {
+        for (int bg = 0; bg < BG; ++bg)
 #pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                const f16x2 a01 = as_h2(T.xg[m].x), a23 = as_h2(T.xg[m].y), b01 = as_h2(T.xr[m].x), b23 = as_h2(T.xr[m].y);
-                T.xr[m].x = as_u32((f16x2){silu_mul(a01.x, b01.x), silu_mul(a01.y, b01.y)});
-                T.xr[m].y = as_u32((f16x2){silu_mul(a23.x, b23.x), silu_mul(a23.y, b23.y)});
-            }
-        }
-        const f16x2 k1024 = {(f16)1024.0f, (f16)1024.0f};
-        const f16x2 k32 = {(f16)kXsScale, (f16)kXsScale};
-        const f16x2 zms = as_h2(T.zms_raw * 0x10001u), zmz = as_h2(T.zmz_raw * 0x10001u);
+            for (int e = 0; e < 2; ++e)
+                zv[bg][e][0] = both(accz[0][bg], e), zv[bg][e][1] = both(accz[1][bg], e);
+        if (phi == 0 && half == 0) {
 #pragma unroll
-        for (int i = 0; i < 10; ++i) {
-            f16x2 s01, s23, z01, z23;
-            if constexpr (Q8) {
-                // bytes -> fp16 exactly (0x6400 | b is 1024 + b), then fp16(fp16(q - mz) * ms) as the reference does
-                const f16x2 q01 = as_h2(__builtin_amdgcn_perm(0x64646464u, T.sraw[i][0], 0x04010400u)) - k1024;
-                const f16x2 q23 = as_h2(__builtin_amdgcn_perm(0x64646464u, T.sraw[i][0], 0x04030402u)) - k1024;
-                s01 = (q01 - as_h2(T.mzr[i].x)) * as_h2(T.msr[i].x);
-                s23 = (q23 - as_h2(T.mzr[i].y)) * as_h2(T.msr[i].y);
-                const f16x2 y01 = as_h2(__builtin_amdgcn_perm(0x64646464u, T.zraw[i][0], 0x04010400u)) - k1024;
-                const f16x2 y23 = as_h2(__builtin_amdgcn_perm(0x64646464u, T.zraw[i][0], 0x04030402u)) - k1024;
-                z01 = (y01 - zmz) * zms;
-                z23 = (y23 - zmz) * zms;
-            } else {
-                s01 = as_h2(T.sraw[i][0]), s23 = as_h2(T.sraw[i][1]);
-                z01 = as_h2(T.zraw[i][0]), z23 = as_h2(T.zraw[i][1]);
-            }
-            s01 = s01 * k32, s23 = s23 * k32;
+            for (int bg = 0; bg < BG; ++bg)
 #pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                const f16x2 a01 = s01 * as_h2(T.xr[m].x), a23 = s23 * as_h2(T.xr[m].y);
-                zacc[i][m] = __builtin_amdgcn_fdot2(z01, a01, zacc[i][m], false);
-                zacc[i][m] = __builtin_amdgcn_fdot2(z23, a23, zacc[i][m], false);
-                *reinterpret_cast<f16x4 *>(&xs_lds[wave][lane][m][i][0]) = (f16x4){a01.x, a01.y, a23.x, a23.y};
-            }
+                for (int e = 0; e < 2; ++e) {
+                    zt_lds[wave][2 * gk + e][4 * bg + mrow] = zv[bg][e][0] * (1.0f / kXsScale);
+                    if (gk == 0)
+                        zt_lds[wave][8 + e][4 * bg + mrow] = zv[bg][e][1] * (1.0f / kXsScale);
+                }
         }
         wave_sync();
-    };
-    // codes: per pair of words and field, perm + and + dot2
-    auto code_phase = [&](const u32x4(&cw)[16]) __attribute__((always_inline)) {
+        float (*const red_w)[10][MT] = red_lds(wave);
 #pragma unroll
-        for (int m = 0; m < 16; ++m) {
-            const int q = 4 * m + c;
-            u32x2 X[MT][10];
+        for (int set = 0; set < 5; ++set) {
+            const int f = w3_set_field(set, half);
+            const float un = w3_set_unscale(set, half);
+            float out[BG][2][2];
 #pragma unroll
-            for (int mm = 0; mm < MT; ++mm) {
-                const u32x4 *src = reinterpret_cast<const u32x4 *>(&xs_lds[wave][q][mm][0][0]);
+            for (int bg = 0; bg < BG; ++bg) {
+                const float zt = zt_lds[wave][f][4 * bg + mrow];
 #pragma unroll
-                for (int v = 0; v < 5; ++v) {
-                    const u32x4 d = src[v];
-                    X[mm][2 * v] = (u32x2){d.x, d.y};
-                    X[mm][2 * v + 1] = (u32x2){d.z, d.w};
-                }
+                for (int g8 = 0; g8 < 2; ++g8)
+#pragma unroll
+                    for (int e = 0; e < 2; ++e)
+                        out[bg][g8][e] = fmaf(both(acc[g8][set][bg], e), un, -zt);
             }
+            if (phi == 0) {
 #pragma unroll
-            for (int i = 0; i < 10; ++i) {
-                const uint32_t pa = __builtin_amdgcn_perm(cw[m].y, cw[m].x, w3_sel(i)) & w3_mask(i);
-                const uint32_t pb = __builtin_amdgcn_perm(cw[m].w, cw[m].z, w3_sel(i)) & w3_mask(i);
+                for (int bg = 0; bg < BG; ++bg)
 #pragma unroll
-                for (int mm = 0; mm < MT; ++mm) {
-                    acc[i][mm] = __builtin_amdgcn_fdot2(as_h2(pa), as_h2(X[mm][i].x), acc[i][mm], false);
-                    acc[i][mm] = __builtin_amdgcn_fdot2(as_h2(pb), as_h2(X[mm][i].y), acc[i][mm], false);
-                }
+                    for (int g8 = 0; g8 < 2; ++g8)
+#pragma unroll
+                        for (int e = 0; e < 2; ++e)
+                            red_w[8 * g8 + 2 * gk + e][f][4 * bg + mrow] = out[bg][g8][e];
             }
         }
-        wave_sync();
-    };
-
-    if (wave < p.KS && slab_lo < slab_hi) {
-        Tab T;
-        u32x4 c0[16];
-        load_tab(T, slab_lo);
-        load_codes(c0, slab_lo);
-        __builtin_amdgcn_sched_barrier(0); // nothing below moves above the loads, no load sinks into the arithmetic
-        table_phase(T);
-        if constexpr (S == 2 && MT == 1) {
-            // The second slab's loads go out before the first slab's codes are worked on (unconditionally: a wave
-            // whose second slab lies past its range re-reads the first and skips the arithmetic), its tables into
-            // the registers the first slab's table phase has just released.
-            const bool two = slab_lo + 1 < slab_hi;
-            const int s1 = two ? slab_lo + 1 : slab_lo;
-            u32x4 c1[16];
-            load_tab(T, s1);
-            load_codes(c1, s1);
-            __builtin_amdgcn_sched_barrier(0);
-            code_phase(c0);
-            if (two) {
-                table_phase(T);
-                code_phase(c1);
-            }
-        } else if constexpr (S == 2) {
-            // two batch rows leave no registers for a second set of codes: one slab after the other
-            code_phase(c0);
-            const bool two = slab_lo + 1 < slab_hi;
-            const int s1 = two ? slab_lo + 1 : slab_lo;
-            load_tab(T, s1);
-            load_codes(c0, s1);
-            __builtin_amdgcn_sched_barrier(0);
-            if (two) {
-                table_phase(T);
-                code_phase(c0);
-            }
-        } else {
-            code_phase(c0);
-        }
-    }
-
-    // ---------------------------------------------------------------- wave result: sum over the column lanes, zero term removed
-#pragma unroll
-    for (int i = 0; i < 10; ++i) {
-#pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            const float a = quad_sum(acc[i][m]) * w3_unscale(i);
-            const float z = wave_sum(zacc[i][m]) * (1.0f / kXsScale);
-            if (c == 0)
-                red_lds[wave][t][i][m] = a - z;
-        }
-    }
     }
 #ifdef HQQ_TUNING_BUILD
     if (p.stamps)
@@ -757,7 +812,7 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
         const int m_t = u % MT, i_t = (u / MT) % 10, t_t = u / (10 * MT);
         float v = 0.f;
         for (int w = 0; w < p.KS; ++w) // fixed order
-            v += red_lds[w][t_t][i_t][m_t];
+            v += red_lds(w)[t_t][i_t][m_t];
         const int64_t wr_t = (int64_t)w0 + (int64_t)p.P * (16 * rb + t_t);
         const int64_t n = 10 * wr_t + i_t;
         if (m_t >= M || wr_t >= p.NW || n >= p.N)
@@ -856,18 +911,20 @@ bool make_plan(const hqq_linear *l, int64_t M, int NL, W3Plan &pl)
     pl.RB = (rows + 15) / 16;
     pl.NS = (int)(l->K / kSlab);
     // blocks along K: enough that the windows cover the chip, and at most 16 slabs (8 waves x 2) per block
-    int BK = (pl.NS + kW3Waves * kW3S - 1) / (kW3Waves * kW3S);
+    // (five to eight batch rows in a pass: the accumulators of every row leave no registers for a second slab's tables)
+    const int per_block = M >= 5 ? kW3Waves : kW3Waves * kW3S;
+    int BK = (pl.NS + per_block - 1) / per_block;
     while ((int64_t)pl.P * pl.RB * NL * BK < 200 && BK < pl.NS)
         ++BK;
     const bool tune = tuning_int("HQQ_W3_K", (int)l->K) == (int)l->K;
     if (tune)
         BK = tuning_int("HQQ_W3_BK", BK);
-    if (BK < 1 || BK > pl.NS || (pl.NS + BK - 1) / BK > kW3Waves * kW3S)
+    if (BK < 1 || BK > pl.NS || (pl.NS + BK - 1) / BK > per_block)
         return false;
     pl.SB = (pl.NS + BK - 1) / BK;
     pl.BK = (pl.NS + pl.SB - 1) / pl.SB;
     pl.S = pl.SB > kW3Waves ? kW3S : 1;
-    if (tune)
+    if (tune && M < 5)
         pl.S = tuning_int("HQQ_W3_S", pl.S) == 2 ? 2 : pl.S;
     pl.KS = (pl.SB + pl.S - 1) / pl.S;
     if ((int64_t)pl.P * NL > 65535 || pl.RB > 65535 || (int64_t)pl.P * pl.RB * NL * sizeof(int) > kTileCounterBytes)
@@ -900,23 +957,32 @@ struct W3Job {
 
 template <int MT, bool Q8, int S> void launch_slabs(const W3Params &p, bool fused, dim3 grid, hipStream_t s)
 {
-    if (fused)
-        gemv_w3_kernel<MT, Q8, 1, S><<<grid, dim3(kW3Waves * 64), 0, s>>>(p);
-    else
-        gemv_w3_kernel<MT, Q8, 0, S><<<grid, dim3(kW3Waves * 64), 0, s>>>(p);
+    if constexpr (MT == 1) {
+        if (fused) {
+            gemv_w3_kernel<MT, Q8, 1, S><<<grid, dim3(kW3Waves * 64), 0, s>>>(p);
+            return;
+        }
+    }
+    gemv_w3_kernel<MT, Q8, 0, S><<<grid, dim3(kW3Waves * 64), 0, s>>>(p); // (a batch is never fused)
 }
 
 template <int MT, bool Q8> void launch_xmode(const W3Params &p, bool fused, dim3 grid, hipStream_t s)
 {
-    if (p.S == 2)
-        launch_slabs<MT, Q8, 2>(p, fused, grid, s);
-    else
-        launch_slabs<MT, Q8, 1>(p, fused, grid, s);
+    if constexpr (MT <= 4) {
+        if (p.S == 2) {
+            launch_slabs<MT, Q8, 2>(p, fused, grid, s);
+            return;
+        }
+    }
+    launch_slabs<MT, Q8, 1>(p, fused, grid, s); // (the plan of five to eight rows has one slab per wave)
 }
 
-size_t job_workspace_bytes(const W3Plan &pl, const hqq_linear *l, int NL)
+// batch rows of one pass over the weights
+int rows_per_pass(int64_t M) { return M >= 2 ? 8 : 1; }
+
+size_t job_workspace_bytes(const W3Plan &pl, const hqq_linear *l, int NL, int rows)
 {
-    return kHeadBytes + (pl.BK > 1 ? (size_t)NL * pl.BK * 2 * (size_t)l->N * sizeof(float) : 0);
+    return kHeadBytes + (pl.BK > 1 ? (size_t)NL * pl.BK * rows * (size_t)l->N * sizeof(float) : 0);
 }
 
 int run_job(const W3Job &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
@@ -936,7 +1002,10 @@ int run_job(const W3Job &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
     for (int i = 0; i < (j.ix ? 1 : j.NL); ++i)
         if (j.layers[i]->bias && (j.NL > 1 || j.ix))
             return HQQ_E_UNSUPPORTED; // the bias is not part of a record
-    if (pl.BK > 1 && (!ws || ws_bytes < job_workspace_bytes(pl, l, j.NL)))
+    if (fused && M != 1)
+        return HQQ_E_UNSUPPORTED; // silu(xa) * xb is built in the loads of the single-row kernel only
+    const int rows = rows_per_pass(M);
+    if (pl.BK > 1 && (!ws || ws_bytes < job_workspace_bytes(pl, l, j.NL, rows)))
         return HQQ_E_WORKSPACE;
     if (fused ? ((reinterpret_cast<uintptr_t>(j.xa) | reinterpret_cast<uintptr_t>(j.xb)) & 7u) != 0
               : (reinterpret_cast<uintptr_t>(j.x) & 15u) != 0)
@@ -955,12 +1024,12 @@ int run_job(const W3Job &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
     p.counter = static_cast<int *>(ws);
     p.part = pl.BK > 1 ? reinterpret_cast<float *>(static_cast<char *>(ws) + kHeadBytes) : nullptr;
     if (pl.BK > 1 && pl.BK * (j.pair ? 2 : 1) <= 14 &&
-        (size_t)(j.pair ? 1 : j.NL) * (size_t)l->N * 2 * sizeof(unsigned long long) <= kSlotBytes)
+        (size_t)(j.pair ? 1 : j.NL) * (size_t)l->N * (M <= 4 ? (M == 1 ? 1 : 4) : rows) * sizeof(unsigned long long) <= kSlotBytes)
         p.slots = reinterpret_cast<unsigned long long *>(static_cast<char *>(ws) + kCounterBytes);
     if (j.pair && (!p.slots || M != 1 || j.NL != 2 || !fused || !j.ep.row_scale))
         return HQQ_E_UNSUPPORTED; // the shared slots are what joins the two experts
     p.pair = j.pair, p.x_lstride = j.x_lstride;
-    p.part_lstride = (int64_t)pl.BK * 2 * l->N;
+    p.part_lstride = (int64_t)pl.BK * rows * l->N;
     p.y_lstride = j.y_lstride;
     p.accumulate = j.ep.accumulate;
     p.meta4 = pl.q8 && l->scale.meta_cols % 16 != 0;
@@ -987,25 +1056,27 @@ int run_job(const W3Job &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
                 break;
             }
     }
-    for (int64_t m0 = 0; m0 < M; m0 += 2) { // passes of two batch rows; later passes find the weights in the caches
-        const int mb = M - m0 >= 2 ? 2 : 1;
+    // passes of eight batch rows; later passes find the weights in the caches
+    for (int64_t m0 = 0; m0 < M; m0 += rows) {
+        const int mb = (int)(M - m0 >= rows ? rows : M - m0);
         if (fused)
             p.xa = j.xa + m0 * l->K, p.xb = j.xb + m0 * l->K;
         else
             p.x = j.x + m0 * l->K;
         p.y = j.y + m0 * l->N, p.M = mb;
         p.row_scale = j.ep.row_scale ? j.ep.row_scale + m0 : nullptr;
-        if (mb == 1) {
+        auto launch = [&](auto mt) {
             if (pl.q8)
-                launch_xmode<1, true>(p, fused, grid, s);
+                launch_xmode<decltype(mt)::value, true>(p, fused, grid, s);
             else
-                launch_xmode<1, false>(p, fused, grid, s);
-        } else {
-            if (pl.q8)
-                launch_xmode<2, true>(p, fused, grid, s);
-            else
-                launch_xmode<2, false>(p, fused, grid, s);
-        }
+                launch_xmode<decltype(mt)::value, false>(p, fused, grid, s);
+        };
+        if (mb > 4)
+            launch(std::integral_constant<int, 8>());
+        else if (mb >= 2)
+            launch(std::integral_constant<int, 4>());
+        else
+            launch(std::integral_constant<int, 1>());
         int rc = launch_status();
         if (rc != HQQ_OK)
             return rc;
@@ -1026,7 +1097,7 @@ size_t vec3_workspace_bytes(const hqq_linear *l, int64_t M)
     W3Plan pl;
     if (!make_plan(l, M, 1, pl))
         return 0;
-    return job_workspace_bytes(pl, l, 1);
+    return job_workspace_bytes(pl, l, 1, rows_per_pass(M));
 }
 
 int launch_vec3_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s)
@@ -1050,12 +1121,12 @@ size_t vec3_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2, int6
     W3Plan a, b;
     if (!make_plan(w1, M, 2 * n_experts, a) || !make_plan(w2, M, 1, b))
         return 0;
-    size_t need = job_workspace_bytes(a, w1, 2 * n_experts);
-    const size_t gb = job_workspace_bytes(b, w2, 1);
+    size_t need = job_workspace_bytes(a, w1, 2 * n_experts, rows_per_pass(M));
+    const size_t gb = job_workspace_bytes(b, w2, 1, rows_per_pass(M));
     need = gb > need ? gb : need;
     W3Plan c;
     if (n_experts == 2 && make_plan(w2, M, 2, c)) { // both down projections in one launch
-        const size_t gc = job_workspace_bytes(c, w2, 2);
+        const size_t gc = job_workspace_bytes(c, w2, 2, rows_per_pass(M));
         need = gc > need ? gc : need;
     }
     return need;
@@ -1071,7 +1142,7 @@ bool vec3_gate_supported(const hqq_linear *w1, const hqq_linear *w3, int64_t M)
 size_t vec3_gate_workspace_bytes(const hqq_linear *w1, int64_t M)
 {
     W3Plan pl;
-    return make_plan(w1, M, 2, pl) ? job_workspace_bytes(pl, w1, 2) : 0;
+    return make_plan(w1, M, 2, pl) ? job_workspace_bytes(pl, w1, 2, rows_per_pass(M)) : 0;
 }
 
 // ab: the gate outputs, layer l (w1 then w3 of each expert) at ab + l * ab_lstride, each (M, N)
@@ -1087,12 +1158,24 @@ int launch_vec3_gate(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, i
     return run_job(j, M, ws, ws_bytes, s);
 }
 
+// h: M * K halves of scratch.  Batches go through it (silu(a) * b in a launch of its own, then the batch kernel, which
+// takes its activations as they are); a single row builds them in the kernel's loads.
 int launch_vec3_down(const hqq_linear *w2, const f16 *a, const f16 *b, int64_t M, f16 *y, void *ws, size_t ws_bytes,
-                     const SmallBatchEpilogue &ep, hipStream_t s, const StripIndex *ix)
+                     const SmallBatchEpilogue &ep, hipStream_t s, f16 *h, const StripIndex *ix)
 {
     W3Job j = {};
     j.layers[0] = w2, j.NL = 1, j.ix = ix, j.lper = 1;
-    j.xa = a, j.xb = b, j.y = y, j.ep = ep;
+    j.y = y, j.ep = ep;
+    if (M >= 2) {
+        if (!h)
+            return HQQ_E_NULL;
+        const int rc = launch_silu_mul(a, b, h, M * w2->K, s);
+        if (rc != HQQ_OK)
+            return rc;
+        j.x = h;
+    } else {
+        j.xa = a, j.xb = b;
+    }
     return run_job(j, M, ws, ws_bytes, s);
 }
 

@@ -238,7 +238,7 @@ size_t vec3_gate_workspace_bytes(const hqq_linear *w1, int64_t M);
 int launch_vec3_gate(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *ab, int64_t ab_lstride,
                      int n_experts, void *ws, size_t ws_bytes, hipStream_t s, const StripIndex *ix = nullptr);
 int launch_vec3_down(const hqq_linear *w2, const f16 *a, const f16 *b, int64_t M, f16 *y, void *ws, size_t ws_bytes,
-                     const SmallBatchEpilogue &ep, hipStream_t s, const StripIndex *ix = nullptr);
+                     const SmallBatchEpilogue &ep, hipStream_t s, f16 *h, const StripIndex *ix = nullptr);
 int launch_router_top2(const f16 *x, const f16 *w, int n_experts, int64_t hidden, int *sel, f16 *weights, f16 *logits,
                        hipStream_t s, int64_t rows = 1);
 int launch_add_rmsnorm(f16 *x, const f16 *delta, const f16 *weight, float eps, f16 *y, int64_t hidden, hipStream_t s,

@@ -124,19 +124,20 @@ def test_shared_memory_family_edges(shape, m):
 
 
 def test_three_bit_small_batches_read_the_stored_words():
-    """Five to sixteen rows of a 3-bit layer go to the family that reads the packed words as they are, not to the one
-    that first rewrites them as 4-bit codes; wider batches and decode batches keep their kernels."""
+    """Up to sixteen rows of a 3-bit layer go to the families that read the packed words as they are (up to eight rows
+    in one pass of the vector family, nine to sixteen through shared memory), not to the one that first rewrites them
+    as 4-bit codes; wider batches keep that one."""
     from mixtral_offloading_amd import _lib
     rng = np.random.default_rng(77)
     layer, _ = o.random_layer(rng, 1024, 512, 3, 64, True, True)
     desc = desc_of(layer)
-    fam = {m: _lib.lib.hqq_matmul_kernel_family(desc.ref, m) for m in (1, 4, 5, 8, 16, 17, 64)}
-    assert fam[5] == fam[8] == fam[16] == 4
-    assert fam[1] == fam[4] == 3 and fam[17] == fam[64] == 2
-    # twenty groups: the rewrite to 4-bit codes does not take them, the stored words are read at every batch from five
+    fam = {m: _lib.lib.hqq_matmul_kernel_family(desc.ref, m) for m in (1, 4, 5, 8, 9, 16, 17, 64)}
+    assert fam[9] == fam[16] == 4
+    assert fam[1] == fam[4] == fam[5] == fam[8] == 3 and fam[17] == fam[64] == 2
+    # twenty groups: the rewrite to 4-bit codes does not take them, the stored words are read at every batch
     layer, _ = o.random_layer(rng, 1280, 512, 3, 64, True, True)
     desc = desc_of(layer)
-    assert [_lib.lib.hqq_matmul_kernel_family(desc.ref, m) for m in (4, 5, 17, 300)] == [3, 4, 4, 4]
+    assert [_lib.lib.hqq_matmul_kernel_family(desc.ref, m) for m in (4, 8, 9, 17, 300)] == [3, 3, 4, 4, 4]
 
 
 def test_bias_leading_dims_and_empty():
@@ -417,6 +418,42 @@ def test_three_bit_single_row_kernel(shape):
     # activations forty times larger: nothing overflows on the way
     x = (rng.standard_normal((1, k)) * 40).astype(np.float16)
     _check(layer, x)
+
+
+@pytest.mark.parametrize("shape", W3_SHAPES, ids=lambda s: "%dx%d_g%d_%s" % (s[:3] + ("q" if s[4] else "f16",)))
+def test_three_bit_batch_rows_on_the_matrix_cores(shape):
+    """Three to eight batch rows in one pass over the words (four or eight columns groups of the matrix instruction),
+    nine to sixteen in two passes when the family is forced; with a bias; a single row afterwards finds the
+    accumulation slots and counters clean."""
+    from mixtral_offloading_amd import _lib
+    n, k, gs, mgs, q8 = shape
+    rng = np.random.default_rng(3 * n + k)
+    layer, _ = o.random_layer(rng, n, k, 3, gs, q8, q8, meta_group_size=mgs)
+    for m in (3, 4, 5, 6, 7, 8):
+        assert _lib.lib.hqq_matmul_kernel_family(desc_of(layer).ref, m) == _lib.FAM_VEC3
+        x = rng.standard_normal((m, k)).astype(np.float16)
+        _check(layer, x, bias=rng.standard_normal(n).astype(np.float16) if m % 2 else None)
+    for m in (9, 11, 16, 1):
+        x = rng.standard_normal((m, k)).astype(np.float16)
+        _check(layer, x, family=3)
+    x = (rng.standard_normal((8, k)) * 40).astype(np.float16)  # nothing overflows on the way
+    _check(layer, x)
+
+
+def test_three_bit_batch_rows_keep_non_finite_activations_to_their_row():
+    """An infinite or NaN activation makes its own batch row non-finite and leaves the others as they were."""
+    from mixtral_offloading_amd import hip_kernels
+    rng = np.random.default_rng(5)
+    layer, _ = o.random_layer(rng, 1280, 512, 3, 64, True, True)
+    desc = desc_of(layer)
+    x = rng.standard_normal((8, 512)).astype(np.float16)
+    clean = hip_kernels.matmul(desc, to_dev(x)).cpu().numpy()
+    x[2, 17] = np.inf
+    x[5, 300] = np.nan
+    y = hip_kernels.matmul(desc, to_dev(x)).cpu().numpy()
+    assert not np.isfinite(y[2]).any() and np.isnan(y[5]).all()
+    rest = [0, 1, 3, 4, 6, 7]
+    assert np.array_equal(y[rest], clean[rest])
 
 
 @pytest.mark.parametrize("nbits,n,k,gs,m", [(2, 14336, 4096, 16, 640), (2, 4096, 14336, 16, 1280), (4, 4096, 4096, 64, 700),

@@ -95,8 +95,9 @@ def test_kernel_family_by_batch_size_is_host_logic():
         assert fam(lin, 4096) == _lib.FAM_DQGEMM
     assert [fam(up, 639), fam(up, 640)] == [_lib.FAM_TILE, _lib.FAM_DQGEMM]
     assert [fam(down, 1279), fam(down, 1280)] == [_lib.FAM_TILE, _lib.FAM_DQGEMM]
-    assert [fam(up3, m) for m in (1, 4, 8, 128, 319, 320)] == [_lib.FAM_VEC3, _lib.FAM_VEC3, _lib.FAM_LDS, _lib.FAM_TILE,
-                                                               _lib.FAM_TILE, _lib.FAM_DQGEMM]
+    assert [fam(up3, m) for m in (1, 4, 8, 9, 16, 128, 319, 320)] == [_lib.FAM_VEC3, _lib.FAM_VEC3, _lib.FAM_VEC3, _lib.FAM_LDS,
+                                                                      _lib.FAM_LDS, _lib.FAM_TILE, _lib.FAM_TILE,
+                                                                      _lib.FAM_DQGEMM]
     small = layer(4, 1024, 1024, 64)  # a million weights: never worth two launches
     assert fam(small, 4096) == _lib.FAM_TILE
     fp16_weights = 2 * 14336 * 4096
