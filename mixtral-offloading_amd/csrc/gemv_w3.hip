@@ -80,6 +80,7 @@ struct W3Params {
     int64_t part_lstride;
     int *counter;
     unsigned long long *slots; // K over several blocks: one accumulation slot per output of the launch (or null)
+    uint32_t *words;           // K over exactly two blocks: one exchange word per output instead (or null)
     int M, N, K, G, P, NW, RB;
     int NS; // K / 256
     int KS; // waves of a block that have slabs
@@ -819,6 +820,17 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
             continue;
         if (alone) {
             finish(m_t, n, v);
+        } else if (p.words) {
+            // Two blocks per output: each swaps its sum into the output's word.  The one that finds the word empty
+            // is done; the other finds its partner's sum there, adds its own (either order gives the same sum),
+            // empties the word again and writes the output.  Zero marks an empty word: a sum of +0 goes in as -0.
+            uint32_t *word = p.words + (((int64_t)layer * p.N + n) * MT + m_t);
+            const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+            const uint32_t other = __hip_atomic_exchange(word, bits ? bits : 0x80000000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (other != 0) {
+                __hip_atomic_store(word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                finish(m_t, n, v + __builtin_bit_cast(float, other));
+            }
         } else if (p.slots) {
             // the K blocks add into the output's slot; the block whose addition completes it writes the output
             // (a pair of experts shares the slots: every block's result enters with its expert's routing weight)
@@ -837,7 +849,7 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
 #ifdef HQQ_TUNING_BUILD
     write_stamps();
 #endif
-    if (alone || p.slots)
+    if (alone || p.slots || p.words)
         return;
 
     // the block that arrives last at the tile's counter adds the partial sums in a fixed order
@@ -1023,9 +1035,11 @@ int run_job(const W3Job &j, int64_t M, void *ws, size_t ws_bytes, hipStream_t s)
     p.lper = j.lper > 0 ? j.lper : 1;
     p.counter = static_cast<int *>(ws);
     p.part = pl.BK > 1 ? reinterpret_cast<float *>(static_cast<char *>(ws) + kHeadBytes) : nullptr;
-    if (pl.BK > 1 && pl.BK * (j.pair ? 2 : 1) <= 14 &&
-        (size_t)(j.pair ? 1 : j.NL) * (size_t)l->N * (M <= 4 ? (M == 1 ? 1 : 4) : rows) * sizeof(unsigned long long) <= kSlotBytes)
+    const size_t per_output = (size_t)(j.pair ? 1 : j.NL) * (size_t)l->N * (M <= 4 ? (M == 1 ? 1 : 4) : rows);
+    if (pl.BK > 1 && pl.BK * (j.pair ? 2 : 1) <= 14 && per_output * sizeof(unsigned long long) <= kSlotBytes)
         p.slots = reinterpret_cast<unsigned long long *>(static_cast<char *>(ws) + kCounterBytes);
+    else if (pl.BK == 2 && !j.pair && per_output * sizeof(uint32_t) <= kSlotBytes) // (the same memory, zero between launches)
+        p.words = reinterpret_cast<uint32_t *>(static_cast<char *>(ws) + kCounterBytes);
     if (j.pair && (!p.slots || M != 1 || j.NL != 2 || !fused || !j.ep.row_scale))
         return HQQ_E_UNSUPPORTED; // the shared slots are what joins the two experts
     p.pair = j.pair, p.x_lstride = j.x_lstride;

@@ -243,6 +243,31 @@ def test_workspace_head_is_left_at_zero():
     assert head.numel() == 576 * 1024 and not bool(head.any())
 
 
+def test_three_bit_eight_rows_exchange_words_are_left_empty():
+    """`14336x4096` 3-bit at eight rows: K is split over two blocks and the launch has more outputs than 64-bit
+    accumulation slots, so the two blocks of an output swap their sums through a 32-bit word in the same memory.
+    Twice over (the second call finds the words empty again), then an input of zeros (a sum of +0 enters its word as
+    -0: zero marks an empty word), and the head of the workspace is at zero afterwards."""
+    from mixtral_offloading_amd import _lib, hip_kernels
+    dev = torch.device("cuda:0")
+    desc = _full_size_layer(3, 14336, 4096, 64, seed=4)
+    assert _lib.lib.hqq_matmul_kernel_family(desc.ref, 8) == _lib.FAM_VEC3
+    g = torch.Generator(device="cuda").manual_seed(8)
+    x = torch.randn((8, 4096), device="cuda", generator=g).half()
+    w = hip_kernels.dequantize(desc).float()
+    ref = x.float() @ w.t()
+    bound = 1e-2 * ref.abs() + 1e-3 * x.float().norm(dim=1)[:, None] * w.norm(dim=1)[None, :] + ref.abs() * 2.0 ** -11
+    first = hip_kernels.matmul(desc, x)
+    assert float(((first.float() - ref).abs() / bound).max()) <= 0.1
+    assert torch.equal(hip_kernels.matmul(desc, x), first)
+    zeros = hip_kernels.matmul(desc, torch.zeros_like(x))
+    assert not bool(zeros.any())
+    one = hip_kernels.matmul(desc, x[:1].contiguous())  # the single-row kernel's slots in the same memory
+    assert float(((one.float() - ref[:1]).abs() / bound[:1]).max()) <= 0.1
+    torch.cuda.synchronize()
+    assert not bool(hip_kernels.workspace(dev, 1)[: 576 * 1024].any())
+
+
 def test_workspace_init_makes_a_dirty_workspace_usable():
     """A caller that brings its own workspace zeroes its head with hqq_workspace_init (a small kernel, so it may be
     recorded into a graph); the split-K launches then work on it."""
