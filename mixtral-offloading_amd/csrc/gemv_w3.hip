@@ -1136,6 +1136,11 @@ size_t vec3_ffn_workspace_bytes(const hqq_linear *w1, const hqq_linear *w2, int6
     if (!make_plan(w1, M, 2 * n_experts, a) || !make_plan(w2, M, 1, b))
         return 0;
     size_t need = job_workspace_bytes(a, w1, 2 * n_experts, rows_per_pass(M));
+    W3Plan single;
+    if (n_experts == 1 && make_plan(w1, M, 1, single)) {
+        const size_t one = job_workspace_bytes(single, w1, 1, rows_per_pass(M));
+        need = one > need ? one : need;
+    }
     const size_t gb = job_workspace_bytes(b, w2, 1, rows_per_pass(M));
     need = gb > need ? gb : need;
     W3Plan c;
@@ -1155,8 +1160,12 @@ bool vec3_gate_supported(const hqq_linear *w1, const hqq_linear *w3, int64_t M)
 
 size_t vec3_gate_workspace_bytes(const hqq_linear *w1, int64_t M)
 {
-    W3Plan pl;
-    return make_plan(w1, M, 2, pl) ? job_workspace_bytes(pl, w1, 2, rows_per_pass(M)) : 0;
+    W3Plan pl, single;
+    if (!make_plan(w1, M, 2, pl))
+        return 0;
+    const size_t both = job_workspace_bytes(pl, w1, 2, rows_per_pass(M));
+    const size_t one = make_plan(w1, M, 1, single) ? job_workspace_bytes(single, w1, 1, rows_per_pass(M)) : 0;
+    return both > one ? both : one; // (five rows and more run the projections one after the other)
 }
 
 // ab: the gate outputs, layer l (w1 then w3 of each expert) at ab + l * ab_lstride, each (M, N)
@@ -1169,6 +1178,17 @@ int launch_vec3_gate(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, i
     j.layers[0] = w1, j.layers[1] = w3, j.layers[2] = w1, j.layers[3] = w3;
     j.NL = 2 * n_experts, j.ix = ix, j.lper = 2;
     j.x = x, j.y = ab, j.y_lstride = ab_lstride;
+    W3Plan single;
+    if (M >= 5 && !ix && n_experts == 1 && make_plan(w1, M, 1, single) && make_plan(w3, M, 1, single) &&
+        ws_bytes >= job_workspace_bytes(single, w1, 1, rows_per_pass(M))) {
+        // Five rows and more, a block per compute unit: the two projections together would need two rounds of blocks and
+        // partial sums in memory; one after the other each covers the chip once and meets in the exchange words.
+        W3Job a = j, b = j;
+        a.NL = b.NL = 1;
+        b.layers[0] = w3, b.y = ab + ab_lstride;
+        const int rc = run_job(a, M, ws, ws_bytes, s);
+        return rc != HQQ_OK ? rc : run_job(b, M, ws, ws_bytes, s);
+    }
     return run_job(j, M, ws, ws_bytes, s);
 }
 
