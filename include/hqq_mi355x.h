@@ -301,8 +301,8 @@ int hqq_quantize_whole(const void *x_f32, int64_t n, int32_t nbits, void *codes_
                        void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- which kernel family a call would use (for tests and profiles): 0 general, 1 MFMA small-batch, 2 MFMA tile,
- *      3 three-bit decode kernel, 4 MFMA kernel with weights dequantised into shared memory (reads 3-bit words as
- *      they are stored), 5 batches of hundreds of rows: hqq_dequantize into the workspace, then one fp16 GEMM of the
+ *      3 three-bit decode kernel (one to eight rows in a pass over the words), 4 MFMA kernel with weights dequantised
+ *      into shared memory (reads 3-bit words as they are stored), 5 batches of hundreds of rows: hqq_dequantize into the workspace, then one fp16 GEMM of the
  *      vendor's library (rocBLAS) with fp32 accumulation, which is the reference's PyTorch path
  *      (src/custom_layers.py:95-116 and torch.matmul); hqq_matmul_workspace_bytes grows by 2 * N * K bytes there.
  *      The first such call on a device creates the library's handle (it allocates: not under stream capture).      */
