@@ -120,6 +120,19 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
                    void *y_f16, const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
                    void *stream);
 
+/* ---- the expert loop of SparseMoeWrapper.forward for several tokens (src/custom_layers.py:298-312: per expert a
+ *      where / gather / expert / scale / index_add_) over rows the caller has already grouped by expert: rows
+ *      row_start[g] .. row_start[g + 1] - 1 of x (fp16, hidden wide) go through expert g (w1[g], w2[g], w3[g]) and
+ *      y[row] = row_scale_f16[row] * expert(x[row]) (row_scale_f16 may be NULL).  row_start is a HOST array of
+ *      n_groups + 1 entries starting at 0; groups without rows may have NULL layers.  One call issues every group's
+ *      launches in order on `stream` with one workspace of hqq_expert_groups_ffn_workspace_bytes(..) bytes (the
+ *      largest group's need; head zeroed as for hqq_matmul_transpose).  Results are hqq_expert_ffn's, bit for bit. */
+size_t hqq_expert_groups_ffn_workspace_bytes(const hqq_linear *const *w1, const hqq_linear *const *w2,
+                                             const hqq_linear *const *w3, int32_t n_groups, const int64_t *row_start);
+int hqq_expert_groups_ffn(const hqq_linear *const *w1, const hqq_linear *const *w2, const hqq_linear *const *w3,
+                          int32_t n_groups, const int64_t *row_start, const void *x_f16, void *y_f16,
+                          const void *row_scale_f16, void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- hqq_expert_ffn for callers that cannot allocate or carry a workspace (code under HIP graph capture, tight
  *      serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The workspace is an
  *      array of HQQ_STATIC_SCRATCH_BYTES built into the library's device code (every GPU the library runs on holds it
@@ -222,6 +235,15 @@ int hqq_add_rmsnorm_rows(void *x_f16, const void *delta_f16, const void *weight_
                          int64_t hidden, void *stream);
 int hqq_router_top2_rows(const void *x_f16, const void *gate_w_f16, int32_t n_experts, int64_t rows, int64_t hidden,
                          int32_t *sel_out, void *weights_f16_out, void *logits_f16_out, void *stream);
+
+/* ---- the (token, slot) pairs of a prompt pass grouped by expert on the device (the reference builds an expert mask
+ *      and runs torch.where per expert, src/custom_layers.py:291-303): sel [tokens][2] and weights_f16 [tokens][2] as
+ *      hqq_router_top2_rows writes them.  Pair p = 2 * token + slot goes to the rows of expert sel[p], pairs of one
+ *      expert in the order of p.  Out: counts_out[e] rows of expert e (the only figure the host needs before it
+ *      launches the experts), and for row r of the grouped order token_of_row_out[r] (the token it came from) and
+ *      scale_of_row_f16_out[r] (its routing weight).                                                                 */
+int hqq_moe_group_pairs(const int32_t *sel, const void *weights_f16, int64_t tokens, int32_t n_experts, int32_t *counts_out,
+                        int64_t *token_of_row_out, void *scale_of_row_f16_out, void *stream);
 
 /* ---- rotary embedding and KV-cache append of `rows` new tokens at positions start .. start + rows - 1 (HF
  *      transformers' apply_rotary_pos_emb in the reference's Mixtral attention): q (rows, n_heads*head_dim) is rotated

@@ -397,6 +397,56 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
     return launch_scale_store(t, y, (const f16 *)row_scale_f16, accumulate, M, w2->N, s);
 }
 
+// ---- the experts of one MoE layer over rows already grouped by expert: hqq_expert_ffn once per group, from one call
+size_t hqq_expert_groups_ffn_workspace_bytes(const hqq_linear *const *w1, const hqq_linear *const *w2,
+                                             const hqq_linear *const *w3, int32_t n_groups, const int64_t *row_start)
+{
+    if (!w1 || !w2 || !w3 || !row_start || n_groups <= 0)
+        return 0;
+    size_t need = 0;
+    for (int g = 0; g < n_groups; ++g) {
+        const int64_t M = row_start[g + 1] - row_start[g];
+        if (M <= 0)
+            continue;
+        if (!w1[g] || !w2[g] || !w3[g])
+            return 0;
+        const size_t one = hqq_expert_ffn_workspace_bytes(w1[g], w2[g], w3[g], M);
+        if (one == 0)
+            return 0;
+        need = one > need ? one : need;
+    }
+    return need;
+}
+
+int hqq_expert_groups_ffn(const hqq_linear *const *w1, const hqq_linear *const *w2, const hqq_linear *const *w3,
+                          int32_t n_groups, const int64_t *row_start, const void *x_f16, void *y_f16,
+                          const void *row_scale_f16, void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!w1 || !w2 || !w3 || !row_start)
+        return HQQ_E_NULL;
+    if (n_groups < 0 || row_start[0] != 0)
+        return HQQ_E_SHAPE;
+    for (int g = 0; g < n_groups; ++g) {
+        if (row_start[g + 1] < row_start[g])
+            return HQQ_E_SHAPE;
+        if (row_start[g + 1] > row_start[g] && (!w1[g] || !w2[g] || !w3[g]))
+            return HQQ_E_NULL;
+    }
+    for (int g = 0; g < n_groups; ++g) {
+        const int64_t lo = row_start[g], M = row_start[g + 1] - lo;
+        if (M == 0)
+            continue;
+        const char *x = static_cast<const char *>(x_f16) + (size_t)lo * (size_t)w1[g]->K * 2;
+        char *y = static_cast<char *>(y_f16) + (size_t)lo * (size_t)w2[g]->N * 2;
+        const char *rs = row_scale_f16 ? static_cast<const char *>(row_scale_f16) + (size_t)lo * 2 : nullptr;
+        const int rc = hqq_expert_ffn(w1[g], w2[g], w3[g], x_f16 ? x : nullptr, M, y_f16 ? y : nullptr, rs, 0, workspace,
+                                      workspace_bytes, stream);
+        if (rc != HQQ_OK)
+            return rc;
+    }
+    return HQQ_OK;
+}
+
 // ---- the expert FFN for callers that cannot allocate.  The workspace is a file-scope device array; each GPU holds
 // its own copy at its own address, found once per device with hipGetSymbolAddress (the array's name is only a
 // host-side handle, never a device address).
@@ -718,6 +768,16 @@ int hqq_router_top2_rows(const void *x_f16, const void *gate_w_f16, int32_t n_ex
         return HQQ_E_NULL;
     return launch_router_top2((const f16 *)x_f16, (const f16 *)gate_w_f16, n_experts, hidden, sel_out,
                               (f16 *)weights_f16_out, (f16 *)logits_f16_out, (hipStream_t)stream, rows);
+}
+
+int hqq_moe_group_pairs(const int32_t *sel, const void *weights_f16, int64_t tokens, int32_t n_experts, int32_t *counts_out,
+                        int64_t *token_of_row_out, void *scale_of_row_f16_out, void *stream)
+{
+    if (!sel || !weights_f16 || !counts_out || !token_of_row_out || !scale_of_row_f16_out)
+        return HQQ_E_NULL;
+    return launch_moe_group_pairs(sel, (const f16 *)weights_f16, tokens, n_experts, counts_out,
+                                  reinterpret_cast<long long *>(token_of_row_out), (f16 *)scale_of_row_f16_out,
+                                  (hipStream_t)stream);
 }
 
 int hqq_rope_append_rows(void *q_f16, const void *k_f16, const void *v_f16, const void *cos_f16, const void *sin_f16,

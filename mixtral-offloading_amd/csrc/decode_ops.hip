@@ -497,6 +497,71 @@ int launch_router_top2(const f16 *x, const f16 *w, int n_experts, int64_t hidden
     return launch_status();
 }
 
+// The (token, slot) pairs of a prompt pass grouped by expert: a stable counting sort of pair p = 2 * token + slot by
+// sel[p], in one block.  Thread t owns the pairs t * chunk .. (t + 1) * chunk - 1: it counts them per expert, thread e
+// turns the counts of expert e into each thread's first place (the experts one after the other, the threads in
+// order), and every thread places its pairs in order.  Out: counts[e]; for row r of the grouped order the token it
+// came from (64-bit, as index_add_ takes it) and its routing weight.
+constexpr int kGroupThreads = 256;
+__global__ __launch_bounds__(kGroupThreads) void moe_group_pairs_kernel(const int *__restrict__ sel,
+                                                                          const f16 *__restrict__ weights, int pairs,
+                                                                          int n_experts, int *__restrict__ counts,
+                                                                          long long *__restrict__ token_of_row,
+                                                                          f16 *__restrict__ scale_of_row)
+{
+    __shared__ int first[kGroupThreads][kMaxExperts + 1]; // (+1: the threads of a wave fall into different banks)
+    __shared__ int base[kMaxExperts];
+    const int t = threadIdx.x;
+    const int chunk = (pairs + kGroupThreads - 1) / kGroupThreads;
+    const int lo = t * chunk < pairs ? t * chunk : pairs, hi = lo + chunk < pairs ? lo + chunk : pairs;
+    for (int e = 0; e < n_experts; ++e)
+        first[t][e] = 0;
+    for (int p = lo; p < hi; ++p) {
+        const int e = sel[p];
+        if (e >= 0 && e < n_experts)
+            ++first[t][e];
+    }
+    __syncthreads();
+    if (t < n_experts) {
+        int run = 0;
+        for (int u = 0; u < kGroupThreads; ++u) {
+            const int c = first[u][t];
+            first[u][t] = run;
+            run += c;
+        }
+        counts[t] = run;
+        base[t] = run;
+    }
+    __syncthreads();
+    if (t == 0) {
+        int run = 0;
+        for (int e = 0; e < n_experts; ++e) {
+            const int c = base[e];
+            base[e] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    for (int p = lo; p < hi; ++p) {
+        const int e = sel[p];
+        if (e < 0 || e >= n_experts)
+            continue;
+        const int row = base[e] + first[t][e]++;
+        token_of_row[row] = p >> 1;
+        scale_of_row[row] = weights[p];
+    }
+}
+
+int launch_moe_group_pairs(const int *sel, const f16 *weights, int64_t tokens, int n_experts, int *counts,
+                           long long *token_of_row, f16 *scale_of_row, hipStream_t s)
+{
+    if (tokens < 1 || tokens > (1 << 28) || n_experts < 2 || n_experts > kMaxExperts)
+        return HQQ_E_SHAPE;
+    moe_group_pairs_kernel<<<1, kGroupThreads, 0, s>>>(sel, weights, (int)(2 * tokens), n_experts, counts, token_of_row,
+                                                       scale_of_row);
+    return launch_status();
+}
+
 int launch_add_rmsnorm(f16 *x, const f16 *delta, const f16 *weight, float eps, f16 *y, int64_t hidden, hipStream_t s,
                        int64_t rows)
 {

@@ -241,6 +241,8 @@ int launch_vec3_down(const hqq_linear *w2, const f16 *a, const f16 *b, int64_t M
                      const SmallBatchEpilogue &ep, hipStream_t s, f16 *h, const StripIndex *ix = nullptr);
 int launch_router_top2(const f16 *x, const f16 *w, int n_experts, int64_t hidden, int *sel, f16 *weights, f16 *logits,
                        hipStream_t s, int64_t rows = 1);
+int launch_moe_group_pairs(const int *sel, const f16 *weights, int64_t tokens, int n_experts, int *counts,
+                           long long *token_of_row, f16 *scale_of_row, hipStream_t s);
 int launch_add_rmsnorm(f16 *x, const f16 *delta, const f16 *weight, float eps, f16 *y, int64_t hidden, hipStream_t s,
                        int64_t rows = 1);
 int launch_rope_append_rows(f16 *q, const f16 *k, const f16 *v, const f16 *cos_t, const f16 *sin_t, int64_t start,

@@ -56,6 +56,10 @@ _SIGNATURES = {
                                c_int, c_void_p, c_size_t, c_void_p]),
     "hqq_expert_ffn_static": (c_int, [_P(HqqLinear), _P(HqqLinear), _P(HqqLinear), c_void_p, c_int64, c_void_p, c_void_p,
                                       c_int, c_void_p]),
+    "hqq_expert_groups_ffn_workspace_bytes": (c_size_t, [c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "hqq_expert_groups_ffn": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_size_t, c_void_p]),
+    "hqq_moe_group_pairs": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "hqq_gate_up_workspace_bytes": (c_size_t, [_P(HqqLinear), _P(HqqLinear), c_int64]),
     "hqq_gate_up": (c_int, [_P(HqqLinear), _P(HqqLinear), c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hqq_expert_record_bytes": (c_size_t, []),

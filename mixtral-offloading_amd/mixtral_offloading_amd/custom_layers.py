@@ -249,6 +249,23 @@ class SparseMoeWrapper(nn.Module):
         self.gate = gate
         self.experts = expert_cache
 
+    def _resident_group(self):
+        """The layer's experts as ``hip_kernels.ExpertGroup`` when all of them are resident and none can be evicted
+        (their device modules then never move), else None."""
+        modules = self.experts.resident_group(self.layer_id) if hasattr(self.experts, "resident_group") else None
+        if modules is None or len(modules) != self.num_experts:
+            return None
+        layers = []
+        for m in modules:
+            ffn = m._expert[0] if hasattr(m, "_expert") else m
+            if getattr(ffn, "hidden_act", "silu") != "silu" or not all(hasattr(ffn, n) for n in ("w1", "w2", "w3")):
+                return None
+            layers.append((ffn.w1._desc(), ffn.w2._desc(), ffn.w3._desc()))
+        key = tuple(id(d) for t in layers for d in t)
+        if getattr(self, "_group_cache", None) is None or self._group_cache[0] != key:
+            self._group_cache = (key, hip_kernels.ExpertGroup(layers))
+        return self._group_cache[1]
+
     @torch.inference_mode()
     def forward_routed(self, hidden_states: torch.Tensor, selected: torch.Tensor, weights: torch.Tensor,
                        out: torch.Tensor, chosen=None) -> torch.Tensor:
@@ -283,6 +300,28 @@ class SparseMoeWrapper(nn.Module):
 
         tokens = hidden_states.shape[0]
         final_hidden_states = torch.zeros((tokens, hidden_dim), dtype=hidden_states.dtype, device=hidden_states.device)
+        if tokens > 1 and selected_experts.dtype == torch.int32 and routing_weights.dtype == torch.float16:
+            # Several tokens, router on the device: the (token, slot) pairs are grouped by expert there as well, the
+            # rows of every expert are gathered at once, and only then does the host wait, for the experts' row counts
+            # alone (reference :291-312 does a where / gather / index_add_ per expert).  Each token receives the same
+            # two fp16 terms in the index_add_ below, and their sum does not depend on the order.
+            counts_dev, top_x, scales = hip_kernels.moe_group_pairs(selected_experts, routing_weights, self.num_experts)
+            gathered = hidden_states.index_select(0, top_x)
+            weighted = torch.empty_like(gathered)
+            group = self._resident_group()
+            counts = counts_dev.cpu().numpy()  # the one host sync of the layer
+            starts = np.concatenate(([0], np.cumsum(counts)))
+            if group is not None:
+                # every expert of the layer is resident for good: all of them from one library call
+                hip_kernels.expert_groups_ffn(group, gathered, starts, scales, weighted)
+            else:
+                active_experts = [e for e in range(self.num_experts) if counts[e] > 0]
+                for (_layer_index, expert_idx), expert_layer in self.experts.load_experts(
+                        *((self.layer_id, expert_idx) for expert_idx in active_experts), unordered=True):
+                    lo, hi = int(starts[expert_idx]), int(starts[expert_idx + 1])
+                    expert_layer(gathered[lo:hi], out=weighted[lo:hi], row_scale=scales[lo:hi])
+            final_hidden_states.index_add_(0, top_x, weighted)
+            return final_hidden_states.reshape(batch_size, sequence_length, hidden_dim), router_logits
         sel_host = selected_experts.cpu()  # one host sync per layer: the cache is driven from the host
         if tokens == 1:
             selected = sel_host[0].tolist()

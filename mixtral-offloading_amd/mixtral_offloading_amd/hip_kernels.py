@@ -220,6 +220,43 @@ def expert_ffn(w1: LinearDesc, w2: LinearDesc, w3: LinearDesc, x: torch.Tensor, 
     return out
 
 
+class ExpertGroup:
+    """The layers of a MoE layer's experts as the pointer arrays ``expert_groups_ffn`` takes (built once per layer;
+    the descriptors are kept alive here)."""
+
+    def __init__(self, experts):
+        self.descs = [tuple(e) for e in experts]  # (w1, w2, w3) LinearDesc per expert
+        n = len(self.descs)
+        arr = ctypes.c_void_p * n
+        self.w1 = arr(*[ctypes.addressof(d[0].c) for d in self.descs])
+        self.w2 = arr(*[ctypes.addressof(d[1].c) for d in self.descs])
+        self.w3 = arr(*[ctypes.addressof(d[2].c) for d in self.descs])
+        self.n = n
+        self.K, self.N = self.descs[0][0].K, self.descs[0][1].N
+
+
+def expert_groups_ffn(group: ExpertGroup, x: torch.Tensor, row_start, row_scale: Optional[torch.Tensor],
+                      out: torch.Tensor) -> torch.Tensor:
+    """Rows ``row_start[g] .. row_start[g + 1] - 1`` of ``x`` through expert ``g``, scaled per row, into ``out``: the
+    expert loop of the reference's ``SparseMoeWrapper.forward`` (src/custom_layers.py:298-312) as one library call."""
+    assert x.dtype == torch.float16 and x.is_contiguous() and x.shape[-1] == group.K
+    rows = x.numel() // group.K
+    assert out.dtype == torch.float16 and out.is_contiguous() and out.numel() == rows * group.N
+    assert len(row_start) == group.n + 1 and int(row_start[0]) == 0 and int(row_start[-1]) == rows
+    assert row_scale is None or (row_scale.dtype == torch.float16 and row_scale.is_contiguous() and row_scale.numel() == rows)
+    starts = (ctypes.c_int64 * (group.n + 1))(*[int(v) for v in row_start])
+    with _on(x.device):
+        need = _lib.lib.hqq_expert_groups_ffn_workspace_bytes(group.w1, group.w2, group.w3, group.n, starts)
+        if rows and need == 0:
+            raise _lib.HqqError(-6, "hqq_expert_groups_ffn_workspace_bytes")
+        ws = workspace(x.device, max(need, 1))
+        _lib.check(_lib.lib.hqq_expert_groups_ffn(group.w1, group.w2, group.w3, group.n, starts, x.data_ptr(), out.data_ptr(),
+                                                  row_scale.data_ptr() if row_scale is not None else None,
+                                                  ws.data_ptr(), ws.numel(), _lib.current_stream_ptr(x.device)),
+                   "hqq_expert_groups_ffn")
+    return out
+
+
 STATIC_SCRATCH_BYTES = 16 << 20  # HQQ_STATIC_SCRATCH_BYTES of include/hqq_mi355x.h
 
 
@@ -560,6 +597,23 @@ def router_top2_rows(x: torch.Tensor, gate_weight: torch.Tensor):
                                                  sel.data_ptr(), weights.data_ptr(), logits.data_ptr(),
                                                  _lib.current_stream_ptr(x.device)), "hqq_router_top2_rows")
     return sel, weights, logits
+
+
+def moe_group_pairs(sel: torch.Tensor, weights: torch.Tensor, n_experts: int):
+    """The (token, slot) pairs of ``router_top2_rows`` grouped by expert on the device (reference
+    src/custom_layers.py:291-303): returns ``counts`` int32 (n_experts,), and per row of the grouped order the token
+    it came from (int64) and its routing weight (fp16).  Nothing here waits for the device."""
+    assert sel.dtype == torch.int32 and sel.dim() == 2 and sel.shape[1] == 2 and sel.is_contiguous()
+    assert weights.dtype == torch.float16 and weights.shape == sel.shape and weights.is_contiguous()
+    tokens = sel.shape[0]
+    counts = torch.empty((n_experts,), dtype=torch.int32, device=sel.device)
+    token_of_row = torch.empty((2 * tokens,), dtype=torch.int64, device=sel.device)
+    scale_of_row = torch.empty((2 * tokens,), dtype=torch.float16, device=sel.device)
+    with _on(sel.device):
+        _lib.check(_lib.lib.hqq_moe_group_pairs(sel.data_ptr(), weights.data_ptr(), tokens, n_experts, counts.data_ptr(),
+                                                token_of_row.data_ptr(), scale_of_row.data_ptr(),
+                                                _lib.current_stream_ptr(sel.device)), "hqq_moe_group_pairs")
+    return counts, token_of_row, scale_of_row
 
 
 def rope_append_rows(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, start: int,

@@ -456,6 +456,32 @@ def test_router_top2_rows_equals_the_one_row_call_and_the_reference_lines(rows, 
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("tokens,n_experts", [(1, 8), (2, 8), (128, 8), (129, 2), (1000, 16), (4096, 8)])
+def test_moe_group_pairs_is_a_stable_sort_by_expert(tokens, n_experts):
+    """The device-side grouping of a prompt pass's (token, slot) pairs equals the stable sort by expert the host would
+    do (numpy), including experts that received no pair; index for index (integers: exact)."""
+    import numpy as np
+    from mixtral_offloading_amd import hip_kernels
+    rng = np.random.default_rng(tokens + n_experts)
+    first = rng.integers(0, n_experts, size=tokens)
+    second = (first + rng.integers(1, n_experts, size=tokens)) % n_experts  # two different experts per token
+    if n_experts > 2:
+        first[first == 1] = 0  # expert 1 is chosen first by nobody ...
+        second[second == 1] = np.where(first[second == 1] == 2, 0, 2)  # ... and second by nobody: an empty group
+    sel = np.stack([first, second], axis=1).astype(np.int32)
+    w = rng.uniform(0.0, 1.0, size=(tokens, 2)).astype(np.float16)
+    counts, token_of_row, scale_of_row = hip_kernels.moe_group_pairs(torch.from_numpy(sel).cuda(), torch.from_numpy(w).cuda(),
+                                                                     n_experts)
+    flat = sel.reshape(-1)
+    order = np.argsort(flat, kind="stable")
+    assert np.array_equal(counts.cpu().numpy(), np.bincount(flat, minlength=n_experts))
+    assert np.array_equal(token_of_row.cpu().numpy(), order // 2)
+    assert np.array_equal(scale_of_row.cpu().numpy(), w.reshape(-1)[order])
+    if n_experts > 2:
+        assert int(counts[1]) == 0
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("T,heads,kv,hd,start,L", [(128, 32, 8, 128, 0, 130), (5, 32, 8, 128, 37, 64), (1, 4, 4, 64, 9, 10),
                                                    (17, 8, 2, 64, 0, 17)])
 def test_rope_append_rows_equals_the_torch_ops(T, heads, kv, hd, start, L):

@@ -155,3 +155,42 @@ def test_gate_up_refuses_bias_and_mismatched_layers():
     with pytest.raises(AssertionError):
         hip_kernels.gate_up(desc_of(w1), desc_of(other), x)
     assert hip_kernels.gate_up(desc_of(w1), desc_of(w3), x[:0]).shape == (0, 512)
+
+
+@pytest.mark.parametrize("nbits,hidden,ffn,gs", [(2, 512, 1792, 16), (3, 768, 1280, 64), (4, 512, 1024, 64)])
+def test_expert_groups_entry_point_equals_one_call_per_expert(nbits, hidden, ffn, gs):
+    """The expert loop of a MoE layer as one call (reference src/custom_layers.py:298-312): rows grouped by expert,
+    ragged groups (an empty one, one row, a decode batch, a prefill batch), every row scaled by its routing weight.
+    The result is that of one hqq_expert_ffn call per expert, bit for bit, and agrees with the oracle."""
+    from mixtral_offloading_amd import hip_kernels
+    rng = np.random.default_rng(nbits + hidden)
+    counts = [5, 0, 1, 40, 16, 3]
+    experts = [_ffn_case(rng, nbits, hidden, ffn, gs, True) for _ in counts]
+    descs = [tuple(desc_of(l) for l in e) for e in experts]
+    group = hip_kernels.ExpertGroup(descs)
+    starts = np.concatenate(([0], np.cumsum(counts)))
+    rows = int(starts[-1])
+    x = rng.standard_normal((rows, hidden)).astype(np.float16)
+    scale = rng.uniform(0.2, 0.8, size=rows).astype(np.float16)
+    xd, sd = to_dev(x), to_dev(scale)
+    out = torch.full((rows, hidden), 7.0, dtype=torch.float16, device="cuda")
+    hip_kernels.expert_groups_ffn(group, xd, starts, sd, out)
+    each = torch.empty_like(out)
+    for g, (w1, w2, w3) in enumerate(descs):
+        lo, hi = int(starts[g]), int(starts[g + 1])
+        if hi > lo:
+            hip_kernels.expert_ffn(w1, w2, w3, xd[lo:hi], out=each[lo:hi], row_scale=sd[lo:hi])
+    assert torch.equal(out, each)
+    # without routing weights: against the oracle as well
+    hip_kernels.expert_groups_ffn(group, xd, starts, None, out)
+    got = out.cpu().numpy()
+    for g, (w1, w2, w3) in enumerate(experts):
+        lo, hi = int(starts[g]), int(starts[g + 1])
+        if hi == lo:
+            continue
+        hip_kernels.expert_ffn(descs[g][0], descs[g][1], descs[g][2], xd[lo:hi], out=each[lo:hi])
+        assert_matmul_close(got[lo:hi], o.expert_ffn(x[lo:hi], w1, w2, w3), _tolerance(x[lo:hi], w1, w2, w3), rtol=2e-2)
+    assert torch.equal(out, each)
+    # a row_start that does not begin at zero is refused
+    with pytest.raises(AssertionError):
+        hip_kernels.expert_groups_ffn(group, xd, starts + 1, None, out)
