@@ -237,7 +237,7 @@ int hqq_router_top2_rows(const void *x_f16, const void *gate_w_f16, int32_t n_ex
                          int32_t *sel_out, void *weights_f16_out, void *logits_f16_out, void *stream);
 
 /* ---- the (token, slot) pairs of a prompt pass grouped by expert on the device (the reference builds an expert mask
- *      and runs torch.where per expert, src/custom_layers.py:291-303): sel [tokens][2] and weights_f16 [tokens][2] as
+ *      and runs torch.where per expert, src/custom_layers.py:288-301): sel [tokens][2] and weights_f16 [tokens][2] as
  *      hqq_router_top2_rows writes them.  Pair p = 2 * token + slot goes to the rows of expert sel[p], pairs of one
  *      expert in the order of p.  Out: counts_out[e] rows of expert e (the only figure the host needs before it
  *      launches the experts), and for row r of the grouped order token_of_row_out[r] (the token it came from) and

@@ -303,7 +303,7 @@ class SparseMoeWrapper(nn.Module):
         if tokens > 1 and selected_experts.dtype == torch.int32 and routing_weights.dtype == torch.float16:
             # Several tokens, router on the device: the (token, slot) pairs are grouped by expert there as well, the
             # rows of every expert are gathered at once, and only then does the host wait, for the experts' row counts
-            # alone (reference :291-312 does a where / gather / index_add_ per expert).  Each token receives the same
+            # alone (reference :288-312 does a where / gather / index_add_ per expert).  Each token receives the same
             # two fp16 terms in the index_add_ below, and their sum does not depend on the order.
             counts_dev, top_x, scales = hip_kernels.moe_group_pairs(selected_experts, routing_weights, self.num_experts)
             gathered = hidden_states.index_select(0, top_x)

@@ -601,7 +601,7 @@ def router_top2_rows(x: torch.Tensor, gate_weight: torch.Tensor):
 
 def moe_group_pairs(sel: torch.Tensor, weights: torch.Tensor, n_experts: int):
     """The (token, slot) pairs of ``router_top2_rows`` grouped by expert on the device (reference
-    src/custom_layers.py:291-303): returns ``counts`` int32 (n_experts,), and per row of the grouped order the token
+    src/custom_layers.py:288-301): returns ``counts`` int32 (n_experts,), and per row of the grouped order the token
     it came from (int64) and its routing weight (fp16).  Nothing here waits for the device."""
     assert sel.dtype == torch.int32 and sel.dim() == 2 and sel.shape[1] == 2 and sel.is_contiguous()
     assert weights.dtype == torch.float16 and weights.shape == sel.shape and weights.is_contiguous()
