@@ -511,6 +511,7 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_pairs_kernel(const in
 {
     __shared__ int first[kGroupThreads][kMaxExperts + 1]; // (+1: the threads of a wave fall into different banks)
     __shared__ int base[kMaxExperts];
+    __shared__ int total;
     const int t = threadIdx.x;
     const int chunk = (pairs + kGroupThreads - 1) / kGroupThreads;
     const int lo = t * chunk < pairs ? t * chunk : pairs, hi = lo + chunk < pairs ? lo + chunk : pairs;
@@ -540,6 +541,7 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_pairs_kernel(const in
             base[e] = run;
             run += c;
         }
+        total = run;
     }
     __syncthreads();
     for (int p = lo; p < hi; ++p) {
@@ -549,6 +551,12 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_pairs_kernel(const in
         const int row = base[e] + first[t][e]++;
         token_of_row[row] = p >> 1;
         scale_of_row[row] = weights[p];
+    }
+    // pairs whose expert is out of range are left out of the counts; the rows that stay free at the end name token 0
+    // with weight zero, so that a caller who indexes with all of them reads valid memory and adds nothing
+    for (int row = total + t; row < pairs; row += kGroupThreads) {
+        token_of_row[row] = 0;
+        scale_of_row[row] = (f16)0.0f;
     }
 }
 

@@ -479,6 +479,13 @@ def test_moe_group_pairs_is_a_stable_sort_by_expert(tokens, n_experts):
     assert np.array_equal(scale_of_row.cpu().numpy(), w.reshape(-1)[order])
     if n_experts > 2:
         assert int(counts[1]) == 0
+    # an expert id out of range is left out; the rows that stay free name token 0 with weight zero
+    bad = sel.copy()
+    bad[0, 0] = n_experts + 3
+    counts, token_of_row, scale_of_row = hip_kernels.moe_group_pairs(torch.from_numpy(bad).cuda(), torch.from_numpy(w).cuda(),
+                                                                     n_experts)
+    assert int(counts.sum()) == 2 * tokens - 1
+    assert int(token_of_row[-1]) == 0 and float(scale_of_row[-1]) == 0.0
 
 
 @pytest.mark.gpu
