@@ -734,46 +734,51 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
         auto both = [&](const f32x4 &c, int e) __attribute__((always_inline)) {
             return c[2 * e] + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, (float)c[2 * e + 1]), 0xB1, 0xF, 0xF, true));
         };
+        // the lane's roles once more, from a copy of the lane number the compiler cannot see through: derived from the
+        // values of the prologue they would stay live through the whole code phase, which has no register to spare
+        int lt = lane;
+        asm volatile("" : "+v"(lt));
+        const int phi_t = lt & 1, half_t = (lt >> 1) & 1, mrow_t = (lt & 15) >> 2, gk_t = lt >> 4;
         float zv[BG][2][2];
 #pragma unroll
         for (int bg = 0; bg < BG; ++bg)
 #pragma unroll
             for (int e = 0; e < 2; ++e)
                 zv[bg][e][0] = both(accz[0][bg], e), zv[bg][e][1] = both(accz[1][bg], e);
-        if (phi == 0 && half == 0) {
+        if (phi_t == 0 && half_t == 0) {
 #pragma unroll
             for (int bg = 0; bg < BG; ++bg)
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
-                    zt_lds[wave][2 * gk + e][4 * bg + mrow] = zv[bg][e][0] * (1.0f / kXsScale);
-                    if (gk == 0)
-                        zt_lds[wave][8 + e][4 * bg + mrow] = zv[bg][e][1] * (1.0f / kXsScale);
+                    zt_lds[wave][2 * gk_t + e][4 * bg + mrow_t] = zv[bg][e][0] * (1.0f / kXsScale);
+                    if (gk_t == 0)
+                        zt_lds[wave][8 + e][4 * bg + mrow_t] = zv[bg][e][1] * (1.0f / kXsScale);
                 }
         }
         wave_sync();
         float (*const red_w)[10][MT] = red_lds(wave);
 #pragma unroll
         for (int set = 0; set < 5; ++set) {
-            const int f = w3_set_field(set, half);
-            const float un = w3_set_unscale(set, half);
+            const int f = w3_set_field(set, half_t);
+            const float un = w3_set_unscale(set, half_t);
             float out[BG][2][2];
 #pragma unroll
             for (int bg = 0; bg < BG; ++bg) {
-                const float zt = zt_lds[wave][f][4 * bg + mrow];
+                const float zt = zt_lds[wave][f][4 * bg + mrow_t];
 #pragma unroll
                 for (int g8 = 0; g8 < 2; ++g8)
 #pragma unroll
                     for (int e = 0; e < 2; ++e)
                         out[bg][g8][e] = fmaf(both(acc[g8][set][bg], e), un, -zt);
             }
-            if (phi == 0) {
+            if (phi_t == 0) {
 #pragma unroll
                 for (int bg = 0; bg < BG; ++bg)
 #pragma unroll
                     for (int g8 = 0; g8 < 2; ++g8)
 #pragma unroll
                         for (int e = 0; e < 2; ++e)
-                            red_w[8 * g8 + 2 * gk + e][f][4 * bg + mrow] = out[bg][g8][e];
+                            red_w[8 * g8 + 2 * gk_t + e][f][4 * bg + mrow_t] = out[bg][g8][e];
             }
         }
     }
