@@ -496,31 +496,35 @@ __global__ __launch_bounds__(kW3Waves * 64) void gemv_w3_kernel(W3Params p)
         const float zt = zt_lds[wave][fcol][0] * (1.0f / kXsScale), zt4 = zt_lds[wave][fcol4][0] * (1.0f / kXsScale);
         const float un = w3_set_unscale(set, half), un4 = w3_set_unscale(4, half);
         // Accumulator element v of a lane is tile row 4 * (lane >> 4) + v = 2 * word row + phase; a column keeps the
-        // rows of its own phase, and the two phases of a word row are lanes one apart.
-        const uint32_t odd = phi ? ~0u : 0u;
+        // rows of its own phase, and the two phases of a word row are lanes one apart: the lanes of phase 0 add their
+        // neighbour's odd element to their own even one (what the lanes of phase 1 compute is not used).
+        auto swapped = [](float v) __attribute__((always_inline)) {
+            return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+        };
+        float out[2][2], out4[2][2];
 #pragma unroll
         for (int g8 = 0; g8 < 2; ++g8) {
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
-                // a bitwise select: written as a conditional the compiler turns it into an indexed read of the vector
-                auto pick = [&](const f32x4 &c) __attribute__((always_inline)) {
-                    return __builtin_bit_cast(float, (__builtin_bit_cast(uint32_t, (float)c[2 * e + 1]) & odd) |
-                                                         (__builtin_bit_cast(uint32_t, (float)c[2 * e]) & ~odd));
-                };
-                float v = pick(acc[g8][0]);
+                float even = acc[g8][0][2 * e], odd = acc[g8][0][2 * e + 1]; // of the lane's own set
 #pragma unroll
                 for (int i = 1; i < 4; ++i) {
-                    const float c = pick(acc[g8][i]);
-                    v = set == i ? c : v;
+                    even = set == i ? (float)acc[g8][i][2 * e] : even;
+                    odd = set == i ? (float)acc[g8][i][2 * e + 1] : odd;
                 }
-                float v4 = pick(acc[g8][4]);
-                v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
-                v4 += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v4), 0xB1, 0xF, 0xF, true));
-                const int row = 8 * g8 + 2 * gk + e;
-                if (phi == 0) {
-                    red_lds(wave)[row][fcol][0] = fmaf(v, un, -zt);
+                out[g8][e] = fmaf(even + swapped(odd), un, -zt);
+                out4[g8][e] = fmaf(acc[g8][4][2 * e] + swapped(acc[g8][4][2 * e + 1]), un4, -zt4);
+            }
+        }
+        if (phi == 0) {
+#pragma unroll
+            for (int g8 = 0; g8 < 2; ++g8) {
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const int row = 8 * g8 + 2 * gk + e;
+                    red_lds(wave)[row][fcol][0] = out[g8][e];
                     if (set == 0)
-                        red_lds(wave)[row][fcol4][0] = fmaf(v4, un4, -zt4);
+                        red_lds(wave)[row][fcol4][0] = out4[g8][e];
                 }
             }
         }
