@@ -34,16 +34,17 @@
 // while the first slab's codes are worked on); when K needs several blocks (or the window count alone would leave
 // most of the chip idle) the blocks of a tile add their results into one 64-bit fixed-point accumulation slot per
 // output with a returning device-scope atomic, and the block whose addition completes a slot writes that output
-// (launches with more outputs than there are slots store fp32 partial sums instead, and the block that arrives
-// last at the tile's counter adds them in a fixed order).
+// (launches with more outputs than there are slots: with two blocks along K the two swap their sums through a 32-bit
+// word per output in the same memory; else they store fp32 partial sums, and the block that arrives last at the
+// tile's counter adds them in a fixed order).
 //
 // A launch may hold up to four layers of one shape (a one-dimensional grid over layer, window, row block and K
 // block, see the kernel): the two projections of an
 // expert's gate, or those of two experts.  Their records come from the kernel arguments or from a device table
 // (record sel[layer / lper] * stride + first + layer % lper), so that the expert can be chosen on the device.
-// XMODE 1 builds the activations on the fly as silu(xa) * xb, which is how the down projection reads the two
-// gate outputs without an elementwise launch in between; the epilogue can multiply by a routing weight per row
-// and add into y.
+// XMODE 1 (one batch row) builds the activations on the fly as silu(xa) * xb, which is how the down projection reads
+// the two gate outputs without an elementwise launch in between; the epilogue can multiply by a routing weight per
+// row and add into y.
 #include "gemv_parts.hpp"
 #include "hqq_common.hpp"
 #include <type_traits>
