@@ -126,7 +126,9 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
  *      y[row] = row_scale_f16[row] * expert(x[row]) (row_scale_f16 may be NULL).  row_start is a HOST array of
  *      n_groups + 1 entries starting at 0; groups without rows may have NULL layers.  One call issues every group's
  *      launches in order on `stream` with one workspace of hqq_expert_groups_ffn_workspace_bytes(..) bytes (the
- *      largest group's need; head zeroed as for hqq_matmul_transpose).  Results are hqq_expert_ffn's, bit for bit. */
+ *      largest group's need, then the partial sums of the down projections that split K: their finishing passes run
+ *      as one launch at the end of the call; head zeroed as for hqq_matmul_transpose).  Results are
+ *      hqq_expert_ffn's, bit for bit.                                                                              */
 size_t hqq_expert_groups_ffn_workspace_bytes(const hqq_linear *const *w1, const hqq_linear *const *w2,
                                              const hqq_linear *const *w3, int32_t n_groups, const int64_t *row_start);
 int hqq_expert_groups_ffn(const hqq_linear *const *w1, const hqq_linear *const *w2, const hqq_linear *const *w3,

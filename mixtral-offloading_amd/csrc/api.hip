@@ -311,9 +311,16 @@ int hqq_gate_up(const hqq_linear *w1, const hqq_linear *w3, const void *x_f16, i
     return launch_silu_mul(a, b, h, M * w1->N, s);
 }
 
-int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *x_f16, int64_t M,
-                   void *y_f16, const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
-                   void *stream)
+// whether the down projection of an expert FFN at M rows is a tile launch whose finishing pass can be left to the caller
+static bool down_finish_deferrable(const hqq_linear *w2, int64_t M)
+{
+    return M > kSmallBatchMax && pick_family(w2, M) == FAM_TILE && tile_epilogue_supported(w2, M) && tile_partial_bytes(w2, M) > 0;
+}
+
+// down_part / defer: see launch_tile_matmul_deferred; used when down_finish_deferrable(w2, M)
+static int expert_ffn_impl(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *x_f16, int64_t M,
+                           void *y_f16, const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
+                           void *stream, void *down_part, TileFinish *defer)
 {
     int rc;
     if ((rc = validate_linear(w1)) != HQQ_OK || (rc = validate_linear(w2)) != HQQ_OK ||
@@ -378,6 +385,12 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
         ep.accumulate = accumulate;
         return launch_smallbatch_matmul(w2, h, M, y, mm, mm_bytes, ep, s);
     }
+    if (defer && down_finish_deferrable(w2, M)) {
+        SmallBatchEpilogue ep;
+        ep.row_scale = (const f16 *)row_scale_f16;
+        ep.accumulate = accumulate;
+        return launch_tile_matmul_deferred(w2, h, M, y, mm, mm_bytes, s, &ep, down_part, defer);
+    }
     if (!row_scale_f16 && !accumulate)
         return run_matmul(w2, h, M, y, mm, mm_bytes, pick_family(w2, M), s);
     if (pick_family(w2, M) == FAM_LDS) {
@@ -397,13 +410,22 @@ int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear 
     return launch_scale_store(t, y, (const f16 *)row_scale_f16, accumulate, M, w2->N, s);
 }
 
-// ---- the experts of one MoE layer over rows already grouped by expert: hqq_expert_ffn once per group, from one call
-size_t hqq_expert_groups_ffn_workspace_bytes(const hqq_linear *const *w1, const hqq_linear *const *w2,
-                                             const hqq_linear *const *w3, int32_t n_groups, const int64_t *row_start)
+int hqq_expert_ffn(const hqq_linear *w1, const hqq_linear *w2, const hqq_linear *w3, const void *x_f16, int64_t M,
+                   void *y_f16, const void *row_scale_f16, int accumulate, void *workspace, size_t workspace_bytes,
+                   void *stream)
 {
-    if (!w1 || !w2 || !w3 || !row_start || n_groups <= 0)
-        return 0;
+    return expert_ffn_impl(w1, w2, w3, x_f16, M, y_f16, row_scale_f16, accumulate, workspace, workspace_bytes, stream,
+                           nullptr, nullptr);
+}
+
+// ---- the experts of one MoE layer over rows already grouped by expert: hqq_expert_ffn once per group, from one call
+// Workspace of the grouped call: what the largest group needs, then the partial sums of every group whose down
+// projection leaves its finishing pass to the end of the call.
+static size_t groups_common_bytes(const hqq_linear *const *w1, const hqq_linear *const *w2, const hqq_linear *const *w3,
+                                  int32_t n_groups, const int64_t *row_start, size_t *parts)
+{
     size_t need = 0;
+    *parts = 0;
     for (int g = 0; g < n_groups; ++g) {
         const int64_t M = row_start[g + 1] - row_start[g];
         if (M <= 0)
@@ -414,8 +436,20 @@ size_t hqq_expert_groups_ffn_workspace_bytes(const hqq_linear *const *w1, const 
         if (one == 0)
             return 0;
         need = one > need ? one : need;
+        if (down_finish_deferrable(w2[g], M))
+            *parts += tile_partial_bytes(w2[g], M);
     }
-    return need;
+    return align256(need);
+}
+
+size_t hqq_expert_groups_ffn_workspace_bytes(const hqq_linear *const *w1, const hqq_linear *const *w2,
+                                             const hqq_linear *const *w3, int32_t n_groups, const int64_t *row_start)
+{
+    if (!w1 || !w2 || !w3 || !row_start || n_groups <= 0)
+        return 0;
+    size_t parts = 0;
+    const size_t common = groups_common_bytes(w1, w2, w3, n_groups, row_start, &parts);
+    return common ? common + parts : 0;
 }
 
 int hqq_expert_groups_ffn(const hqq_linear *const *w1, const hqq_linear *const *w2, const hqq_linear *const *w3,
@@ -432,6 +466,15 @@ int hqq_expert_groups_ffn(const hqq_linear *const *w1, const hqq_linear *const *
         if (row_start[g + 1] > row_start[g] && (!w1[g] || !w2[g] || !w3[g]))
             return HQQ_E_NULL;
     }
+    // The down projections that split K write their partial sums to a place of their own behind the common workspace,
+    // and one launch at the end finishes them all (sum over the K blocks, routing weight, store): between the experts
+    // no finishing launch waits for its projection to drain.
+    size_t parts = 0;
+    const size_t common = groups_common_bytes(w1, w2, w3, n_groups, row_start, &parts);
+    const bool defer = workspace && common > 0 && parts > 0 && workspace_bytes >= common + parts;
+    TileFinish fin[kTileFinishGroupMax];
+    int nf = 0;
+    char *part_at = static_cast<char *>(workspace) + common;
     for (int g = 0; g < n_groups; ++g) {
         const int64_t lo = row_start[g], M = row_start[g + 1] - lo;
         if (M == 0)
@@ -439,12 +482,18 @@ int hqq_expert_groups_ffn(const hqq_linear *const *w1, const hqq_linear *const *
         const char *x = static_cast<const char *>(x_f16) + (size_t)lo * (size_t)w1[g]->K * 2;
         char *y = static_cast<char *>(y_f16) + (size_t)lo * (size_t)w2[g]->N * 2;
         const char *rs = row_scale_f16 ? static_cast<const char *>(row_scale_f16) + (size_t)lo * 2 : nullptr;
-        const int rc = hqq_expert_ffn(w1[g], w2[g], w3[g], x_f16 ? x : nullptr, M, y_f16 ? y : nullptr, rs, 0, workspace,
-                                      workspace_bytes, stream);
+        const bool later = defer && nf < kTileFinishGroupMax && down_finish_deferrable(w2[g], M);
+        const int rc = expert_ffn_impl(w1[g], w2[g], w3[g], x_f16 ? x : nullptr, M, y_f16 ? y : nullptr, rs, 0, workspace,
+                                       defer ? common : workspace_bytes, stream, later ? part_at : nullptr,
+                                       later ? &fin[nf] : nullptr);
         if (rc != HQQ_OK)
             return rc;
+        if (later && fin[nf].part) {
+            part_at += tile_partial_bytes(w2[g], M);
+            ++nf;
+        }
     }
-    return HQQ_OK;
+    return nf ? launch_tile_finish_group(fin, nf, (hipStream_t)stream) : HQQ_OK;
 }
 
 // ---- the expert FFN for callers that cannot allocate.  The workspace is a file-scope device array; each GPU holds

@@ -680,10 +680,9 @@ __global__ __launch_bounds__(JW * NFW * KW * 64) void gemm_tile2_kernel(TilePara
 // GATE: two sets of partial sums, lstride floats apart; y = silu(a) * b with both projections rounded to fp16, SiLU
 // in fp32 rounded once, product in fp16 (the reference's three ops, src/custom_layers.py:253-256).
 template <int F, bool GATE>
-__global__ __launch_bounds__(256) void tile_finish_kernel(const float *__restrict__ part, int KSP, int M, int N,
-                                                           const f16 *__restrict__ bias, f16 *__restrict__ y,
-                                                           int64_t lstride, const f16 *__restrict__ row_scale,
-                                                           int accumulate)
+__device__ __forceinline__ void tile_finish_block(const float *__restrict__ part, int KSP, int M, int N,
+                                                  const f16 *__restrict__ bias, f16 *__restrict__ y, int64_t lstride,
+                                                  const f16 *__restrict__ row_scale, int accumulate)
 {
     __shared__ f16 t_lds[16][16][F];
     const int NG = N / F;
@@ -729,6 +728,29 @@ __global__ __launch_bounds__(256) void tile_finish_kernel(const float *__restric
                 dst[i] = accumulate ? (f16)(dst[i] + t_lds[threadIdx.x >> 4][gl][i]) : t_lds[threadIdx.x >> 4][gl][i];
         }
     }
+}
+
+template <int F, bool GATE>
+__global__ __launch_bounds__(256) void tile_finish_kernel(const float *__restrict__ part, int KSP, int M, int N,
+                                                           const f16 *__restrict__ bias, f16 *__restrict__ y,
+                                                           int64_t lstride, const f16 *__restrict__ row_scale,
+                                                           int accumulate)
+{
+    tile_finish_block<F, GATE>(part, KSP, M, N, bias, y, lstride, row_scale, accumulate);
+}
+
+// The finishing passes of several launches as one: blockIdx.z names the launch, whose own grid may be smaller than
+// this one's.
+struct TileFinishGroup {
+    TileFinish f[kTileFinishGroupMax];
+};
+template <int F> __global__ __launch_bounds__(256) void tile_finish_group_kernel(TileFinishGroup g)
+{
+    const TileFinish &d = g.f[blockIdx.z];
+    if ((int)blockIdx.x * 16 >= d.N / F || (int)blockIdx.y * 16 >= d.M)
+        return;
+    tile_finish_block<F, false>(d.part, d.KSP, d.M, d.N, d.bias, d.y, 0, d.row_scale, d.accumulate);
+
 }
 
 // 3-bit codes (ten per 32-bit word, rows 10p .. 10p+9) rewritten as 4-bit codes (rows 2q, 2q+1 per byte, the even
@@ -938,9 +960,16 @@ static size_t tile_job_bytes(const hqq_linear *l, int64_t M, int nl)
 }
 
 // one layer (lb == nullptr) or the two projections of a gate: y = x W^T (+ bias), or y = silu(x Wa^T) * (x Wb^T)
+// part_at / defer (one layer only): the partial sums of a K split go to part_at instead of the workspace, and the
+// finishing pass is described in *defer instead of launched (defer->part is null when there is nothing to finish)
 static int tile_job(const hqq_linear *la, const hqq_linear *lb, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes,
-                    hipStream_t s, const SmallBatchEpilogue *ep = nullptr)
+                    hipStream_t s, const SmallBatchEpilogue *ep = nullptr, void *part_at = nullptr, TileFinish *defer = nullptr)
 {
+    if (defer) {
+        *defer = TileFinish{};
+        if (lb || !part_at || (reinterpret_cast<uintptr_t>(part_at) & 255u))
+            return HQQ_E_UNSUPPORTED;
+    }
     const int nl = lb ? 2 : 1;
     TilePlan pl;
     hqq_linear view[2] = {tile_view(la), tile_view(lb ? lb : la)};
@@ -982,7 +1011,7 @@ static int tile_job(const hqq_linear *la, const hqq_linear *lb, const f16 *x, in
     p.M = (int)M, p.N = (int)l->N, p.K = (int)l->K, p.GP = pl.GP, p.KT = pl.KT;
     p.KSP = pl.KSP, p.KTS = pl.KTS;
     p.row_scale = scaled ? ep->row_scale : nullptr, p.accumulate = scaled ? ep->accumulate : 0;
-    p.part = partial ? reinterpret_cast<float *>(body) : nullptr;
+    p.part = partial ? reinterpret_cast<float *>(defer ? static_cast<char *>(part_at) : body) : nullptr;
     // blocks along x: packed rows (per projection, unless a block holds both) by K blocks
     const int jrows = pl.JW == 2 ? pl.GP : pl.GP / pl.JW * nl;
     const dim3 grid((unsigned)(jrows * pl.KSP), (unsigned)pl.RB, (unsigned)((M + pl.BM - 1) / pl.BM));
@@ -1006,6 +1035,11 @@ static int tile_job(const hqq_linear *la, const hqq_linear *lb, const f16 *x, in
     int rc = launch_status();
     if (rc != HQQ_OK || !partial)
         return rc;
+    if (defer) {
+        defer->part = p.part, defer->KSP = pl.KSP, defer->M = (int)M, defer->N = (int)l->N, defer->F = pl.F;
+        defer->bias = p.bias, defer->y = y, defer->row_scale = p.row_scale, defer->accumulate = p.accumulate;
+        return HQQ_OK;
+    }
     const dim3 fgrid((unsigned)((l->N / pl.F + 15) / 16), (unsigned)((M + 15) / 16));
     if (nl == 2) {
         if (pl.F == 4)
@@ -1021,6 +1055,51 @@ static int tile_job(const hqq_linear *la, const hqq_linear *lb, const f16 *x, in
 }
 
 size_t tile_workspace_bytes(const hqq_linear *l, int64_t M) { return tile_job_bytes(l, M, 1); }
+
+// bytes of partial sums a one-layer launch writes (0: K is not split, nothing to finish)
+size_t tile_partial_bytes(const hqq_linear *l, int64_t M)
+{
+    TilePlan pl;
+    const hqq_linear v = tile_view(l);
+    if (!make_plan(&v, M, pl, 1) || pl.KSP <= 1)
+        return 0;
+    return ((size_t)pl.KSP * (size_t)M * (size_t)l->N * sizeof(float) + 255) & ~(size_t)255;
+}
+
+int launch_tile_matmul_deferred(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s,
+                                const SmallBatchEpilogue *ep, void *part_at, TileFinish *finish)
+{
+    return tile_job(l, nullptr, x, M, y, ws, ws_bytes, s, ep, part_at, finish);
+}
+
+// the finishing passes of up to kTileFinishGroupMax deferred launches in one launch per code width
+int launch_tile_finish_group(const TileFinish *f, int n, hipStream_t s)
+{
+    for (int F = 2; F <= 4; F += 2) {
+        TileFinishGroup g = {};
+        int cnt = 0, gx = 0, gy = 0;
+        for (int i = 0; i < n; ++i) {
+            if (!f[i].part || f[i].F != F)
+                continue;
+            if (cnt == kTileFinishGroupMax)
+                return HQQ_E_UNSUPPORTED;
+            g.f[cnt++] = f[i];
+            const int x = (f[i].N / F + 15) / 16, y = (f[i].M + 15) / 16;
+            gx = x > gx ? x : gx, gy = y > gy ? y : gy;
+        }
+        if (!cnt)
+            continue;
+        const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)cnt);
+        if (F == 4)
+            tile_finish_group_kernel<4><<<grid, 256, 0, s>>>(g);
+        else
+            tile_finish_group_kernel<2><<<grid, 256, 0, s>>>(g);
+        const int rc = launch_status();
+        if (rc != HQQ_OK)
+            return rc;
+    }
+    return HQQ_OK;
+}
 
 int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s,
                        const SmallBatchEpilogue *ep)

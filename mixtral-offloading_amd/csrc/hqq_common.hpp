@@ -215,6 +215,21 @@ size_t tile_workspace_bytes(const hqq_linear *l, int64_t M);
 int launch_tile_matmul(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s,
                        const SmallBatchEpilogue *ep = nullptr);
 bool tile_epilogue_supported(const hqq_linear *l, int64_t M);
+// A tile launch whose finishing pass (the sum over its K blocks, bias, routing weight, accumulation) is left to the
+// caller, who runs the passes of several launches as one (launch_tile_finish_group).
+struct TileFinish {
+    const float *part; // null: the launch has written its output itself
+    int KSP, M, N, F;
+    const f16 *bias;
+    f16 *y;
+    const f16 *row_scale;
+    int accumulate;
+};
+constexpr int kTileFinishGroupMax = 16;
+size_t tile_partial_bytes(const hqq_linear *l, int64_t M);
+int launch_tile_matmul_deferred(const hqq_linear *l, const f16 *x, int64_t M, f16 *y, void *ws, size_t ws_bytes, hipStream_t s,
+                                const SmallBatchEpilogue *ep, void *part_at, TileFinish *finish);
+int launch_tile_finish_group(const TileFinish *f, int n, hipStream_t s);
 bool tile_gate_supported(const hqq_linear *w1, const hqq_linear *w3, int64_t M);
 size_t tile_gate_workspace_bytes(const hqq_linear *w1, const hqq_linear *w3, int64_t M);
 int launch_tile_gate_up(const hqq_linear *w1, const hqq_linear *w3, const f16 *x, int64_t M, f16 *h, void *ws,

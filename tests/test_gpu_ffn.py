@@ -194,3 +194,33 @@ def test_expert_groups_entry_point_equals_one_call_per_expert(nbits, hidden, ffn
     # a row_start that does not begin at zero is refused
     with pytest.raises(AssertionError):
         hip_kernels.expert_groups_ffn(group, xd, starts + 1, None, out)
+
+
+def test_expert_groups_at_full_size_leave_the_finishing_passes_to_the_end():
+    """Mixtral-sized 2-bit experts with 17 to 64 rows each: their down projections split K, write their partial sums
+    to places of their own and are finished by one launch at the end of the call.  Bit for bit what one call per
+    expert gives, twice over (the second call finds the workspace as the first left it), and a decode-sized call in
+    between on the same workspace."""
+    from mixtral_offloading_amd import hip_kernels
+    from test_gpu_matmul import _full_size_layer
+    counts = [33, 20, 0, 64, 7, 40]
+    descs = [(_full_size_layer(2, 14336, 4096, 16, seed=3 * e), _full_size_layer(2, 4096, 14336, 16, seed=3 * e + 1),
+              _full_size_layer(2, 14336, 4096, 16, seed=3 * e + 2)) for e in range(len(counts))]
+    group = hip_kernels.ExpertGroup(descs)
+    starts = np.concatenate(([0], np.cumsum(counts)))
+    rows = int(starts[-1])
+    g = torch.Generator(device="cuda").manual_seed(11)
+    x = torch.randn((rows, 4096), device="cuda", generator=g).half()
+    scale = (torch.rand((rows,), device="cuda", generator=g) * 0.6 + 0.2).half()
+    each = torch.empty((rows, 4096), dtype=torch.float16, device="cuda")
+    for e, (w1, w2, w3) in enumerate(descs):
+        lo, hi = int(starts[e]), int(starts[e + 1])
+        if hi > lo:
+            hip_kernels.expert_ffn(w1, w2, w3, x[lo:hi], out=each[lo:hi], row_scale=scale[lo:hi])
+    assert bool(torch.isfinite(each).all()) and float(each.float().abs().max()) > 0
+    for rep in range(2):
+        out = torch.full((rows, 4096), 3.0, dtype=torch.float16, device="cuda")
+        hip_kernels.expert_groups_ffn(group, x, starts, scale, out)
+        assert torch.equal(out, each)
+        one = hip_kernels.expert_ffn(descs[0][0], descs[0][1], descs[0][2], x[:1].contiguous())
+        assert bool(torch.isfinite(one).all())
