@@ -483,6 +483,8 @@ int hqq_expert_groups_ffn(const hqq_linear *const *w1, const hqq_linear *const *
         char *y = static_cast<char *>(y_f16) + (size_t)lo * (size_t)w2[g]->N * 2;
         const char *rs = row_scale_f16 ? static_cast<const char *>(row_scale_f16) + (size_t)lo * 2 : nullptr;
         const bool later = defer && nf < kTileFinishGroupMax && down_finish_deferrable(w2[g], M);
+        if (later)
+            fin[nf] = TileFinish{};
         const int rc = expert_ffn_impl(w1[g], w2[g], w3[g], x_f16 ? x : nullptr, M, y_f16 ? y : nullptr, rs, 0, workspace,
                                        defer ? common : workspace_bytes, stream, later ? part_at : nullptr,
                                        later ? &fin[nf] : nullptr);
